@@ -1,0 +1,111 @@
+/*
+ * C ABI of librosa_soft_hip.so: the MI355X (gfx950) device side of the
+ * rosa_soft / rosa_soft_varlen training operators.
+ *
+ * Plain pointers and sizes only.  Every pointer is a DEVICE pointer unless the
+ * comment says otherwise; `stream` is a hipStream_t passed as void*.  Nothing
+ * here synchronises with the host and nothing allocates: the caller owns the
+ * outputs and the workspace.  All entry points return 0 on success or a
+ * non-zero code; rosa_hip_last_error() then describes the failure (thread
+ * local).
+ *
+ * Each entry point replaces one launcher of the reference
+ * (/root/reference/rosa_soft/csrc/cuda/rosa_soft_kernels.cu), cited below.
+ * The dispatcher layer above it (rosa_soft_amd/csrc/rosa_dispatch.cpp) plays
+ * the role of the reference's rosa_soft/csrc/rosa_soft.cpp:379-549.
+ */
+#ifndef ROSA_SOFT_HIP_H_
+#define ROSA_SOFT_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of query/key/value/grad_output/output */
+enum { ROSA_DTYPE_F32 = 0, ROSA_DTYPE_F16 = 1, ROSA_DTYPE_BF16 = 2 };
+
+/* gradient_mask bits, as in the reference (rosa_soft_kernels.cu:24-26) */
+enum { ROSA_GRAD_QUERY = 1, ROSA_GRAD_KEY = 2, ROSA_GRAD_VALUE = 4 };
+
+/*
+ * Problem description shared by all entry points.
+ *   dense  layout: query/key [B,T,H,D], value [B,T,Hv,Dv]; set S = 0,
+ *                  cu_seqlens = NULL, N = B*T.
+ *   packed layout: query/key [N,H,D], value [N,Hv,Dv], cu_seqlens int32 [S+1]
+ *                  on the device; set B = 0, T = 0.
+ * W is max_suffix_length already clamped to T (dense) or N (packed).
+ */
+typedef struct rosa_problem {
+  int dtype;
+  int B, T;      /* dense only */
+  int N, S;      /* packed token count, number of packed sequences */
+  int H, D;      /* query/key heads and symbol width (1..32) */
+  int Hv, Dv;    /* value heads (H % Hv == 0) and value width */
+  int W;
+  const int32_t* cu_seqlens; /* device, packed layout only */
+} rosa_problem;
+
+/* Library version (major*10000 + minor*100 + patch) and build target string. */
+int rosa_hip_version(void);
+const char* rosa_hip_target(void);
+const char* rosa_hip_last_error(void);
+
+/*
+ * Workspace sizes in bytes for the calls below (host-side arithmetic only).
+ * `dropout` is non-zero when dropout_p > 0.
+ */
+size_t rosa_hip_forward_workspace_bytes(const rosa_problem* problem);
+size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_mask,
+                                    float scale, int dropout);
+
+/*
+ * Exact hard forward.  Replaces hard_forward_cuda (rosa_soft_kernels.cu:1766-1834)
+ * and hard_forward_varlen_cuda (:1837-1920): sign-packs query and key into
+ * head-major int32 words (dense [B,H,T], packed [H,N]), finds the
+ * latest-longest route of every row and gathers sign(value[route]) (exact zero
+ * for the null route) into `output` (same dtype as the inputs).
+ * `routes` is optional (may be NULL): int32 in the packed-symbol layout, the
+ * selected route index local to its sequence, 0 for null.  The reference's
+ * device API has no such output; it exists so that index parity can be
+ * checked.
+ */
+int rosa_hip_hard_forward(const rosa_problem* problem, const void* query,
+                          const void* key, const void* value, void* output,
+                          int32_t* packed_query, int32_t* packed_key,
+                          int32_t* routes, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/*
+ * Dense surrogate VJP.  Replaces surrogate_vjp_cuda (rosa_soft_kernels.cu:1923-2379)
+ * and surrogate_vjp_varlen_cuda (:2382-2638).  Gradients are float32 in the
+ * layout of the corresponding input and are fully overwritten; pass NULL for
+ * a gradient whose mask bit is clear.  `dropout_seed` is a device int64
+ * scalar, read only when dropout_p > 0.  `inverse_keep` is 1.0f/(1.0f-p)
+ * computed by the caller in float32 (rosa_soft.cpp:101-128).
+ */
+int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
+                           const void* key, const void* value,
+                           const void* grad_output, const int32_t* packed_query,
+                           const int32_t* packed_key, const int64_t* dropout_seed,
+                           float scale, float dropout_p, float inverse_keep,
+                           float mismatch_scale, int gradient_mask,
+                           float* grad_query, float* grad_key, float* grad_value,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Asynchronous device-side diagnostics.  Invalid cu_seqlens values (not
+ * starting at 0, decreasing, or not ending at N) cannot be seen by the host
+ * without a synchronisation, so the kernels clamp them to a safe range, and
+ * record the fact in the first int32 of the workspace.  This call copies that
+ * word back (it synchronises `stream`) and returns it: 0 = offsets were valid.
+ * The reference aborts the process instead (rosa_soft_kernels.cu:287-308).
+ */
+int rosa_hip_read_offset_error(const void* workspace, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ROSA_SOFT_HIP_H_ */

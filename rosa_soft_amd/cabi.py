@@ -1,0 +1,224 @@
+"""ctypes binding of ``librosa_soft_hip.so`` (declared in ``include/rosa_soft_hip.h``).
+
+This is the thinnest way to reach the kernels: tensors are passed as raw
+device pointers and the current torch stream as ``hipStream_t``.  The operator
+itself goes through the dispatcher extension (``rosa_soft_amd._C``); the parity
+tests, ``bench.py`` and the route-index side channel use this module.  Loading
+fails loudly when the library has not been built: there is no CPU fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "librosa_soft_hip.so")
+
+GRAD_QUERY, GRAD_KEY, GRAD_VALUE = 1, 2, 4
+
+EXPORTED_SYMBOLS = (
+    "rosa_hip_version",
+    "rosa_hip_target",
+    "rosa_hip_last_error",
+    "rosa_hip_forward_workspace_bytes",
+    "rosa_hip_vjp_workspace_bytes",
+    "rosa_hip_hard_forward",
+    "rosa_hip_surrogate_vjp",
+    "rosa_hip_read_offset_error",
+)
+
+_DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+class RosaProblem(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int),
+        ("B", ctypes.c_int),
+        ("T", ctypes.c_int),
+        ("N", ctypes.c_int),
+        ("S", ctypes.c_int),
+        ("H", ctypes.c_int),
+        ("D", ctypes.c_int),
+        ("Hv", ctypes.c_int),
+        ("Dv", ctypes.c_int),
+        ("W", ctypes.c_int),
+        ("cu_seqlens", ctypes.c_void_p),
+    ]
+
+
+_library: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library and declare every prototype of the header."""
+
+    global _library
+    if _library is not None:
+        return _library
+    if not os.path.exists(LIBRARY_PATH):
+        raise RuntimeError(
+            f"{LIBRARY_PATH} is missing: build it with "
+            "`python -c 'import __graft_entry__ as g; g.build()'` or `python setup.py build_ext --inplace`"
+        )
+    library = ctypes.CDLL(LIBRARY_PATH)
+    problem_p = ctypes.POINTER(RosaProblem)
+    vp = ctypes.c_void_p
+    library.rosa_hip_version.restype = ctypes.c_int
+    library.rosa_hip_target.restype = ctypes.c_char_p
+    library.rosa_hip_last_error.restype = ctypes.c_char_p
+    library.rosa_hip_forward_workspace_bytes.restype = ctypes.c_size_t
+    library.rosa_hip_forward_workspace_bytes.argtypes = [problem_p]
+    library.rosa_hip_vjp_workspace_bytes.restype = ctypes.c_size_t
+    library.rosa_hip_vjp_workspace_bytes.argtypes = [
+        problem_p, ctypes.c_int, ctypes.c_float, ctypes.c_int,
+    ]
+    library.rosa_hip_hard_forward.restype = ctypes.c_int
+    library.rosa_hip_hard_forward.argtypes = [
+        problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_surrogate_vjp.restype = ctypes.c_int
+    library.rosa_hip_surrogate_vjp.argtypes = [
+        problem_p, vp, vp, vp, vp, vp, vp, vp,
+        ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int,
+        vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_read_offset_error.restype = ctypes.c_int
+    library.rosa_hip_read_offset_error.argtypes = [vp, vp]
+    _library = library
+    return library
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        message = load().rosa_hip_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed with status {status}: {message}")
+
+
+def make_problem(
+    query: Tensor, value: Tensor, max_suffix_length: int, cu_seqlens: Optional[Tensor] = None
+) -> RosaProblem:
+    if query.dtype not in _DTYPE_CODES:
+        raise ValueError("rosa_soft supports float32, float16, and bfloat16")
+    problem = RosaProblem()
+    problem.dtype = _DTYPE_CODES[query.dtype]
+    if cu_seqlens is None:
+        batch, seq_len, heads, width = query.shape
+        problem.B, problem.T = batch, seq_len
+        problem.N, problem.S = batch * seq_len, 0
+        problem.Hv, problem.Dv = value.shape[2], value.shape[3]
+        problem.cu_seqlens = None
+        bound = seq_len
+    else:
+        tokens, heads, width = query.shape
+        problem.B, problem.T = 0, 0
+        problem.N, problem.S = tokens, cu_seqlens.numel() - 1
+        problem.Hv, problem.Dv = value.shape[1], value.shape[2]
+        problem.cu_seqlens = cu_seqlens.data_ptr()
+        bound = tokens
+    problem.H, problem.D = heads, width
+    problem.W = min(int(max_suffix_length), bound)
+    return problem
+
+
+def _stream(tensor: Tensor) -> int:
+    return torch.cuda.current_stream(tensor.device).cuda_stream
+
+
+def _ptr(tensor: Optional[Tensor]):
+    return None if tensor is None else tensor.data_ptr()
+
+
+def hard_forward(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    max_suffix_length: int,
+    cu_seqlens: Optional[Tensor] = None,
+    want_routes: bool = True,
+) -> Tuple[Tensor, Tensor, Tensor, Optional[Tensor]]:
+    """Run the hard forward; returns ``(output, packed_q, packed_k, routes)``.
+
+    Inputs must be contiguous device tensors.  ``routes`` (int32, in the packed
+    symbol layout, sequence-local, 0 = null) is the index side channel.
+    """
+
+    library = load()
+    assert query.is_cuda and query.is_contiguous() and key.is_contiguous() and value.is_contiguous()
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    if cu_seqlens is None:
+        word_shape = (problem.B, problem.H, problem.T)
+        out_shape = (problem.B, problem.T, problem.H, problem.Dv)
+    else:
+        word_shape = (problem.H, problem.N)
+        out_shape = (problem.N, problem.H, problem.Dv)
+    with torch.cuda.device(query.device):
+        output = torch.empty(out_shape, dtype=query.dtype, device=query.device)
+        packed_q = torch.empty(word_shape, dtype=torch.int32, device=query.device)
+        packed_k = torch.empty(word_shape, dtype=torch.int32, device=query.device)
+        routes = torch.empty(word_shape, dtype=torch.int32, device=query.device) if want_routes else None
+        size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
+        workspace = torch.empty(max(size, 256), dtype=torch.uint8, device=query.device)
+        status = library.rosa_hip_hard_forward(
+            ctypes.byref(problem), _ptr(query), _ptr(key), _ptr(value), _ptr(output),
+            _ptr(packed_q), _ptr(packed_k), _ptr(routes), _ptr(workspace), workspace.numel(),
+            _stream(query),
+        )
+    _check(status, "rosa_hip_hard_forward")
+    return output, packed_q, packed_k, routes
+
+
+def surrogate_vjp(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    grad_output: Tensor,
+    packed_q: Tensor,
+    packed_k: Tensor,
+    dropout_seed: Optional[Tensor],
+    max_suffix_length: int,
+    scale: float,
+    dropout_p: float,
+    mismatch_scale: float,
+    gradient_mask: int = 7,
+    cu_seqlens: Optional[Tensor] = None,
+    workspace: Optional[Tensor] = None,
+) -> Tuple[Optional[Tensor], Optional[Tensor], Optional[Tensor]]:
+    """Run the surrogate VJP; returns float32 ``(grad_q, grad_k, grad_v)``."""
+
+    library = load()
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    p32 = torch.tensor(float(dropout_p), dtype=torch.float32)
+    inverse_keep = float(torch.tensor(1.0, dtype=torch.float32) / (1.0 - p32))
+    with torch.cuda.device(query.device):
+        grads = [
+            torch.empty(t.shape, dtype=torch.float32, device=query.device)
+            if gradient_mask & bit
+            else None
+            for bit, t in zip((1, 2, 4), (query, key, value))
+        ]
+        size = library.rosa_hip_vjp_workspace_bytes(
+            ctypes.byref(problem), gradient_mask, float(scale), int(dropout_p > 0)
+        )
+        if workspace is None or workspace.numel() < size:
+            workspace = torch.empty(max(size, 256), dtype=torch.uint8, device=query.device)
+        status = library.rosa_hip_surrogate_vjp(
+            ctypes.byref(problem), _ptr(query), _ptr(key), _ptr(value), _ptr(grad_output),
+            _ptr(packed_q), _ptr(packed_k),
+            _ptr(dropout_seed) if dropout_p > 0 else None,
+            float(scale), float(p32), inverse_keep, float(mismatch_scale), int(gradient_mask),
+            _ptr(grads[0]), _ptr(grads[1]), _ptr(grads[2]),
+            _ptr(workspace), workspace.numel(), _stream(query),
+        )
+    _check(status, "rosa_hip_surrogate_vjp")
+    return tuple(grads)
+
+
+def vjp_workspace_bytes(query: Tensor, value: Tensor, max_suffix_length: int,
+                        cu_seqlens: Optional[Tensor] = None) -> int:
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0))

@@ -1,0 +1,1559 @@
+// MI355X (gfx950, wave64) kernels and C ABI of the rosa_soft training operators.
+//
+// Work decomposition
+// ------------------
+// A (row t, route a) pair compares the query suffix ending at t with the key
+// suffix ending at a-1.  Every recurrence of the operator runs along a
+// diagonal t - a = const, so the pair space of one (sequence, head) is cut
+// into BANDS of 64 adjacent diagonals.  One wavefront owns one band; lane l
+// owns diagonal 64*j + l and the wave marches over rows t, so that at a given
+// step every lane works on the same row t (row data is wave-uniform and lives
+// in scalar registers) while the per-column data (key word, value sign bits)
+// slides from lane to lane with one DPP wave shift per step.  All suffix
+// state (run length, soft evidence, window mismatch count, reverse adjoint)
+// is private to a lane: no cross-lane traffic is needed for the recurrences.
+//
+// The hard forward uses the transposed arrangement (lane = row, the wave walks
+// over routes) because its only reduction is per row.
+//
+// Numerics: every score, normaliser and gradient is float32; exp/rsqrt use the
+// hardware approximations, like the reference's --use_fast_math build.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <type_traits>
+
+#include "../../include/rosa_soft_hip.h"
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr float kNullScore = 0.5f;
+constexpr float kSqrtScale = 2.414213562373095f;  // sqrt(2) + 1
+constexpr float kLog2e = 1.4426950408889634f;
+
+constexpr int kChunk = 16;     // rows kept in registers between the forward and reverse sweeps
+constexpr int kSegment = 512;  // rows between two checkpoints kept in LDS
+constexpr int kSegChunks = kSegment / kChunk;
+constexpr int kColumnRing = 128;  // circular column accumulators (>= kChunk + 63)
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* message) {
+  snprintf(g_error, sizeof(g_error), "%s", message);
+  return code;
+}
+
+int fail_hip(hipError_t status, const char* what) {
+  snprintf(g_error, sizeof(g_error), "%s: %s", what, hipGetErrorString(status));
+  return 100 + static_cast<int>(status);
+}
+
+// ---------------------------------------------------------------------------
+// small device helpers
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ int dpp_wave_shr1(int fill_lane0, int src) {
+  // lane i receives src of lane i-1; lane 0 receives fill_lane0
+  return __builtin_amdgcn_update_dpp(fill_lane0, src, 0x138, 0xf, 0xf, false);
+}
+
+__device__ __forceinline__ uint32_t dpp_wave_shr1(uint32_t fill_lane0, uint32_t src) {
+  return static_cast<uint32_t>(
+      dpp_wave_shr1(static_cast<int>(fill_lane0), static_cast<int>(src)));
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float acc, float src) {
+  const int moved =
+      __builtin_amdgcn_update_dpp(0, __float_as_int(src), CTRL, ROW_MASK, 0xf, false);
+  return acc + __int_as_float(moved);
+}
+
+// Sum over the 64 lanes; the total is valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+  v = dpp_add<0x111, 0xf>(v, v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v, v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v, v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v, v);  // row_shr:8
+  v = dpp_add<0x142, 0xa>(v, v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v, v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_max(float acc, float src) {
+  // lanes without a valid source keep their own value
+  const int moved = __builtin_amdgcn_update_dpp(
+      __float_as_int(acc), __float_as_int(src), CTRL, ROW_MASK, 0xf, false);
+  return fmaxf(acc, __int_as_float(moved));
+}
+
+__device__ __forceinline__ float wave_max_lane63(float v) {
+  v = dpp_max<0x111, 0xf>(v, v);
+  v = dpp_max<0x112, 0xf>(v, v);
+  v = dpp_max<0x114, 0xf>(v, v);
+  v = dpp_max<0x118, 0xf>(v, v);
+  v = dpp_max<0x142, 0xa>(v, v);
+  v = dpp_max<0x143, 0xc>(v, v);
+  return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+template <int DTYPE>
+__device__ __forceinline__ float load_as_float(const void* base, int64_t index) {
+  if constexpr (DTYPE == ROSA_DTYPE_F32) {
+    return static_cast<const float*>(base)[index];
+  } else if constexpr (DTYPE == ROSA_DTYPE_F16) {
+    return static_cast<float>(static_cast<const _Float16*>(base)[index]);
+  } else {
+    const uint32_t bits = static_cast<const uint16_t*>(base)[index];
+    return __uint_as_float(bits << 16);
+  }
+}
+
+template <int DTYPE>
+__device__ __forceinline__ void store_sign(void* base, int64_t index, int sign) {
+  // sign in {-1, 0, +1}
+  if constexpr (DTYPE == ROSA_DTYPE_F32) {
+    static_cast<float*>(base)[index] = static_cast<float>(sign);
+  } else if constexpr (DTYPE == ROSA_DTYPE_F16) {
+    static_cast<uint16_t*>(base)[index] =
+        sign == 0 ? uint16_t(0) : (sign > 0 ? uint16_t(0x3C00) : uint16_t(0xBC00));
+  } else {
+    static_cast<uint16_t*>(base)[index] =
+        sign == 0 ? uint16_t(0) : (sign > 0 ? uint16_t(0x3F80) : uint16_t(0xBF80));
+  }
+}
+
+__device__ __forceinline__ uint32_t mix32(uint32_t s) {
+  s ^= s >> 16;
+  s *= 0x7feb352du;
+  s ^= s >> 15;
+  s *= 0x846ca68bu;
+  s ^= s >> 16;
+  return s;
+}
+
+// Dropout multiplier of one (row, route); head/batch/seed salts are folded by
+// the caller into wave-uniform constants.
+struct DropoutKey {
+  uint32_t row_salt;    // row ^ 0xb5297a4d
+  uint32_t head_salt;   // head ^ 0x63d83595
+  uint32_t batch_salt;  // batch ^ 0xa511e9b3
+  uint32_t seed_low;
+  uint32_t seed_high_salt;  // seed_high ^ 0x9e3779b9
+};
+
+__device__ __forceinline__ float dropout_multiplier(const DropoutKey& key, int route,
+                                                    float dropout_p, float inverse_keep) {
+  uint32_t s = mix32(static_cast<uint32_t>(route) ^ 0x68e31da4u);
+  s = mix32(s ^ key.row_salt);
+  s = mix32(s ^ key.head_salt);
+  s = mix32(s ^ key.batch_salt);
+  s = mix32(s ^ key.seed_low);
+  s = mix32(s ^ key.seed_high_salt);
+  const float uniform = static_cast<float>(s >> 8) * 0x1.0p-24f;
+  return uniform >= dropout_p ? inverse_keep : 0.0f;
+}
+
+// ---------------------------------------------------------------------------
+// layout
+// ---------------------------------------------------------------------------
+
+struct Layout {
+  int B, T, N, S, H, D, Hv, Dv, W;
+  int varlen;
+  // packed-sequence tables (device), valid when varlen != 0
+  const int32_t* seq_start;
+  const int32_t* seq_len;
+  const int32_t* block_prefix;  // [S+1] prefix sums of ceil(len / 64)
+  int slots;                    // number of 64-row block slots over all sequences (upper bound)
+};
+
+struct Unit {
+  int seq;     // batch index (dense) or packed sequence index
+  int block;   // 64-row block / 64-diagonal band index inside the sequence
+  int start;   // first token of the sequence in token-major tensors
+  int len;     // sequence length
+  int head;
+  int64_t word_base;  // offset of (seq, head, t = 0) in the head-major word tensors
+  bool valid;
+};
+
+// slot order is block-major so that equal block indices of all sequences are adjacent
+template <bool VARLEN>
+__device__ __forceinline__ Unit decode_unit(const Layout& L, int unit_index) {
+  Unit u;
+  u.head = unit_index % L.H;
+  const int slot = unit_index / L.H;
+  u.valid = true;
+  if constexpr (VARLEN) {
+    int low = 0, high = L.S;  // find seq with prefix[seq] <= slot < prefix[seq+1]
+    while (low < high) {
+      const int mid = (low + high) >> 1;
+      if (L.block_prefix[mid + 1] <= slot) low = mid + 1; else high = mid;
+    }
+    if (low >= L.S) {
+      u.valid = false;
+      u.seq = 0; u.block = 0; u.start = 0; u.len = 0; u.word_base = 0;
+      return u;
+    }
+    u.seq = low;
+    u.block = slot - L.block_prefix[low];
+    u.start = L.seq_start[low];
+    u.len = L.seq_len[low];
+    u.word_base = static_cast<int64_t>(u.head) * L.N + u.start;
+  } else {
+    u.seq = slot % L.B;
+    u.block = slot / L.B;
+    u.start = u.seq * L.T;
+    u.len = L.T;
+    u.word_base = (static_cast<int64_t>(u.seq) * L.H + u.head) * L.T;
+  }
+  return u;
+}
+
+// ---------------------------------------------------------------------------
+// packed-sequence table: sanitised offsets and block prefix sums
+// ---------------------------------------------------------------------------
+
+__global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens, int S, int N,
+                                         int32_t* __restrict__ seq_start,
+                                         int32_t* __restrict__ seq_len,
+                                         int32_t* __restrict__ block_prefix,
+                                         int32_t* __restrict__ header) {
+  // single block; offsets are clamped into [previous, N] so that no later
+  // kernel can index outside the tensors, and any violation is recorded.
+  __shared__ int bad;
+  __shared__ int partial[256];
+  if (threadIdx.x == 0) bad = 0;
+  __syncthreads();
+  const int per_thread = (S + blockDim.x - 1) / blockDim.x;
+  const int first = threadIdx.x * per_thread;
+  const int last = min(S, first + per_thread);
+  int local_bad = 0;
+  int blocks = 0;
+  for (int s = first; s < last; ++s) {
+    const int raw_begin = cu_seqlens[s];
+    const int raw_end = cu_seqlens[s + 1];
+    if (raw_begin > raw_end || raw_begin < 0 || raw_end > N) local_bad = 1;
+    const int begin = min(max(raw_begin, 0), N);
+    const int end = min(max(raw_end, begin), N);
+    seq_start[s] = begin;
+    seq_len[s] = end - begin;
+    blocks += (end - begin + 63) >> 6;
+  }
+  if (threadIdx.x == 0) {
+    if (cu_seqlens[0] != 0) local_bad = 1;
+    if (cu_seqlens[S] != N) local_bad = 1;
+  }
+  if (local_bad) atomicOr(&bad, 1);
+  partial[threadIdx.x] = blocks;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int running = 0;
+    for (int i = 0; i < static_cast<int>(blockDim.x); ++i) {
+      const int value = partial[i];
+      partial[i] = running;
+      running += value;
+    }
+    block_prefix[S] = running;
+    header[0] = bad;
+  }
+  __syncthreads();
+  int running = partial[threadIdx.x];
+  for (int s = first; s < last; ++s) {
+    block_prefix[s] = running;
+    running += (seq_len[s] + 63) >> 6;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// sign packing (wave64 ballot)
+// ---------------------------------------------------------------------------
+
+// Each lane reads one element of query and key; one 64-bit ballot then holds
+// 64 / D complete symbols, which the first 64 / D lanes write out head-major.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void pack_symbols_ballot_kernel(
+    const void* __restrict__ query, const void* __restrict__ key,
+    int32_t* __restrict__ packed_query, int32_t* __restrict__ packed_key, int64_t elements,
+    int D, int H, int T, int N, int varlen) {
+  const int64_t element = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool in_range = element < elements;
+  const bool q_bit = in_range && load_as_float<DTYPE>(query, element) > 0.0f;
+  const bool k_bit = in_range && load_as_float<DTYPE>(key, element) > 0.0f;
+  const uint64_t q_mask = __ballot(q_bit);
+  const uint64_t k_mask = __ballot(k_bit);
+  const int lane = threadIdx.x & 63;
+  const int symbols_per_wave = 64 / D;
+  if (lane < symbols_per_wave) {
+    const int64_t wave_first = element - lane;       // multiple of 64, hence of D
+    const int64_t row = wave_first / D + lane;       // row = token * H + h
+    if (row * D < elements) {
+      const uint32_t field = D == 32 ? 0xffffffffu : ((1u << D) - 1u);
+      const uint32_t q_word = static_cast<uint32_t>(q_mask >> (lane * D)) & field;
+      const uint32_t k_word = static_cast<uint32_t>(k_mask >> (lane * D)) & field;
+      const int64_t token = row / H;
+      const int h = static_cast<int>(row - token * H);
+      int64_t dst;
+      if (varlen) {
+        dst = static_cast<int64_t>(h) * N + token;
+      } else {
+        const int64_t b = token / T;
+        dst = (b * H + h) * T + (token - b * T);
+      }
+      packed_query[dst] = static_cast<int32_t>(q_word);
+      packed_key[dst] = static_cast<int32_t>(k_word);
+    }
+  }
+}
+
+// Widths that do not divide 64: one lane per symbol.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void pack_symbols_rows_kernel(
+    const void* __restrict__ query, const void* __restrict__ key,
+    int32_t* __restrict__ packed_query, int32_t* __restrict__ packed_key, int64_t rows, int D,
+    int H, int T, int N, int varlen) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  uint32_t q_word = 0u, k_word = 0u;
+  for (int bit = 0; bit < D; ++bit) {
+    if (load_as_float<DTYPE>(query, row * D + bit) > 0.0f) q_word |= 1u << bit;
+    if (load_as_float<DTYPE>(key, row * D + bit) > 0.0f) k_word |= 1u << bit;
+  }
+  const int64_t token = row / H;
+  const int h = static_cast<int>(row - token * H);
+  int64_t dst;
+  if (varlen) {
+    dst = static_cast<int64_t>(h) * N + token;
+  } else {
+    const int64_t b = token / T;
+    dst = (b * H + h) * T + (token - b * T);
+  }
+  packed_query[dst] = static_cast<int32_t>(q_word);
+  packed_key[dst] = static_cast<int32_t>(k_word);
+}
+
+// ---------------------------------------------------------------------------
+// hard forward: latest-longest route per row
+// ---------------------------------------------------------------------------
+
+// One wave owns 64 consecutive rows (lane = row) and walks over routes a.
+// The run length obeys run(t, a) = eq(t, a) ? min(run(t-1, a-1) + 1, W) : 0;
+// run(t-1, a-1) is the previous step's value of the lane above, fetched with
+// one DPP shift.  Lane 0 has no lane above: its predecessor row t0-1 is
+// evaluated directly, 64 routes at a time, by an early-exit compare loop.
+// The winner is the maximum of the packed key (run << shift) | a, which is
+// "longest first, latest on ties"; a zero run never produces a route.
+template <bool VARLEN, bool WIDE>
+__global__ __launch_bounds__(kWave) void hard_route_kernel(
+    Layout L, const uint32_t* __restrict__ packed_query,
+    const uint32_t* __restrict__ packed_key, int32_t* __restrict__ routes,
+    int32_t* __restrict__ source_token, int shift) {
+  const Unit u = decode_unit<VARLEN>(L, blockIdx.x);
+  if (!u.valid) return;
+  const int blocks = (u.len + 63) >> 6;
+  if (u.block >= blocks) return;
+  const int row_block = blocks - 1 - u.block;  // longest rows are scheduled first
+  const int t0 = row_block * kWave;
+  const int lane = threadIdx.x;
+  const uint32_t* q = packed_query + u.word_base;
+  const uint32_t* k = packed_key + u.word_base;
+  const int t = t0 + lane;
+  const bool row_ok = t < u.len;
+  const uint32_t q_word = row_ok ? q[t] : 0u;
+  const int W = L.W;
+  using Best = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+  Best best = 0;
+  int run = 0;
+  const int a_last = min(t0 + kWave - 1, u.len - 1);
+  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+    const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
+    int halo = 0;
+    if (column >= 1 && column <= t0 - 1) {
+      const int limit = min(W, column);
+      while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+    }
+    const uint32_t key_chunk = column < u.len ? k[column] : 0u;  // key word of route a0 + lane
+    const int count = min(kWave, a_last - a0 + 1);
+#pragma unroll
+    for (int j = 0; j < kWave; ++j) {
+      if (j >= count) break;
+      const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
+      const int halo_j = __builtin_amdgcn_readlane(halo, j);
+      const int above = dpp_wave_shr1(halo_j, run);
+      const int a = a0 + j;
+      const bool match = (q_word == k_word) && (a <= t);
+      run = match ? min(above + 1, W) : 0;
+      if constexpr (WIDE) {
+        best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
+      } else {
+        best = max(best, (static_cast<uint32_t>(run) << shift) | static_cast<uint32_t>(a));
+      }
+    }
+  }
+  if (!row_ok) return;
+  int best_run, best_route;
+  if constexpr (WIDE) {
+    best_run = static_cast<int>(best >> 32);
+    best_route = static_cast<int>(best & 0xffffffffu);
+  } else {
+    best_run = static_cast<int>(best >> shift);
+    best_route = static_cast<int>(best & ((1u << shift) - 1u));
+  }
+  const int route = best_run > 0 ? best_route : 0;
+  if (routes != nullptr) routes[u.word_base + t] = route;
+  source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
+}
+
+// output[token, h, :] = sign(value[source, h / group, :]) or exact zero
+template <int DTYPE>
+__global__ __launch_bounds__(256) void gather_values_kernel(
+    const int32_t* __restrict__ source_token, const void* __restrict__ value,
+    void* __restrict__ output, int64_t elements, int H, int Hv, int Dv, int T, int N,
+    int varlen) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= elements) return;
+  const int d = static_cast<int>(index % Dv);
+  const int64_t row = index / Dv;
+  const int h = static_cast<int>(row % H);
+  const int64_t token = row / H;
+  int64_t word;
+  if (varlen) {
+    word = static_cast<int64_t>(h) * N + token;
+  } else {
+    const int64_t b = token / T;
+    word = (b * H + h) * T + (token - b * T);
+  }
+  const int source = source_token[word];
+  int sign = 0;
+  if (source >= 0) {
+    const int hv = h / (H / Hv);
+    const float x = load_as_float<DTYPE>(
+        value, (static_cast<int64_t>(source) * Hv + hv) * Dv + d);
+    sign = x > 0.0f ? 1 : -1;
+  }
+  store_sign<DTYPE>(output, index, sign);
+}
+
+// ---------------------------------------------------------------------------
+// backward: preparation
+// ---------------------------------------------------------------------------
+
+struct VjpParams {
+  Layout L;
+  const uint32_t* packed_query;
+  const uint32_t* packed_key;
+  const uint32_t* value_bits;   // [value_words_total][NVW], head-major over value heads
+  const float* grad_rows;       // [head-major row][DVP] float32, zero padded
+  const float* grad_row_sum;    // [head-major row]
+  float4* stats;                // [head-major row] (reference logit, denominator, numerator, base)
+  const int64_t* dropout_seed;
+  float scale, dropout_p, inverse_keep, mismatch_scale;
+  float gate_log2;              // mismatch_scale * log2(e) / D
+  float logit_gain;             // scale * (sqrt2+1) * log2(e)
+  float null_logit;             // 0.5 * scale
+  float tail_threshold;         // window products below this are treated as zero in the reverse sweep
+  int gradient_mask;
+  int dvp;                      // padded value width
+  float* grad_query;            // symbol-space accumulators, token-major
+  float* grad_key;
+  float* grad_value;
+  int32_t* work_counter;
+  float* block_scratch;         // per resident block: ring + segment checkpoints
+  int64_t block_scratch_floats;
+  int ring_rows;                // W + 1 clipped to the longest possible diagonal
+  int total_units;
+};
+
+// grad_output -> float32 head-major rows padded to DVP, plus the row sums
+template <int DTYPE>
+__global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
+    const void* __restrict__ grad_output, float* __restrict__ grad_rows,
+    float* __restrict__ grad_row_sum, int64_t rows, int H, int Dv, int dvp, int T, int N,
+    int varlen) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (row >= rows) return;  // row = token * H + h (token-major)
+  const int64_t token = row / H;
+  const int h = static_cast<int>(row - token * H);
+  int64_t dst;
+  if (varlen) {
+    dst = static_cast<int64_t>(h) * N + token;
+  } else {
+    const int64_t b = token / T;
+    dst = (b * H + h) * T + (token - b * T);
+  }
+  float total = 0.0f;
+  for (int d = 0; d < dvp; ++d) {
+    float g = 0.0f;
+    if (d < Dv) g = load_as_float<DTYPE>(grad_output, row * Dv + d);
+    grad_rows[dst * dvp + d] = g;
+    total += g;
+  }
+  grad_row_sum[dst] = total;
+}
+
+// value sign bits, head-major over value heads: word index (seq, hv, t) like the symbol words
+template <int DTYPE>
+__global__ __launch_bounds__(256) void pack_value_bits_kernel(
+    const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
+    int Dv, int nvw, int T, int N, int varlen) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (row >= rows) return;  // row = token * Hv + hv
+  const int64_t token = row / Hv;
+  const int hv = static_cast<int>(row - token * Hv);
+  int64_t dst;
+  if (varlen) {
+    dst = static_cast<int64_t>(hv) * N + token;
+  } else {
+    const int64_t b = token / T;
+    dst = (b * Hv + hv) * T + (token - b * T);
+  }
+  for (int w = 0; w < nvw; ++w) {
+    uint32_t word = 0u;
+    for (int bit = 0; bit < 32; ++bit) {
+      const int d = w * 32 + bit;
+      if (d < Dv && load_as_float<DTYPE>(value, row * Dv + d) > 0.0f) word |= 1u << bit;
+    }
+    value_bits[dst * nvw + w] = word;
+  }
+}
+
+// Per row: the reference point of the softmax exponent and the constant part
+// of the logit.  With `analytic` the reference point is the upper bound
+// max(null, scale*U(min(W, t)) - log t) of every logit of the row, otherwise it
+// starts at the null logit and a separate pass raises it to the row maximum.
+template <bool VARLEN>
+__global__ __launch_bounds__(256) void init_row_stats_kernel(Layout L, float4* __restrict__ stats,
+                                                             float scale, int analytic,
+                                                             int32_t* __restrict__ work_counter) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index == 0) *work_counter = 0;
+  const int64_t rows = static_cast<int64_t>(L.N) * L.H;
+  if (index >= rows) return;
+  // head-major index -> local row t
+  int t;
+  if constexpr (VARLEN) {
+    const int token = static_cast<int>(index % L.N);
+    int low = 0, high = L.S;  // sequence containing the token (empty sequences are skipped)
+    while (low < high) {
+      const int mid = (low + high) >> 1;
+      if (L.seq_start[mid] + L.seq_len[mid] <= token) low = mid + 1; else high = mid;
+    }
+    t = low < L.S ? token - L.seq_start[low] : 0;
+    if (t < 0) t = 0;
+  } else {
+    t = static_cast<int>(index % L.T);
+  }
+  const float null_logit = kNullScore * scale;
+  const float log_count = t > 0 ? logf(static_cast<float>(t)) : 0.0f;
+  float reference = null_logit;
+  if (analytic) {
+    const float longest = static_cast<float>(min(L.W, t));
+    const float bound = scale * kSqrtScale * (sqrtf(1.0f + longest) - 1.0f) - log_count;
+    reference = fmaxf(null_logit, bound);
+  }
+  const float base = (scale * kSqrtScale + log_count) * kLog2e;
+  stats[index] = make_float4(reference, 0.0f, 0.0f, base);
+}
+
+// ---------------------------------------------------------------------------
+// backward: diagonal-band sweeps
+// ---------------------------------------------------------------------------
+
+template <int NVW>
+struct Band {
+  // sliding per-column registers (lane l holds the column a = a0 - l)
+  uint32_t key_word;      // key word of column a     (key position a - 1)
+  uint32_t old_key_word;  // key word of column a - W - 1, leaving the window
+  uint32_t value_bits[NVW];
+  // per-diagonal state
+  float evidence;   // S of the previous row on this diagonal
+  int window;       // mismatching bits over the last min(n, W + 1) gates
+};
+
+struct BandView {
+  const uint32_t* q;       // head-major words of this (sequence, head)
+  const uint32_t* k;
+  const uint32_t* vbits;   // value sign words of this (sequence, value head), NVW per token
+  const float* grad_rows;  // [t][dvp]
+  const float* grad_sum;   // [t]
+  float4* stats;           // [t]
+  int len;
+  int diag0;               // first diagonal of the band
+  int steps;               // rows of the band: t = diag0 + 1 + i
+};
+
+// Load the sliding registers so that the shift of step i produces columns a0 - l, a0 = i + 1.
+template <int NVW>
+__device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& view, int i,
+                                             int lane, int W) {
+  const int a = i - lane;  // column held before the shift
+  band.key_word = (a >= 1) ? view.k[a - 1] : 0u;
+  band.old_key_word = (a - W - 2 >= 0) ? view.k[a - W - 2] : 0u;
+#pragma unroll
+  for (int w = 0; w < NVW; ++w) {
+    band.value_bits[w] = (a >= 1) ? view.vbits[static_cast<int64_t>(a) * NVW + w] : 0u;
+  }
+}
+
+struct StepOut {
+  float gate;     // local match gate of this pair
+  float overflow; // product of the W+1 gates ending here (0 while the window is not full)
+  float evidence; // S(t, a)
+  bool active;    // a >= 1
+  int a;
+};
+
+// One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
+template <int NVW>
+__device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const BandView& view, int i,
+                                                int lane, int W, float gate_log2) {
+  const int t = view.diag0 + 1 + i;
+  const int a0 = i + 1;
+  const uint32_t q_word = view.q[t];
+  const uint32_t q_old = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+  const uint32_t k_new = view.k[a0 - 1];
+  const uint32_t k_old_new = (a0 - W - 2 >= 0) ? view.k[a0 - W - 2] : 0u;
+  band.key_word = dpp_wave_shr1(k_new, band.key_word);
+  band.old_key_word = dpp_wave_shr1(k_old_new, band.old_key_word);
+#pragma unroll
+  for (int w = 0; w < NVW; ++w) {
+    const uint32_t v_new = view.vbits[static_cast<int64_t>(a0) * NVW + w];
+    band.value_bits[w] = dpp_wave_shr1(v_new, band.value_bits[w]);
+  }
+  StepOut out;
+  out.a = a0 - lane;
+  out.active = out.a >= 1;
+  const int mismatches = __popc(q_word ^ band.key_word);
+  const int leaving = (out.a >= W + 2) ? __popc(q_old ^ band.old_key_word) : 0;
+  band.window = out.active ? band.window + mismatches - leaving : 0;
+  out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
+  out.overflow =
+      (out.a >= W + 1) ? fast_exp2(-gate_log2 * static_cast<float>(band.window)) : 0.0f;
+  const float next = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
+  band.evidence = out.active ? next : 0.0f;
+  out.evidence = band.evidence;
+  return out;
+}
+
+template <int NVW, int DVP>
+__device__ __forceinline__ float route_utility(const Band<NVW>& band, const float* grad_row,
+                                               float grad_sum) {
+  // u = sum_d go[d] * sign_d = 2 * sum_{d: bit set} go[d] - sum_d go[d]
+  float picked = 0.0f;
+#pragma unroll
+  for (int d = 0; d < DVP; ++d) {
+    const int mask = static_cast<int>(band.value_bits[d >> 5] << (31 - (d & 31))) >> 31;
+    picked += __int_as_float(__float_as_int(grad_row[d]) & mask);
+  }
+  return fmaf(2.0f, picked, -grad_sum);
+}
+
+template <int NVW, bool VARLEN>
+__device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, BandView& view,
+                                          int& value_head) {
+  view.len = u.len;
+  view.diag0 = u.block * kWave;
+  view.steps = u.len - 1 - view.diag0;
+  if (view.steps <= 0) return false;
+  view.q = P.packed_query + u.word_base;
+  view.k = P.packed_key + u.word_base;
+  value_head = u.head / (P.L.H / P.L.Hv);
+  const int64_t value_base = VARLEN
+      ? static_cast<int64_t>(value_head) * P.L.N + u.start
+      : (static_cast<int64_t>(u.seq) * P.L.Hv + value_head) * P.L.T;
+  view.vbits = P.value_bits + value_base * NVW;
+  view.grad_rows = P.grad_rows + u.word_base * P.dvp;
+  view.grad_sum = P.grad_row_sum + u.word_base;
+  view.stats = P.stats + u.word_base;
+  return true;
+}
+
+// Row-maximum pass (only when the analytic bound is too loose to be a safe
+// exponent reference): raises stats[t].x to the largest logit of the row.
+template <int NVW, bool VARLEN>
+__global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
+  const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
+  if (!u.valid) return;
+  BandView view;
+  int hv;
+  if (!make_view<NVW, VARLEN>(P, u, view, hv)) return;
+  const int lane = threadIdx.x;
+  const int W = P.L.W;
+  Band<NVW> band;
+  band.evidence = 0.0f;
+  band.window = 0;
+  load_sliding<NVW>(band, view, 0, lane, W);
+  for (int i = 0; i < view.steps; ++i) {
+    const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
+    const int t = view.diag0 + 1 + i;
+    const float root = sqrtf(1.0f + s.evidence);
+    const float logit =
+        P.scale * kSqrtScale * (root - 1.0f) - logf(static_cast<float>(t));
+    float best = s.active ? fmaxf(logit, 0.0f) : 0.0f;
+    best = wave_max_lane63(best);
+    if (lane == 63) {
+      atomicMax(reinterpret_cast<int*>(&view.stats[t].x), __float_as_int(best));
+    }
+  }
+}
+
+// Row-statistics pass: denominator and expected dropped utility of every row.
+template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
+__global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
+  const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
+  if (!u.valid) return;
+  BandView view;
+  int hv;
+  if (!make_view<NVW, VARLEN>(P, u, view, hv)) return;
+  const int lane = threadIdx.x;
+  const int W = P.L.W;
+  DropoutKey key;
+  if constexpr (DROPOUT) {
+    const uint64_t seed = static_cast<uint64_t>(*P.dropout_seed);
+    key.head_salt = static_cast<uint32_t>(u.head) ^ 0x63d83595u;
+    key.batch_salt = static_cast<uint32_t>(u.seq) ^ 0xa511e9b3u;
+    key.seed_low = static_cast<uint32_t>(seed);
+    key.seed_high_salt = static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u;
+  }
+  Band<NVW> band;
+  band.evidence = 0.0f;
+  band.window = 0;
+  load_sliding<NVW>(band, view, 0, lane, W);
+  const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
+  for (int i = 0; i < view.steps; ++i) {
+    const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
+    const int t = view.diag0 + 1 + i;
+    const float4 row = view.stats[t];
+    const float shift = fmaf(row.x, kLog2e, row.w);
+    const float one_plus = 1.0f + s.evidence;
+    const float root = one_plus * fast_rsq(one_plus);
+    const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
+    float numerator = 0.0f;
+    if (needs_utility) {
+      const float utility =
+          route_utility<NVW, DVP>(band, view.grad_rows + static_cast<int64_t>(t) * DVP,
+                                  view.grad_sum[t]);
+      float keep = 1.0f;
+      if constexpr (DROPOUT) {
+        key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+        keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
+      }
+      numerator = weight * keep * utility;
+    }
+    const float weight_sum = wave_sum_lane63(weight);
+    const float numerator_sum = wave_sum_lane63(numerator);
+    if (lane == 63) {
+      atomicAdd(&view.stats[t].y, weight_sum);
+      if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
+    }
+  }
+}
+
+// Gradient pass.  Persistent blocks pull bands from a work counter.  A band is
+// processed from its last row upwards because the gate adjoint
+//   h(n) = b(n) (S(n) + overflow(n)) - sum_{m=n..n+W} b(m) overflow(m),
+//   b(n) = A(n) + gate(n+1) b(n+1)
+// needs the adjoints of later rows, while S needs earlier rows.  S is
+// therefore rebuilt from checkpoints: one cheap forward sweep per band stores
+// (S, window) every kSegment rows, one per segment stores them every kChunk
+// rows in LDS, and each chunk is then replayed forward into registers and
+// walked backwards.  The windowed sum of b*overflow lives in a ring of W+1
+// rows in global memory that is touched only while some overflow term of the
+// wave is above `tail_threshold` (long near-exact matches).
+//
+// Each chunk leaves its route weights d*p and gate adjoints h in LDS as
+// [row][lane] tiles, from which the three contractions are formed with one
+// output element per lane:
+//   dV[a, :]   += sum_t  d p(t, a) go[t, :]
+//   dK[a-1, :] += c sum_t h(t, a) z(q[t, :])
+//   dQ[t, :]   += c sum_a h(t, a) z(k[a-1, :]),   c = mismatch_scale / (2 D)
+// Column sums complete after 64 rows, so they are kept in circular LDS
+// accumulators and flushed with one global atomic per element.
+template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
+__global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
+  extern __shared__ float lds[];
+  float* ck_evidence = lds;                                  // [kSegChunks][64]
+  int* ck_window = reinterpret_cast<int*>(lds + kSegChunks * kWave);
+  float* weight_tile = lds + 2 * kSegChunks * kWave;         // [kChunk][64]
+  float* adjoint_tile = weight_tile + kChunk * kWave;        // [kChunk][64]
+  float* grad_tile = adjoint_tile + kChunk * kWave;          // [kChunk][DVP]
+  uint32_t* key_tile = reinterpret_cast<uint32_t*>(grad_tile + kChunk * DVP);  // [kChunk + 64]
+  uint32_t* query_tile = key_tile + kChunk + kWave;          // [kChunk]
+  float* value_acc = reinterpret_cast<float*>(query_tile + kChunk);  // [kColumnRing][DVP]
+  float* key_acc = value_acc + kColumnRing * DVP;            // [kColumnRing][D]
+
+  const int lane = threadIdx.x;
+  const int W = P.L.W;
+  const int D = P.L.D;
+  const int Dv = P.L.Dv;
+  const bool want_q = (P.gradient_mask & ROSA_GRAD_QUERY) != 0;
+  const bool want_k = (P.gradient_mask & ROSA_GRAD_KEY) != 0;
+  const bool want_v = (P.gradient_mask & ROSA_GRAD_VALUE) != 0;
+  const bool want_qk = want_q || want_k;
+  const float symbol_scale = 0.5f * P.mismatch_scale / static_cast<float>(D);
+  float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
+  float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
+
+  for (;;) {
+    int unit_index = 0;
+    if (lane == 0) unit_index = atomicAdd(P.work_counter, 1);
+    unit_index = __builtin_amdgcn_readfirstlane(unit_index);
+    if (unit_index >= P.total_units) break;
+    const Unit u = decode_unit<VARLEN>(P.L, unit_index);
+    if (!u.valid) continue;
+    BandView view;
+    int hv;
+    if (!make_view<NVW, VARLEN>(P, u, view, hv)) continue;
+    DropoutKey key;
+    if constexpr (DROPOUT) {
+      const uint64_t seed = static_cast<uint64_t>(*P.dropout_seed);
+      key.head_salt = static_cast<uint32_t>(u.head) ^ 0x63d83595u;
+      key.batch_salt = static_cast<uint32_t>(u.seq) ^ 0xa511e9b3u;
+      key.seed_low = static_cast<uint32_t>(seed);
+      key.seed_high_salt = static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u;
+    }
+
+    // clear the circular column accumulators
+    for (int index = lane; index < kColumnRing * DVP; index += kWave) value_acc[index] = 0.0f;
+    for (int index = lane; index < kColumnRing * D; index += kWave) key_acc[index] = 0.0f;
+
+    const int segments = (view.steps + kSegment - 1) / kSegment;
+    Band<NVW> band;
+    // band-level forward sweep: checkpoint (S, window) before the first row of every segment
+    if (segments > 1) {
+      band.evidence = 0.0f;
+      band.window = 0;
+      load_sliding<NVW>(band, view, 0, lane, W);
+      for (int i = 0; i < (segments - 1) * kSegment; ++i) {
+        if ((i % kSegment) == 0) {
+          const int segment = i / kSegment;
+          seg_ck[(2 * segment) * kWave + lane] = band.evidence;
+          seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+        }
+        forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
+      }
+      const int segment = segments - 1;
+      seg_ck[(2 * segment) * kWave + lane] = band.evidence;
+      seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+    }
+
+    // reverse state carried across chunks and segments
+    float adjoint_carry = 0.0f;   // b of the row below on this diagonal
+    float gate_below = 0.0f;      // gate of the row below
+    float ring_sum = 0.0f;        // sum of b * overflow over the next W + 1 rows
+    int ring_live = 0;            // rows for which the ring still holds non-zero terms
+    int ring_fresh = 0;           // ring reads that must be treated as zero
+
+    for (int segment = segments - 1; segment >= 0; --segment) {
+      const int seg_first = segment * kSegment;
+      const int seg_last = min(view.steps, seg_first + kSegment);
+      if (segments > 1) {
+        band.evidence = seg_ck[(2 * segment) * kWave + lane];
+        band.window = __float_as_int(seg_ck[(2 * segment + 1) * kWave + lane]);
+      } else {
+        band.evidence = 0.0f;
+        band.window = 0;
+      }
+      load_sliding<NVW>(band, view, seg_first, lane, W);
+      const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
+      // segment-level forward sweep: checkpoint before every chunk
+      for (int chunk = 0; chunk < chunks; ++chunk) {
+        ck_evidence[chunk * kWave + lane] = band.evidence;
+        ck_window[chunk * kWave + lane] = band.window;
+        if (chunk + 1 < chunks) {
+          const int first = seg_first + chunk * kChunk;
+#pragma unroll 4
+          for (int r = 0; r < kChunk; ++r) {
+            forward_step<NVW>(band, view, first + r, lane, W, P.gate_log2);
+          }
+        }
+      }
+
+      for (int chunk = chunks - 1; chunk >= 0; --chunk) {
+        const int first = seg_first + chunk * kChunk;   // step index of the chunk's first row
+        const int rows = min(kChunk, seg_last - first);
+        band.evidence = ck_evidence[chunk * kWave + lane];
+        band.window = ck_window[chunk * kWave + lane];
+        load_sliding<NVW>(band, view, first, lane, W);
+
+        float keep_evidence[kChunk];  // S + overflow
+        float keep_overflow[kChunk];
+        float keep_gate[kChunk];
+        float keep_adjoint[kChunk];   // external adjoint A of the route score
+
+        // forward replay of the chunk
+#pragma unroll
+        for (int r = 0; r < kChunk; ++r) {
+          if (r < rows) {
+            const int i = first + r;
+            const int t = view.diag0 + 1 + i;
+            const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
+            const float4 row = view.stats[t];
+            const float shift = fmaf(row.x, kLog2e, row.w);
+            const float one_plus = 1.0f + s.evidence;
+            const float inv_root = fast_rsq(one_plus);
+            const float root = one_plus * inv_root;
+            const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
+            const float null_weight = fast_exp2((P.null_logit - row.x) * kLog2e);
+            const float inv_denominator = fast_rcp(row.y + null_weight);
+            const float probability = weight * inv_denominator;
+            float keep = 1.0f;
+            if constexpr (DROPOUT) {
+              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+              keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
+            }
+            weight_tile[r * kWave + lane] = probability * keep;
+            float adjoint = 0.0f;
+            if (want_qk) {
+              const float utility = route_utility<NVW, DVP>(
+                  band, view.grad_rows + static_cast<int64_t>(t) * DVP, view.grad_sum[t]);
+              const float expected = row.z * inv_denominator;
+              adjoint = P.scale * probability * (keep * utility - expected) *
+                        (0.5f * kSqrtScale * inv_root);
+            }
+            keep_adjoint[r] = adjoint;
+            keep_gate[r] = s.gate;
+            keep_overflow[r] = s.overflow;
+            keep_evidence[r] = s.evidence + s.overflow;
+          } else {
+            keep_adjoint[r] = 0.0f;
+            keep_gate[r] = 0.0f;
+            keep_overflow[r] = 0.0f;
+            keep_evidence[r] = 0.0f;
+            weight_tile[r * kWave + lane] = 0.0f;
+          }
+        }
+
+        // reverse walk of the chunk
+        if (want_qk) {
+#pragma unroll
+          for (int r = kChunk - 1; r >= 0; --r) {
+            if (r < rows) {
+              const int i = first + r;
+              const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
+              adjoint_carry = b;
+              gate_below = keep_gate[r];
+              const float overflow = keep_overflow[r];
+              const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
+              const bool any_term = __ballot(term != 0.0f) != 0ull;
+              if (any_term) {
+                if (ring_live == 0) ring_fresh = P.ring_rows;
+                ring_live = P.ring_rows;
+              }
+              if (ring_live > 0) {
+                const int slot = i % P.ring_rows;
+                float leaving = 0.0f;
+                if (ring_fresh > 0) {
+                  --ring_fresh;
+                } else {
+                  leaving = ring[slot * kWave + lane];
+                }
+                ring[slot * kWave + lane] = term;
+                ring_sum += term - leaving;
+                --ring_live;
+              }
+              const float h = fmaf(b, keep_evidence[r], -ring_sum);
+              if (ring_live == 0) ring_sum = 0.0f;
+              const bool active = (i + 1 - lane) >= 1;
+              adjoint_tile[r * kWave + lane] = active ? h : 0.0f;
+            } else {
+              adjoint_tile[r * kWave + lane] = 0.0f;
+            }
+          }
+        }
+
+        // stage the row data of the chunk
+        const int t_first = view.diag0 + 1 + first;
+        const int a_first = first + 1;  // column of lane 0 in the chunk's first row
+        for (int index = lane; index < kChunk * DVP; index += kWave) {
+          const int r = index / DVP;
+          grad_tile[index] =
+              r < rows ? view.grad_rows[static_cast<int64_t>(t_first + r) * DVP + (index % DVP)]
+                       : 0.0f;
+        }
+        if (lane < kChunk) query_tile[lane] = lane < rows ? view.q[t_first + lane] : 0u;
+        for (int index = lane; index < kChunk + kWave - 1; index += kWave) {
+          const int a = a_first - 63 + index;  // column; key position a - 1
+          key_tile[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
+        }
+        __syncthreads();
+
+        const int columns = kChunk + kWave - 1;  // a = a_first - 63 + c
+        if (want_v) {
+          for (int out = lane; out < columns * DVP; out += kWave) {
+            const int c = out / DVP;
+            const int d = out - c * DVP;
+            const int a = a_first - 63 + c;
+            if (a < 1) continue;
+            // pair (row r, column a) sits in lane l = 63 - c + r
+            const int r_low = max(0, c - 63);
+            const int r_high = min(kChunk - 1, c);
+            float total = 0.0f;
+            for (int r = r_low; r <= r_high; ++r) {
+              total = fmaf(weight_tile[r * kWave + (63 - c + r)], grad_tile[r * DVP + d], total);
+            }
+            value_acc[(a & (kColumnRing - 1)) * DVP + d] += total;
+          }
+        }
+        if (want_k) {
+          for (int out = lane; out < columns * D; out += kWave) {
+            const int c = out / D;
+            const int bit = out - c * D;
+            const int a = a_first - 63 + c;
+            if (a < 1) continue;
+            const int r_low = max(0, c - 63);
+            const int r_high = min(kChunk - 1, c);
+            float total = 0.0f;
+            for (int r = r_low; r <= r_high; ++r) {
+              const float h = adjoint_tile[r * kWave + (63 - c + r)];
+              total += ((query_tile[r] >> bit) & 1u) ? h : -h;
+            }
+            key_acc[(a & (kColumnRing - 1)) * D + bit] += total;
+          }
+        }
+        if (want_q) {
+          for (int out = lane; out < kChunk * D; out += kWave) {
+            const int r = out / D;
+            const int bit = out - r * D;
+            if (r >= rows) continue;
+            float total = 0.0f;
+            for (int l = 0; l < kWave; ++l) {
+              const float h = adjoint_tile[r * kWave + l];
+              total += ((key_tile[63 + r - l] >> bit) & 1u) ? h : -h;
+            }
+            const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
+            atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit], symbol_scale * total);
+          }
+        }
+        __syncthreads();
+        // columns a_first .. a_first + rows - 1 are complete for this band
+        if (want_v) {
+          for (int out = lane; out < rows * DVP; out += kWave) {
+            const int c = out / DVP;
+            const int d = out - c * DVP;
+            const int a = a_first + c;
+            float* slot = &value_acc[(a & (kColumnRing - 1)) * DVP + d];
+            const float total = *slot;
+            *slot = 0.0f;
+            if (d < Dv && total != 0.0f) {
+              const int64_t token = static_cast<int64_t>(u.start) + a;
+              atomicAdd(&P.grad_value[(token * P.L.Hv + hv) * Dv + d], total);
+            }
+          }
+        }
+        if (want_k) {
+          for (int out = lane; out < rows * D; out += kWave) {
+            const int c = out / D;
+            const int bit = out - c * D;
+            const int a = a_first + c;
+            float* slot = &key_acc[(a & (kColumnRing - 1)) * D + bit];
+            const float total = *slot;
+            *slot = 0.0f;
+            if (total != 0.0f) {
+              const int64_t token = static_cast<int64_t>(u.start) + a - 1;
+              atomicAdd(&P.grad_key[(token * P.L.H + u.head) * D + bit], symbol_scale * total);
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// Softsign Jacobian 1 / (1 + |x|)^2 applied once to the symbol-space sums.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void finalize_gradients_kernel(
+    const void* __restrict__ query, const void* __restrict__ key,
+    const void* __restrict__ value, float* __restrict__ grad_query,
+    float* __restrict__ grad_key, float* __restrict__ grad_value, int64_t symbol_elements,
+    int64_t value_elements) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index < symbol_elements) {
+    if (grad_query != nullptr) {
+      const float den = 1.0f + fabsf(load_as_float<DTYPE>(query, index));
+      grad_query[index] *= 1.0f / (den * den);
+    }
+    if (grad_key != nullptr) {
+      const float den = 1.0f + fabsf(load_as_float<DTYPE>(key, index));
+      grad_key[index] *= 1.0f / (den * den);
+    }
+  }
+  if (index < value_elements && grad_value != nullptr) {
+    const float den = 1.0f + fabsf(load_as_float<DTYPE>(value, index));
+    grad_value[index] *= 1.0f / (den * den);
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_fill_kernel(float* __restrict__ a, int64_t na,
+                                                        float* __restrict__ b, int64_t nb,
+                                                        float* __restrict__ c, int64_t nc) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+       i < na || i < nb || i < nc; i += stride) {
+    if (a != nullptr && i < na) a[i] = 0.0f;
+    if (b != nullptr && i < nb) b[i] = 0.0f;
+    if (c != nullptr && i < nc) c[i] = 0.0f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+size_t align_up(size_t bytes) { return (bytes + 255) & ~static_cast<size_t>(255); }
+
+struct ProblemView {
+  Layout L;
+  int64_t tokens;        // B*T or N
+  int64_t symbol_rows;   // tokens * H
+  int64_t value_rows;    // tokens * Hv
+};
+
+int check_problem(const rosa_problem* p, ProblemView* out) {
+  if (p == nullptr) return fail(1, "problem is NULL");
+  if (p->dtype < ROSA_DTYPE_F32 || p->dtype > ROSA_DTYPE_BF16) return fail(1, "unsupported dtype");
+  if (p->H < 1 || p->Hv < 1 || p->H % p->Hv != 0)
+    return fail(1, "query heads must be a positive multiple of value heads");
+  if (p->D < 1 || p->D > 32) return fail(1, "query/key bit dimension must be in [1, 32]");
+  if (p->Dv < 1) return fail(1, "value dimension must be positive");
+  if (p->W < 1) return fail(1, "max_suffix_length must be >= 1");
+  Layout L;
+  memset(&L, 0, sizeof(L));
+  L.H = p->H; L.D = p->D; L.Hv = p->Hv; L.Dv = p->Dv; L.W = p->W;
+  int64_t tokens;
+  if (p->cu_seqlens != nullptr || p->S > 0) {
+    if (p->cu_seqlens == nullptr || p->S < 1 || p->N < 1)
+      return fail(1, "packed layout needs cu_seqlens, S >= 1 and N >= 1");
+    L.varlen = 1; L.N = p->N; L.S = p->S; L.B = 0; L.T = 0;
+    tokens = p->N;
+    const int64_t slots = static_cast<int64_t>(p->N) / 64 + p->S;
+    if (slots > INT32_MAX) return fail(1, "number of packed sequences is too large");
+    L.slots = static_cast<int>(slots);
+  } else {
+    if (p->B < 1 || p->T < 1) return fail(1, "dense layout needs B >= 1 and T >= 1");
+    tokens = static_cast<int64_t>(p->B) * p->T;
+    if (tokens > INT32_MAX) return fail(1, "B * T must fit in int32");
+    L.varlen = 0; L.B = p->B; L.T = p->T; L.N = static_cast<int>(tokens); L.S = 0;
+    L.slots = p->B * ((p->T + 63) / 64);
+  }
+  if (tokens * p->H > INT32_MAX) return fail(1, "tokens * H must fit in int32");
+  if (static_cast<int64_t>(L.slots) * p->H > INT32_MAX) return fail(1, "too many work units");
+  const int bound = L.varlen ? L.N : L.T;
+  if (L.W > bound) L.W = bound;
+  out->L = L;
+  out->tokens = tokens;
+  out->symbol_rows = tokens * p->H;
+  out->value_rows = tokens * p->Hv;
+  return 0;
+}
+
+// Workspace carving shared by the size queries and the launches.
+struct ForwardWorkspace {
+  size_t header, seq_start, seq_len, block_prefix, source_token, total;
+};
+
+ForwardWorkspace carve_forward(const ProblemView& v) {
+  ForwardWorkspace w;
+  size_t cursor = 0;
+  w.header = cursor; cursor += align_up(256);
+  const size_t s = static_cast<size_t>(v.L.varlen ? v.L.S : 0);
+  w.seq_start = cursor; cursor += align_up(sizeof(int32_t) * s);
+  w.seq_len = cursor; cursor += align_up(sizeof(int32_t) * s);
+  w.block_prefix = cursor; cursor += align_up(sizeof(int32_t) * (s + 1));
+  w.source_token = cursor; cursor += align_up(sizeof(int32_t) * static_cast<size_t>(v.symbol_rows));
+  w.total = cursor;
+  return w;
+}
+
+int value_words(int Dv) { return (Dv + 31) / 32; }
+
+int padded_value_width(int Dv) {
+  if (Dv <= 8) return 8;
+  if (Dv <= 16) return 16;
+  if (Dv <= 32) return 32;
+  return 64;
+}
+
+struct VjpWorkspace {
+  size_t header, seq_start, seq_len, block_prefix, stats, grad_rows, grad_sum, value_bits,
+      block_scratch, total;
+  int resident_blocks;
+  int64_t block_scratch_floats;
+  int ring_rows;
+};
+
+constexpr int kMaxResidentBlocks = 2048;
+
+VjpWorkspace carve_vjp(const ProblemView& v) {
+  VjpWorkspace w;
+  size_t cursor = 0;
+  w.header = cursor; cursor += align_up(256);
+  const size_t s = static_cast<size_t>(v.L.varlen ? v.L.S : 0);
+  w.seq_start = cursor; cursor += align_up(sizeof(int32_t) * s);
+  w.seq_len = cursor; cursor += align_up(sizeof(int32_t) * s);
+  w.block_prefix = cursor; cursor += align_up(sizeof(int32_t) * (s + 1));
+  const size_t rows = static_cast<size_t>(v.symbol_rows);
+  const int dvp = padded_value_width(v.L.Dv);
+  w.stats = cursor; cursor += align_up(sizeof(float) * 4 * rows);
+  w.grad_rows = cursor; cursor += align_up(sizeof(float) * rows * dvp);
+  w.grad_sum = cursor; cursor += align_up(sizeof(float) * rows);
+  w.value_bits = cursor;
+  cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
+  const int longest = v.L.varlen ? v.L.N : v.L.T;
+  w.ring_rows = std::min(v.L.W, longest) + 1;
+  const int max_segments = (longest + kSegment - 1) / kSegment + 1;
+  w.block_scratch_floats =
+      static_cast<int64_t>(w.ring_rows) * kWave + static_cast<int64_t>(max_segments) * 2 * kWave;
+  const int64_t units = static_cast<int64_t>(v.L.slots) * v.L.H;
+  w.resident_blocks = static_cast<int>(std::min<int64_t>(units, kMaxResidentBlocks));
+  // keep the ring pool below 1 GiB by running fewer resident blocks for huge windows
+  const int64_t budget_floats = (int64_t(1) << 30) / 4;
+  while (w.resident_blocks > 64 &&
+         static_cast<int64_t>(w.resident_blocks) * w.block_scratch_floats > budget_floats) {
+    w.resident_blocks /= 2;
+  }
+  w.block_scratch = cursor;
+  cursor += align_up(sizeof(float) * static_cast<size_t>(w.resident_blocks) *
+                     static_cast<size_t>(w.block_scratch_floats));
+  w.total = cursor;
+  return w;
+}
+
+template <typename T>
+T* at(void* base, size_t offset) {
+  return reinterpret_cast<T*>(static_cast<char*>(base) + offset);
+}
+
+unsigned blocks_for(int64_t items, int threads) {
+  return static_cast<unsigned>((items + threads - 1) / threads);
+}
+
+int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, size_t seq_start,
+                             size_t seq_len, size_t block_prefix, size_t header,
+                             hipStream_t stream) {
+  if (!L.varlen) return 0;
+  L.seq_start = at<int32_t>(workspace, seq_start);
+  L.seq_len = at<int32_t>(workspace, seq_len);
+  L.block_prefix = at<int32_t>(workspace, block_prefix);
+  hipLaunchKernelGGL(prepare_sequences_kernel, dim3(1), dim3(256), 0, stream, p->cu_seqlens, L.S,
+                     L.N, at<int32_t>(workspace, seq_start), at<int32_t>(workspace, seq_len),
+                     at<int32_t>(workspace, block_prefix), at<int32_t>(workspace, header));
+  return 0;
+}
+
+template <int DTYPE>
+int run_forward(const rosa_problem* p, const ProblemView& view, const void* query,
+                const void* key, const void* value, void* output, int32_t* packed_query,
+                int32_t* packed_key, int32_t* routes, void* workspace, hipStream_t stream) {
+  Layout L = view.L;
+  const ForwardWorkspace w = carve_forward(view);
+  launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
+                           stream);
+  const int64_t elements = view.symbol_rows * L.D;
+  if (64 % L.D == 0) {
+    hipLaunchKernelGGL(pack_symbols_ballot_kernel<DTYPE>, dim3(blocks_for(elements, 256)),
+                       dim3(256), 0, stream, query, key, packed_query, packed_key, elements, L.D,
+                       L.H, L.T, L.N, L.varlen);
+  } else {
+    hipLaunchKernelGGL(pack_symbols_rows_kernel<DTYPE>, dim3(blocks_for(view.symbol_rows, 256)),
+                       dim3(256), 0, stream, query, key, packed_query, packed_key,
+                       view.symbol_rows, L.D, L.H, L.T, L.N, L.varlen);
+  }
+  const int longest = L.varlen ? L.N : L.T;
+  int shift = 1;
+  while ((1 << shift) <= longest) ++shift;  // routes and runs are <= longest < 2^shift
+  const bool wide = 2 * shift > 32;
+  const unsigned units = static_cast<unsigned>(L.slots) * static_cast<unsigned>(L.H);
+  int32_t* source_token = at<int32_t>(workspace, w.source_token);
+  const uint32_t* pq = reinterpret_cast<const uint32_t*>(packed_query);
+  const uint32_t* pk = reinterpret_cast<const uint32_t*>(packed_key);
+  if (L.varlen) {
+    if (wide) {
+      hipLaunchKernelGGL((hard_route_kernel<true, true>), dim3(units), dim3(kWave), 0, stream, L,
+                         pq, pk, routes, source_token, shift);
+    } else {
+      hipLaunchKernelGGL((hard_route_kernel<true, false>), dim3(units), dim3(kWave), 0, stream, L,
+                         pq, pk, routes, source_token, shift);
+    }
+  } else {
+    if (wide) {
+      hipLaunchKernelGGL((hard_route_kernel<false, true>), dim3(units), dim3(kWave), 0, stream, L,
+                         pq, pk, routes, source_token, shift);
+    } else {
+      hipLaunchKernelGGL((hard_route_kernel<false, false>), dim3(units), dim3(kWave), 0, stream,
+                         L, pq, pk, routes, source_token, shift);
+    }
+  }
+  const int64_t out_elements = view.symbol_rows * L.Dv;
+  hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)), dim3(256),
+                     0, stream, source_token, value, output, out_elements, L.H, L.Hv, L.Dv, L.T,
+                     L.N, L.varlen);
+  const hipError_t status = hipGetLastError();
+  if (status != hipSuccess) return fail_hip(status, "hard forward launch");
+  return 0;
+}
+
+template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
+int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
+                      hipStream_t stream) {
+  const unsigned units = static_cast<unsigned>(P.total_units);
+  if (!analytic) {
+    hipLaunchKernelGGL((vjp_row_max_kernel<NVW, VARLEN>), dim3(units), dim3(kWave), 0, stream, P);
+  }
+  hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
+                     0, stream, P);
+  const size_t lds_floats = 2 * kSegChunks * kWave + 2 * kChunk * kWave + kChunk * DVP +
+                            (kChunk + kWave) + kChunk + kColumnRing * DVP +
+                            kColumnRing * static_cast<size_t>(P.L.D);
+  const hipError_t attribute = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
+  if (attribute != hipSuccess) return fail_hip(attribute, "gradient kernel LDS size");
+  hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
+                     dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave),
+                     lds_floats * sizeof(float), stream, P);
+  return 0;
+}
+
+template <int NVW, int DVP>
+int dispatch_vjp(const VjpParams& P, const VjpWorkspace& w, bool analytic, bool dropout,
+                 hipStream_t stream) {
+  if (P.L.varlen) {
+    return dropout ? launch_vjp_passes<NVW, DVP, true, true>(P, w, analytic, stream)
+                   : launch_vjp_passes<NVW, DVP, true, false>(P, w, analytic, stream);
+  }
+  return dropout ? launch_vjp_passes<NVW, DVP, false, true>(P, w, analytic, stream)
+                 : launch_vjp_passes<NVW, DVP, false, false>(P, w, analytic, stream);
+}
+
+// the analytic exponent reference is safe while it stays within 2^80 of the null weight
+bool analytic_reference_is_safe(const Layout& L, float scale) {
+  const int longest = L.varlen ? L.N : L.T;
+  const float window = static_cast<float>(std::min(L.W, longest));
+  const float bound = scale * kSqrtScale * (std::sqrt(1.0f + window) - 1.0f);
+  return (bound - kNullScore * scale) * kLog2e < 80.0f;
+}
+
+template <int DTYPE>
+int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, const void* key,
+            const void* value, const void* grad_output, const int32_t* packed_query,
+            const int32_t* packed_key, const int64_t* dropout_seed, float scale, float dropout_p,
+            float inverse_keep, float mismatch_scale, int gradient_mask, float* grad_query,
+            float* grad_key, float* grad_value, void* workspace, hipStream_t stream) {
+  Layout L = view.L;
+  const VjpWorkspace w = carve_vjp(view);
+  launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
+                           stream);
+  const int dvp = padded_value_width(L.Dv);
+  const int nvw = value_words(L.Dv);
+  const int64_t symbol_elements = view.symbol_rows * L.D;
+  const int64_t value_elements = view.value_rows * L.Dv;
+  {
+    const int64_t largest = std::max(symbol_elements, value_elements);
+    const unsigned fill_blocks = static_cast<unsigned>(std::min<int64_t>(blocks_for(largest, 256), 8192));
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(fill_blocks), dim3(256), 0, stream, grad_query,
+                       grad_query ? symbol_elements : 0, grad_key, grad_key ? symbol_elements : 0,
+                       grad_value, grad_value ? value_elements : 0);
+  }
+
+  float4* stats = at<float4>(workspace, w.stats);
+  float* grad_rows = at<float>(workspace, w.grad_rows);
+  float* grad_sum = at<float>(workspace, w.grad_sum);
+  uint32_t* value_bits = at<uint32_t>(workspace, w.value_bits);
+  int32_t* counter = at<int32_t>(workspace, w.header) + 1;
+  const bool analytic = analytic_reference_is_safe(L, scale);
+
+  hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>, dim3(blocks_for(view.symbol_rows, 256)),
+                     dim3(256), 0, stream, grad_output, grad_rows, grad_sum, view.symbol_rows,
+                     L.H, L.Dv, dvp, L.T, L.N, L.varlen);
+  hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
+                     dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
+                     L.T, L.N, L.varlen);
+  if (L.varlen) {
+    hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
+                       dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
+  } else {
+    hipLaunchKernelGGL(init_row_stats_kernel<false>, dim3(blocks_for(view.symbol_rows, 256)),
+                       dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
+  }
+
+  VjpParams P;
+  memset(&P, 0, sizeof(P));
+  P.L = L;
+  P.packed_query = reinterpret_cast<const uint32_t*>(packed_query);
+  P.packed_key = reinterpret_cast<const uint32_t*>(packed_key);
+  P.value_bits = value_bits;
+  P.grad_rows = grad_rows;
+  P.grad_row_sum = grad_sum;
+  P.stats = stats;
+  P.dropout_seed = dropout_seed;
+  P.scale = scale;
+  P.dropout_p = dropout_p;
+  P.inverse_keep = inverse_keep;
+  P.mismatch_scale = mismatch_scale;
+  P.gate_log2 = mismatch_scale * kLog2e / static_cast<float>(L.D);
+  P.logit_gain = scale * kSqrtScale * kLog2e;
+  P.null_logit = kNullScore * scale;
+  {
+    // window products this far below one cannot move a float32 gradient:
+    // 2^-34 / (W^2 * longest)
+    const int longest = L.varlen ? L.N : L.T;
+    const float exponent =
+        -34.0f - 2.0f * std::log2(static_cast<float>(L.W)) - std::log2(static_cast<float>(longest));
+    P.tail_threshold = std::exp2(std::max(exponent, -120.0f));
+  }
+  P.gradient_mask = gradient_mask;
+  P.dvp = dvp;
+  P.grad_query = grad_query;
+  P.grad_key = grad_key;
+  P.grad_value = grad_value;
+  P.work_counter = counter;
+  P.block_scratch = at<float>(workspace, w.block_scratch);
+  P.block_scratch_floats = w.block_scratch_floats;
+  P.ring_rows = w.ring_rows;
+  P.total_units = L.slots * L.H;
+  const bool dropout = dropout_p > 0.0f;
+
+  int status = 0;
+  if (nvw == 1) {
+    if (dvp == 8) status = dispatch_vjp<1, 8>(P, w, analytic, dropout, stream);
+    else if (dvp == 16) status = dispatch_vjp<1, 16>(P, w, analytic, dropout, stream);
+    else status = dispatch_vjp<1, 32>(P, w, analytic, dropout, stream);
+  } else {
+    status = dispatch_vjp<2, 64>(P, w, analytic, dropout, stream);
+  }
+  if (status != 0) return status;
+  const int64_t finalize_items = std::max(symbol_elements, value_elements);
+  hipLaunchKernelGGL(finalize_gradients_kernel<DTYPE>, dim3(blocks_for(finalize_items, 256)),
+                     dim3(256), 0, stream, query, key, value, grad_query, grad_key, grad_value,
+                     symbol_elements, value_elements);
+  const hipError_t launch = hipGetLastError();
+  if (launch != hipSuccess) return fail_hip(launch, "surrogate vjp launch");
+  return 0;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+
+extern "C" {
+
+int rosa_hip_version(void) { return 100; }
+
+const char* rosa_hip_target(void) { return "rocm-gfx950"; }
+
+const char* rosa_hip_last_error(void) { return g_error; }
+
+size_t rosa_hip_forward_workspace_bytes(const rosa_problem* problem) {
+  ProblemView view;
+  if (check_problem(problem, &view) != 0) return 0;
+  return carve_forward(view).total;
+}
+
+size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_mask, float scale,
+                                    int dropout) {
+  (void)gradient_mask;
+  (void)scale;
+  (void)dropout;
+  ProblemView view;
+  if (check_problem(problem, &view) != 0) return 0;
+  return carve_vjp(view).total;
+}
+
+int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const void* key,
+                          const void* value, void* output, int32_t* packed_query,
+                          int32_t* packed_key, int32_t* routes, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  ProblemView view;
+  const int bad = check_problem(problem, &view);
+  if (bad != 0) return bad;
+  if (!query || !key || !value || !output || !packed_query || !packed_key || !workspace)
+    return fail(2, "hard_forward: NULL tensor or workspace pointer");
+  if (workspace_bytes < carve_forward(view).total) return fail(3, "hard_forward: workspace too small");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (problem->dtype) {
+    case ROSA_DTYPE_F32:
+      return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
+                                         packed_key, routes, workspace, s);
+    case ROSA_DTYPE_F16:
+      return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
+                                         packed_key, routes, workspace, s);
+    default:
+      return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
+                                          packed_key, routes, workspace, s);
+  }
+}
+
+int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const void* key,
+                           const void* value, const void* grad_output,
+                           const int32_t* packed_query, const int32_t* packed_key,
+                           const int64_t* dropout_seed, float scale, float dropout_p,
+                           float inverse_keep, float mismatch_scale, int gradient_mask,
+                           float* grad_query, float* grad_key, float* grad_value, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  ProblemView view;
+  const int bad = check_problem(problem, &view);
+  if (bad != 0) return bad;
+  if (gradient_mask < 1 || gradient_mask > 7)
+    return fail(1, "gradient_mask must be an integer bit mask in [1, 7]");
+  if (!query || !key || !value || !grad_output || !packed_query || !packed_key || !workspace)
+    return fail(2, "surrogate_vjp: NULL tensor or workspace pointer");
+  if (((gradient_mask & ROSA_GRAD_QUERY) && !grad_query) ||
+      ((gradient_mask & ROSA_GRAD_KEY) && !grad_key) ||
+      ((gradient_mask & ROSA_GRAD_VALUE) && !grad_value))
+    return fail(2, "surrogate_vjp: a requested gradient has a NULL pointer");
+  if (!(scale > 0.0f) || !(mismatch_scale > 0.0f) || !(dropout_p >= 0.0f) || !(dropout_p < 1.0f))
+    return fail(1, "surrogate_vjp: scale, mismatch_scale > 0 and 0 <= dropout_p < 1 required");
+  if (dropout_p > 0.0f && dropout_seed == nullptr)
+    return fail(2, "surrogate_vjp: dropout_seed must be given exactly when dropout_p > 0");
+  if (problem->Dv > 64)
+    return fail(4, "surrogate_vjp: value dimension above 64 is not supported by this build");
+  if (workspace_bytes < carve_vjp(view).total) return fail(3, "surrogate_vjp: workspace too small");
+  if (!(gradient_mask & ROSA_GRAD_QUERY)) grad_query = nullptr;
+  if (!(gradient_mask & ROSA_GRAD_KEY)) grad_key = nullptr;
+  if (!(gradient_mask & ROSA_GRAD_VALUE)) grad_value = nullptr;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (problem->dtype) {
+    case ROSA_DTYPE_F32:
+      return run_vjp<ROSA_DTYPE_F32>(problem, view, query, key, value, grad_output, packed_query,
+                                     packed_key, dropout_seed, scale, dropout_p, inverse_keep,
+                                     mismatch_scale, gradient_mask, grad_query, grad_key,
+                                     grad_value, workspace, s);
+    case ROSA_DTYPE_F16:
+      return run_vjp<ROSA_DTYPE_F16>(problem, view, query, key, value, grad_output, packed_query,
+                                     packed_key, dropout_seed, scale, dropout_p, inverse_keep,
+                                     mismatch_scale, gradient_mask, grad_query, grad_key,
+                                     grad_value, workspace, s);
+    default:
+      return run_vjp<ROSA_DTYPE_BF16>(problem, view, query, key, value, grad_output, packed_query,
+                                      packed_key, dropout_seed, scale, dropout_p, inverse_keep,
+                                      mismatch_scale, gradient_mask, grad_query, grad_key,
+                                      grad_value, workspace, s);
+  }
+}
+
+int rosa_hip_read_offset_error(const void* workspace, void* stream) {
+  int32_t flag = 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (hipMemcpyAsync(&flag, workspace, sizeof(flag), hipMemcpyDeviceToHost, s) != hipSuccess)
+    return -1;
+  if (hipStreamSynchronize(s) != hipSuccess) return -1;
+  return flag;
+}
+
+}  // extern "C"
