@@ -1,0 +1,306 @@
+"""Throughput of the rosa_soft training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload metric]
+
+A step is one forward + backward of the public operator over one batch of
+synthetic inputs already resident in HBM: ``rosa_soft`` (or
+``rosa_soft_varlen``), loss ``output.float().square().mean()``, ``backward()``.
+The default workload is the one the headline metric is quoted on:
+B=2, T=4096, H=64, D=8 float32 with the remaining controls of the reference's
+README configuration (value_heads=16, value_dim=8, max_suffix_length=128,
+dropout_p=0.1, mismatch_scale=3.0).  One JSON line is printed.
+
+Besides whole-step tokens/s the line carries
+
+* ``fwd_tokens_per_s``: forward-only (no-grad) tokens/s;
+* ``roofline``: the dominant kernel (``vjp_gradients``) priced by its
+  algorithmic MFMA-equivalent flops ``2 * pairs * (3 D + 2 Dv)`` over its
+  average launch time, measured with HIP events recorded by the library on the
+  stream the kernel runs on, against the MI355X fp32 matrix peak;
+* ``kernels``: average milliseconds and achieved HBM GB/s (algorithmic bytes)
+  of every stage;
+* ``cpu_baseline``: the float64 CPU oracle timed on a bounded slice of the same
+  workload on this box's host cores, extrapolated to tokens/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+
+# name: dense  -> dict(B, T, H, D, Hv, Dv, W, p, ms, dtype, pattern)
+#       packed -> dict(lengths, H, D, Hv, Dv, W, p, ms, dtype)
+WORKLOADS = {
+    "metric": dict(B=2, T=4096, H=64, D=8, Hv=16, Dv=8, W=128, p=0.1, ms=3.0, dtype="float32"),
+    "config1": dict(B=1, T=256, H=4, D=4, Hv=4, Dv=8, W=16, p=0.0, ms=3.0, dtype="float32"),
+    "config2": dict(B=2, T=1024, H=64, D=8, Hv=16, Dv=8, W=128, p=0.1, ms=3.0, dtype="float32"),
+    "config3": dict(B=4, T=4096, H=32, D=16, Hv=32, Dv=64, W=32, p=0.0, ms=3.0, dtype="bfloat16"),
+    "config4": dict(B=1, T=8192, H=16, D=2, Hv=16, Dv=32, W=256, p=0.0, ms=3.0, dtype="float16",
+                    pattern="motif"),
+    "config5": dict(lengths=[1024, 7168, 2048, 4096, 512, 8192, 3072, 6656], H=64, D=32, Hv=8,
+                    Dv=32, W=64, p=0.1, ms=9.0, dtype="bfloat16"),
+}
+
+
+def make_workload(name: str, device="cpu"):
+    """Seeded synthetic inputs of a named configuration, built in their final dtype.
+
+    Returns ``(config, query, key, value, cu_seqlens_or_None)``.  A private
+    generator is used so that the result does not depend on global RNG state.
+    """
+
+    config = dict(WORKLOADS[name])
+    dtype = getattr(torch, config["dtype"])
+    generator = torch.Generator().manual_seed(1234 + sorted(WORKLOADS).index(name))
+    randn = lambda *shape: torch.randn(*shape, generator=generator)
+    if "lengths" in config:
+        total = sum(config["lengths"])
+        query = randn(total, config["H"], config["D"]).to(dtype)
+        key = randn(total, config["H"], config["D"]).to(dtype)
+        value = randn(total, config["Hv"], config["Dv"]).to(dtype)
+        offsets = [0]
+        for length in config["lengths"]:
+            offsets.append(offsets[-1] + length)
+        cu_seqlens = torch.tensor(offsets, dtype=torch.int32)
+        return config, query.to(device), key.to(device), value.to(device), cu_seqlens.to(device)
+    B, T, H, D = config["B"], config["T"], config["H"], config["D"]
+    if config.get("pattern") == "motif":
+        # per head a random 64-step motif tiled over T, 10 % of positions
+        # sign-flipped; query = key + N(0, 0.1), rounded to the final dtype
+        motif = randn(B, 64, H, D)
+        key = motif.repeat(1, (T + 63) // 64, 1, 1)[:, :T].clone()
+        flip = torch.rand(B, T, H, 1, generator=generator) < 0.10
+        key = torch.where(flip, -key, key).to(dtype)
+        query = (key.float() + 0.1 * randn(B, T, H, D)).to(dtype)
+    else:
+        query = randn(B, T, H, D).to(dtype)
+        key = randn(B, T, H, D).to(dtype)
+    value = randn(B, T, config["Hv"], config["Dv"]).to(dtype)
+    return config, query.to(device), key.to(device), value.to(device), None
+
+
+def pair_count(config) -> int:
+    if "lengths" in config:
+        return config["H"] * sum(n * (n - 1) // 2 for n in config["lengths"])
+    return config["B"] * config["H"] * config["T"] * (config["T"] - 1) // 2
+
+
+def token_count(config) -> int:
+    return sum(config["lengths"]) if "lengths" in config else config["B"] * config["T"]
+
+
+def algorithmic_bytes(config) -> dict:
+    """Bytes each stage must move at least once (inputs read, outputs written)."""
+
+    tokens = token_count(config)
+    item = 4 if config["dtype"] == "float32" else 2
+    symbols = tokens * config["H"] * config["D"]
+    values = tokens * config["Hv"] * config["Dv"]
+    outputs = tokens * config["H"] * config["Dv"]
+    words = tokens * config["H"] * 4
+    forward = 2 * symbols * item + 2 * words + values * item + outputs * item
+    backward = (2 * symbols + values + outputs) * item + 2 * words + (2 * symbols + values) * 4
+    return dict(forward=forward, backward=backward)
+
+
+def run_step(rosa, config, leaves, cu_seqlens):
+    controls = dict(
+        max_suffix_length=config["W"], scale=1.0, dropout_p=config["p"],
+        mismatch_scale=config["ms"],
+    )
+    for leaf in leaves:
+        leaf.grad = None
+    if cu_seqlens is None:
+        output = rosa.rosa_soft(*leaves, **controls)
+    else:
+        output = rosa.rosa_soft_varlen(*leaves, cu_seqlens, **controls)
+    loss = output.float().square().mean()
+    loss.backward()
+    return loss
+
+
+def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
+    """Time the CPU oracle (a port, float64, OpenMP) on a slice of the workload.
+
+    The slice is one batch element and one value-head group over a prefix of
+    the sequence chosen so that the run stays near the budget; its time is
+    scaled by the pair count to the whole workload.
+    """
+
+    from oracle import c_oracle
+
+    config, query, key, value, cu_seqlens = make_workload(name)
+    if cu_seqlens is not None:
+        start, end = int(cu_seqlens[0]), int(cu_seqlens[1])
+        query, key, value = (t[start:end].unsqueeze(0) for t in (query, key, value))
+    group = config["H"] // config["Hv"]
+    query, key, value = query[:1, :, :group], key[:1, :, :group], value[:1, :, :1]
+    threads = c_oracle.num_threads()
+    rows = min(query.size(1), 512)
+    grad_output = None
+    elapsed = 0.0
+    while True:
+        q, k, v = (t[:, :rows].contiguous() for t in (query, key, value))
+        grad_output = torch.ones(1, rows, group, config["Dv"]) / (rows * group * config["Dv"])
+        begin = time.perf_counter()
+        out, _, _ = c_oracle.hard_forward(q, k, v, config["W"])
+        forward_seconds = time.perf_counter() - begin
+        c_oracle.surrogate_vjp(
+            q, k, v, (2.0 * out.float() * grad_output), max_suffix_length=config["W"],
+            dropout_p=config["p"], mismatch_scale=config["ms"], seed=12345 if config["p"] > 0 else None,
+        )
+        elapsed = time.perf_counter() - begin
+        if rows >= query.size(1) or elapsed * 4.0 > budget_seconds:
+            break
+        rows = min(query.size(1), rows * 2)
+    slice_pairs = group * rows * (rows - 1) // 2
+    seconds_full = elapsed * pair_count(config) / max(slice_pairs, 1)
+    return dict(
+        value=token_count(config) / seconds_full,
+        unit="tokens/s",
+        cores=threads,
+        kind="port",
+        sample=(
+            f"float64 C oracle, fwd+bwd, 1 batch x {group} heads x first {rows} rows "
+            f"({slice_pairs} pairs, {elapsed:.2f} s, forward {forward_seconds:.3f} s), "
+            "scaled by pair count"
+        ),
+    )
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=10)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--workload", default="metric", choices=sorted(WORKLOADS))
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(
+            "bench.py measures one GPU: this operator shards over (batch, value-head group) "
+            "without any exchange and no multi-GPU path is built; run with --gpus 1",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+
+    import rosa_soft_amd
+    from rosa_soft_amd import cabi
+
+    assert rosa_soft_amd.BUILD_CAPABILITIES.variant == "rocm", "HIP extension is not built"
+    device = torch.device("cuda:0")
+    config, query, key, value, cu_seqlens = make_workload(args.workload, device)
+    leaves = [t.requires_grad_() for t in (query, key, value)]
+    tokens = token_count(config)
+
+    cabi.stage_timing(True)
+    for _ in range(args.warmup):
+        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
+    torch.cuda.synchronize()
+    stage_totals = {}
+    begin = time.perf_counter()
+    for _ in range(args.steps):
+        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
+        # the events of this step were recorded on the stream; reading them
+        # waits for the step, which the closing synchronize would do anyway
+        for stage, ms in cabi.stage_times().items():
+            stage_totals[stage] = stage_totals.get(stage, 0.0) + ms
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    cabi.stage_timing(False)
+    ms_per_step = 1e3 * elapsed / args.steps
+
+    # forward only
+    with torch.no_grad():
+        for _ in range(2):
+            run_forward = (
+                rosa_soft_amd.rosa_soft(query, key, value, max_suffix_length=config["W"])
+                if cu_seqlens is None
+                else rosa_soft_amd.rosa_soft_varlen(query, key, value, cu_seqlens,
+                                                    max_suffix_length=config["W"])
+            )
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(args.steps):
+            if cu_seqlens is None:
+                rosa_soft_amd.rosa_soft(query, key, value, max_suffix_length=config["W"])
+            else:
+                rosa_soft_amd.rosa_soft_varlen(query, key, value, cu_seqlens,
+                                               max_suffix_length=config["W"])
+        torch.cuda.synchronize()
+        forward_ms = 1e3 * (time.perf_counter() - begin) / args.steps
+
+    pairs = pair_count(config)
+    stage_ms = {stage: total / args.steps for stage, total in stage_totals.items()}
+    bytes_needed = algorithmic_bytes(config)
+    flops = 2.0 * pairs * (3 * config["D"] + 2 * config["Dv"])
+    gradient_ms = stage_ms.get("vjp_gradients", float("nan"))
+    achieved_tflops = flops / (gradient_ms * 1e-3) / 1e12
+    backward_ms = sum(ms for stage, ms in stage_ms.items() if stage.startswith("vjp_"))
+    kernels = {
+        stage: dict(ms=round(ms, 4)) for stage, ms in stage_ms.items()
+    }
+    if "hard_forward" in stage_ms:
+        kernels["hard_forward"]["hbm_gbs"] = round(
+            bytes_needed["forward"] / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2
+        )
+        kernels["hard_forward"]["gpairs_per_s"] = round(pairs / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2)
+    if backward_ms > 0:
+        kernels["vjp_total"] = dict(
+            ms=round(backward_ms, 4),
+            hbm_gbs=round(bytes_needed["backward"] / (backward_ms * 1e-3) / 1e9, 2),
+            gpairs_per_s=round(pairs / (backward_ms * 1e-3) / 1e9, 2),
+        )
+
+    record = {
+        "metric": "fwd+bwd tokens/sec",
+        "value": tokens / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if config["dtype"] == "float32" else config["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: " + ", ".join(f"{k}={v}" for k, v in config.items()),
+            "loss": "output.float().square().mean()",
+            "tokens_per_step": tokens,
+            "pairs_per_step": pairs,
+        },
+        "fwd_tokens_per_s": tokens / (forward_ms * 1e-3),
+        "fwd_ms": forward_ms,
+        "roofline": {
+            "kernel": "vjp_gradients_kernel",
+            "bound": "mfma",
+            "achieved": achieved_tflops,
+            "peak": FP32_MATRIX_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tflops / FP32_MATRIX_PEAK_TFLOPS,
+            "traffic": None,
+            "note": "algorithmic flops 2*pairs*(3D+2Dv) over the kernel's mean launch time",
+        },
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        record["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(record))
+
+
+if __name__ == "__main__":
+    main()

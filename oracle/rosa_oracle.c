@@ -217,23 +217,30 @@ int rosa_oracle_surrogate_vjp(const float* q, const float* k, const float* v,
   const double null_logit = ROSA_NULL_SCORE * scale;
   int failed = 0;
 
+  const size_t row_q = (size_t)T * D, row_v = (size_t)T * Dv;
+  for (int bh = 0; bh < B * H && !failed; ++bh) {
+    const int b = bh / H, h = bh % H;
+    const int hv = h / group;
+    const uint32_t* qw = (const uint32_t*)pq + (int64_t)bh * T;
+    const uint32_t* kw = (const uint32_t*)pk + (int64_t)bh * T;
 #pragma omp parallel
-  {
-    double* scores = (double*)malloc(sizeof(double) * (size_t)(T + 1));
-    double* utils = (double*)malloc(sizeof(double) * (size_t)(T + 1));
-    double* drops = (double*)malloc(sizeof(double) * (size_t)(T + 1));
-    if (!scores || !utils || !drops) {
+    {
+      /* per-thread scratch rows and private gradient slabs for this (b, h) */
+      double* scores = (double*)malloc(sizeof(double) * (size_t)(T + 1));
+      double* utils = (double*)malloc(sizeof(double) * (size_t)(T + 1));
+      double* drops = (double*)malloc(sizeof(double) * (size_t)(T + 1));
+      double* local_q = grad_q ? (double*)calloc(row_q, sizeof(double)) : NULL;
+      double* local_k = grad_k ? (double*)calloc(row_q, sizeof(double)) : NULL;
+      double* local_v = grad_v ? (double*)calloc(row_v, sizeof(double)) : NULL;
+      const int ok = scores && utils && drops && (!grad_q || local_q) &&
+                     (!grad_k || local_k) && (!grad_v || local_v);
+      if (!ok) {
 #pragma omp atomic write
-      failed = 1;
-    }
-#pragma omp for collapse(2) schedule(dynamic, 4)
-    for (int bh = 0; bh < B * H; ++bh) {
+        failed = 1;
+      }
+#pragma omp for schedule(dynamic, 8)
       for (int t = 1; t < T; ++t) {
-        if (failed) continue;
-        const int b = bh / H, h = bh % H;
-        const int hv = h / group;
-        const uint32_t* qw = (const uint32_t*)pq + (int64_t)bh * T;
-        const uint32_t* kw = (const uint32_t*)pk + (int64_t)bh * T;
+        if (!ok) continue;
         const float* go_row = go + (((int64_t)b * T + t) * H + h) * Dv;
         const double log_count = log((double)t);
         /* pass 1: scores, utilities, dropout, softmax statistics */
@@ -269,14 +276,11 @@ int rosa_oracle_surrogate_vjp(const float* q, const float* k, const float* v,
           const double logit = scale * ROSA_SQRT_SCALE * (root - 1.0) - log_count;
           const double prob = exp(logit - row_max) / denom;
           const double dropped = prob * drops[a];
-          if (grad_v && dropped != 0.0) {
-            double* gv = grad_v + (((int64_t)b * T + a) * Hv + hv) * Dv;
-            for (int d = 0; d < Dv; ++d) {
-#pragma omp atomic
-              gv[d] += dropped * (double)go_row[d];
-            }
+          if (local_v && dropped != 0.0) {
+            double* gv = local_v + (size_t)a * Dv;
+            for (int d = 0; d < Dv; ++d) gv[d] += dropped * (double)go_row[d];
           }
-          if (!grad_q && !grad_k) continue;
+          if (!local_q && !local_k) continue;
           const double adjoint = scale * prob * (drops[a] * utils[a] - expected) *
                                  (0.5 * ROSA_SQRT_SCALE / root);
           if (adjoint == 0.0) continue;
@@ -288,21 +292,11 @@ int rosa_oracle_surrogate_vjp(const float* q, const float* k, const float* v,
             product *= gate_of(qword, kword, gate_table);
             const double weight = symbol_scale * adjoint * (tail > 0.0 ? tail : 0.0);
             if (weight != 0.0) {
-              double* gq = grad_q
-                  ? grad_q + (((int64_t)b * T + (t - j)) * H + h) * D : NULL;
-              double* gk = grad_k
-                  ? grad_k + (((int64_t)b * T + (a - 1 - j)) * H + h) * D : NULL;
+              double* gq = local_q ? local_q + (size_t)(t - j) * D : NULL;
+              double* gk = local_k ? local_k + (size_t)(a - 1 - j) * D : NULL;
               for (int bit = 0; bit < D; ++bit) {
-                const double qs = ((qword >> bit) & 1u) ? 1.0 : -1.0;
-                const double ks = ((kword >> bit) & 1u) ? 1.0 : -1.0;
-                if (gq) {
-#pragma omp atomic
-                  gq[bit] += weight * ks;
-                }
-                if (gk) {
-#pragma omp atomic
-                  gk[bit] += weight * qs;
-                }
+                if (gq) gq[bit] += ((kword >> bit) & 1u) ? weight : -weight;
+                if (gk) gk[bit] += ((qword >> bit) & 1u) ? weight : -weight;
               }
             }
             tail -= product;
@@ -310,10 +304,34 @@ int rosa_oracle_surrogate_vjp(const float* q, const float* k, const float* v,
           }
         }
       }
+      /* fold the private slabs into the outputs (query/key are owned by this
+       * (b, h); value rows are shared by the heads of a group, visited serially) */
+#pragma omp critical
+      {
+        if (ok) {
+          for (int t = 0; t < T; ++t) {
+            if (local_q) {
+              double* dst = grad_q + (((int64_t)b * T + t) * H + h) * D;
+              for (int bit = 0; bit < D; ++bit) dst[bit] += local_q[(size_t)t * D + bit];
+            }
+            if (local_k) {
+              double* dst = grad_k + (((int64_t)b * T + t) * H + h) * D;
+              for (int bit = 0; bit < D; ++bit) dst[bit] += local_k[(size_t)t * D + bit];
+            }
+            if (local_v) {
+              double* dst = grad_v + (((int64_t)b * T + t) * Hv + hv) * Dv;
+              for (int d = 0; d < Dv; ++d) dst[d] += local_v[(size_t)t * Dv + d];
+            }
+          }
+        }
+      }
+      free(scores);
+      free(utils);
+      free(drops);
+      free(local_q);
+      free(local_k);
+      free(local_v);
     }
-    free(scores);
-    free(utils);
-    free(drops);
   }
   free(pq);
   free(pk);

@@ -30,6 +30,10 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_hard_forward",
     "rosa_hip_surrogate_vjp",
     "rosa_hip_read_offset_error",
+    "rosa_hip_stage_timing",
+    "rosa_hip_stage_count",
+    "rosa_hip_stage_name",
+    "rosa_hip_stage_times",
 )
 
 _DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
@@ -89,6 +93,13 @@ def load() -> ctypes.CDLL:
     ]
     library.rosa_hip_read_offset_error.restype = ctypes.c_int
     library.rosa_hip_read_offset_error.argtypes = [vp, vp]
+    library.rosa_hip_stage_timing.restype = ctypes.c_int
+    library.rosa_hip_stage_timing.argtypes = [ctypes.c_int]
+    library.rosa_hip_stage_count.restype = ctypes.c_int
+    library.rosa_hip_stage_name.restype = ctypes.c_char_p
+    library.rosa_hip_stage_name.argtypes = [ctypes.c_int]
+    library.rosa_hip_stage_times.restype = ctypes.c_int
+    library.rosa_hip_stage_times.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_int]
     _library = library
     return library
 
@@ -222,3 +233,23 @@ def vjp_workspace_bytes(query: Tensor, value: Tensor, max_suffix_length: int,
                         cu_seqlens: Optional[Tensor] = None) -> int:
     problem = make_problem(query, value, max_suffix_length, cu_seqlens)
     return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0))
+
+
+def stage_timing(enable: bool) -> None:
+    """Switch per-stage HIP event timing of the library on or off."""
+
+    _check(load().rosa_hip_stage_timing(1 if enable else 0), "rosa_hip_stage_timing")
+
+
+def stage_times() -> dict:
+    """Elapsed milliseconds per stage of the last call (waits for its events)."""
+
+    library = load()
+    count = library.rosa_hip_stage_count()
+    buffer = (ctypes.c_float * count)()
+    _check(library.rosa_hip_stage_times(buffer, count), "rosa_hip_stage_times")
+    return {
+        library.rosa_hip_stage_name(i).decode(): float(buffer[i])
+        for i in range(count)
+        if buffer[i] >= 0.0
+    }

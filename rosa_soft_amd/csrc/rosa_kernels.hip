@@ -54,6 +54,33 @@ int fail_hip(hipError_t status, const char* what) {
   return 100 + static_cast<int>(status);
 }
 
+// Optional stage timing: when enabled, every launch sequence brackets its
+// stages with HIP events recorded on the caller's stream.  Nothing is read
+// back until rosa_hip_stage_times() is called.
+enum Stage { kStageForward = 0, kStagePrepare, kStageRowMax, kStageRowStats, kStageGradients,
+             kStageFinalize, kStageCount };
+
+struct StageTimer {
+  bool enabled = false;
+  bool created = false;
+  hipEvent_t begin[kStageCount];
+  hipEvent_t end[kStageCount];
+  bool used[kStageCount];
+};
+
+StageTimer g_timer;
+
+void stage_begin(Stage stage, hipStream_t stream) {
+  if (!g_timer.enabled) return;
+  g_timer.used[stage] = true;
+  (void)hipEventRecord(g_timer.begin[stage], stream);
+}
+
+void stage_end(Stage stage, hipStream_t stream) {
+  if (!g_timer.enabled) return;
+  (void)hipEventRecord(g_timer.end[stage], stream);
+}
+
 // ---------------------------------------------------------------------------
 // small device helpers
 // ---------------------------------------------------------------------------
@@ -1260,6 +1287,7 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
                 int32_t* packed_key, int32_t* routes, void* workspace, hipStream_t stream) {
   Layout L = view.L;
   const ForwardWorkspace w = carve_forward(view);
+  stage_begin(kStageForward, stream);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
                            stream);
   const int64_t elements = view.symbol_rows * L.D;
@@ -1301,6 +1329,7 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)), dim3(256),
                      0, stream, source_token, value, output, out_elements, L.H, L.Hv, L.Dv, L.T,
                      L.N, L.varlen);
+  stage_end(kStageForward, stream);
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "hard forward launch");
   return 0;
@@ -1311,10 +1340,14 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
                       hipStream_t stream) {
   const unsigned units = static_cast<unsigned>(P.total_units);
   if (!analytic) {
+    stage_begin(kStageRowMax, stream);
     hipLaunchKernelGGL((vjp_row_max_kernel<NVW, VARLEN>), dim3(units), dim3(kWave), 0, stream, P);
+    stage_end(kStageRowMax, stream);
   }
+  stage_begin(kStageRowStats, stream);
   hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
                      0, stream, P);
+  stage_end(kStageRowStats, stream);
   const size_t lds_floats = 2 * kSegChunks * kWave + 2 * kChunk * kWave + kChunk * DVP +
                             (kChunk + kWave) + kChunk + kColumnRing * DVP +
                             kColumnRing * static_cast<size_t>(P.L.D);
@@ -1322,9 +1355,11 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
   if (attribute != hipSuccess) return fail_hip(attribute, "gradient kernel LDS size");
+  stage_begin(kStageGradients, stream);
   hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
                      dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave),
                      lds_floats * sizeof(float), stream, P);
+  stage_end(kStageGradients, stream);
   return 0;
 }
 
@@ -1361,6 +1396,7 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   const int nvw = value_words(L.Dv);
   const int64_t symbol_elements = view.symbol_rows * L.D;
   const int64_t value_elements = view.value_rows * L.Dv;
+  stage_begin(kStagePrepare, stream);
   {
     const int64_t largest = std::max(symbol_elements, value_elements);
     const unsigned fill_blocks = static_cast<unsigned>(std::min<int64_t>(blocks_for(largest, 256), 8192));
@@ -1389,6 +1425,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     hipLaunchKernelGGL(init_row_stats_kernel<false>, dim3(blocks_for(view.symbol_rows, 256)),
                        dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
   }
+
+  stage_end(kStagePrepare, stream);
 
   VjpParams P;
   memset(&P, 0, sizeof(P));
@@ -1437,9 +1475,11 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   }
   if (status != 0) return status;
   const int64_t finalize_items = std::max(symbol_elements, value_elements);
+  stage_begin(kStageFinalize, stream);
   hipLaunchKernelGGL(finalize_gradients_kernel<DTYPE>, dim3(blocks_for(finalize_items, 256)),
                      dim3(256), 0, stream, query, key, value, grad_query, grad_key, grad_value,
                      symbol_elements, value_elements);
+  stage_end(kStageFinalize, stream);
   const hipError_t launch = hipGetLastError();
   if (launch != hipSuccess) return fail_hip(launch, "surrogate vjp launch");
   return 0;
@@ -1545,6 +1585,41 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const
                                       mismatch_scale, gradient_mask, grad_query, grad_key,
                                       grad_value, workspace, s);
   }
+}
+
+int rosa_hip_stage_timing(int enable) {
+  if (enable && !g_timer.created) {
+    for (int i = 0; i < kStageCount; ++i) {
+      if (hipEventCreate(&g_timer.begin[i]) != hipSuccess) return fail(5, "hipEventCreate failed");
+      if (hipEventCreate(&g_timer.end[i]) != hipSuccess) return fail(5, "hipEventCreate failed");
+    }
+    g_timer.created = true;
+  }
+  for (int i = 0; i < kStageCount; ++i) g_timer.used[i] = false;
+  g_timer.enabled = enable != 0;
+  return 0;
+}
+
+int rosa_hip_stage_count(void) { return kStageCount; }
+
+const char* rosa_hip_stage_name(int stage) {
+  static const char* names[kStageCount] = {"hard_forward", "vjp_prepare", "vjp_row_max",
+                                           "vjp_row_stats", "vjp_gradients", "vjp_finalize"};
+  return (stage >= 0 && stage < kStageCount) ? names[stage] : "";
+}
+
+int rosa_hip_stage_times(float* milliseconds, int count) {
+  if (!g_timer.created) return fail(5, "stage timing was never enabled");
+  for (int i = 0; i < count && i < kStageCount; ++i) {
+    milliseconds[i] = -1.0f;
+    if (!g_timer.used[i]) continue;
+    if (hipEventSynchronize(g_timer.end[i]) != hipSuccess) return fail(5, "event sync failed");
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, g_timer.begin[i], g_timer.end[i]) != hipSuccess)
+      return fail(5, "event elapsed failed");
+    milliseconds[i] = ms;
+  }
+  return 0;
 }
 
 int rosa_hip_read_offset_error(const void* workspace, void* stream) {

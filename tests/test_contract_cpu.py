@@ -1,0 +1,247 @@
+"""Host-side contract: validation, capabilities, schemas, C-ABI symbols (no GPU)."""
+
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+import rosa_soft_amd
+from rosa_soft_amd import cabi, soft_contract
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_defaults_are_frozen():
+    # reference tests/test_soft_reference.py:28-31
+    assert soft_contract.ROSA_SOFT_DEFAULT_SCALE == 1.0
+    assert soft_contract.ROSA_SOFT_DEFAULT_DROPOUT_P == 0.0
+    assert soft_contract.ROSA_SOFT_DEFAULT_MISMATCH_SCALE == 3.0
+    assert soft_contract.ROSA_SOFT_NULL_ROUTE_SCORE == 0.5
+
+
+def _validate(**kwargs):
+    tensor = torch.ones(1, 5, 1, 1)
+    controls = dict(max_suffix_length=32, scale=1.0, dropout_p=0.0, mismatch_scale=3.0)
+    controls.update(kwargs)
+    horizon = soft_contract.validate_rosa_soft_inputs(tensor, tensor, tensor, **controls)
+    soft_contract.validate_fp32_surrogate_scalars(
+        horizon, controls["scale"], controls["dropout_p"], controls["mismatch_scale"]
+    )
+    return horizon
+
+
+@pytest.mark.parametrize(
+    ("kwargs", "message"),
+    [
+        ({"max_suffix_length": 0}, "max_suffix_length"),
+        ({"scale": True}, "scale"),
+        ({"scale": 0.0}, "scale"),
+        ({"scale": math.inf}, "scale"),
+        ({"scale": math.nan}, "scale"),
+        ({"scale": 1e-300}, "scale"),
+        ({"scale": 1e300}, "scale"),
+        ({"dropout_p": True}, "dropout_p"),
+        ({"dropout_p": -0.1}, "dropout_p"),
+        ({"dropout_p": 1.0}, "dropout_p"),
+        ({"dropout_p": math.nan}, "dropout_p"),
+        ({"dropout_p": math.inf}, "dropout_p"),
+        ({"mismatch_scale": 0.0}, "mismatch_scale"),
+        ({"mismatch_scale": True}, "mismatch_scale"),
+        ({"mismatch_scale": math.nan}, "mismatch_scale"),
+        ({"mismatch_scale": math.inf}, "mismatch_scale"),
+        ({"mismatch_scale": 1e-300}, "mismatch_scale"),
+        ({"mismatch_scale": 1e300}, "mismatch_scale"),
+    ],
+)
+def test_static_parameter_validation(kwargs, message):
+    # reference tests/test_soft_reference.py:609-635
+    with pytest.raises(ValueError, match=message):
+        _validate(**kwargs)
+
+
+def test_window_is_integral_and_clamped():
+    # reference tests/test_soft_reference.py:565-583
+    assert _validate(max_suffix_length=10**9) == 5
+    assert _validate(max_suffix_length=3) == 3
+    for invalid in (True, 1.5):
+        with pytest.raises(TypeError, match="integer"):
+            _validate(max_suffix_length=invalid)
+    assert _validate(dropout_p=1.0 - 2.0**-24) == 5
+
+
+def test_shape_head_bit_and_dtype_validation():
+    # reference tests/test_soft_reference.py:651-670
+    query = torch.ones(1, 3, 2, 4)
+    key = torch.ones_like(query)
+    value = torch.ones(1, 3, 1, 2)
+    check = lambda q, k, v: soft_contract.validate_rosa_soft_inputs(q, k, v, 4, 1.0, 0.0, 3.0)
+    with pytest.raises(ValueError, match="sequence"):
+        check(query, key[:, :-1], value)
+    with pytest.raises(ValueError, match="divisible"):
+        check(query[:, :, :1], key[:, :, :1], value.repeat(1, 1, 2, 1))
+    with pytest.raises(ValueError, match=r"\[1, 32\]"):
+        check(torch.ones(1, 3, 1, 33), torch.ones(1, 3, 1, 33), value)
+    with pytest.raises(ValueError, match="same dtype"):
+        check(query.double(), key, value)
+    with pytest.raises(ValueError, match="floating-point"):
+        check(query.long(), key.long(), value.long())
+
+
+def test_packed_validation_and_host_offsets():
+    # reference tests/test_soft_varlen.py:144-178
+    query = torch.ones(6, 2, 3)
+    value = torch.ones(6, 1, 2)
+
+    def check(offsets, dtype=torch.int32):
+        return soft_contract.validate_rosa_soft_varlen_inputs(
+            query, query, value, torch.tensor(offsets, dtype=dtype), 4, 1.0, 0.0, 3.0
+        )
+
+    assert check([0, 2, 2, 6]) == 4
+    with pytest.raises(ValueError, match="start at zero"):
+        check([1, 6])
+    with pytest.raises(ValueError, match="end at the packed token count"):
+        check([0, 5])
+    with pytest.raises(ValueError, match="nondecreasing"):
+        check([0, 4, 3, 6])
+    with pytest.raises(ValueError, match="int32"):
+        check([0, 6], dtype=torch.int64)
+    with pytest.raises(ValueError, match="one-dimensional"):
+        soft_contract.validate_rosa_soft_varlen_inputs(
+            query, query, value, torch.tensor([[0, 6]], dtype=torch.int32), 4, 1.0, 0.0, 3.0
+        )
+
+
+def test_seed_rule_draws_only_when_needed():
+    # reference rosa_soft/soft_contract.py:18-31, tests/test_soft_reference.py:468-490
+    reference = torch.ones(1)
+    state = torch.random.get_rng_state()
+    assert soft_contract.make_dropout_seed(reference, 0.0, True).numel() == 0
+    assert soft_contract.make_dropout_seed(reference, 0.5, False).numel() == 0
+    assert torch.equal(state, torch.random.get_rng_state())
+    seed = soft_contract.make_dropout_seed(reference, 0.5, True)
+    assert seed.dtype == torch.int64 and seed.ndim == 0 and int(seed) >= 0
+    assert not torch.equal(state, torch.random.get_rng_state())
+
+
+def test_capabilities_and_public_surface():
+    # reference tests/test_build_contract.py:276-334 (the variant set gains "rocm")
+    caps = rosa_soft_amd.BUILD_CAPABILITIES
+    assert caps.variant in {"reference", "rocm"}
+    assert caps.compiled_extension and caps.rosa_soft_cuda and caps.variant == "rocm"
+    assert caps.rosa_runtime is False
+    with pytest.raises(Exception):
+        caps.variant = "other"
+    assert rosa_soft_amd.__all__ == [
+        "__version__", "BUILD_CAPABILITIES", "RosaRuntime", "rosa_soft",
+        "rosa_soft_reference", "rosa_soft_varlen", "rosa_soft_varlen_reference",
+    ]
+    with pytest.raises(RuntimeError, match="unavailable"):
+        rosa_soft_amd.RosaRuntime(1, 1, 1, 1, 1)
+    with pytest.raises(RuntimeError, match="test infrastructure"):
+        rosa_soft_amd.rosa_soft_reference()
+
+
+def test_exact_operator_schemas_and_dispatch_key():
+    # reference tests/test_soft_cuda.py:1088-1102, tests/test_soft_varlen.py:281-301
+    triple = "(Tensor output, Tensor packed_query_symbols, Tensor packed_key_symbols)"
+    grads = "(Tensor grad_query, Tensor grad_key, Tensor grad_value)"
+    expected = {
+        "hard_forward": "rosa_soft::hard_forward(Tensor query, Tensor key, Tensor value, "
+        f"int max_suffix_length) -> {triple}",
+        "hard_forward_varlen": "rosa_soft::hard_forward_varlen(Tensor query, Tensor key, "
+        f"Tensor value, Tensor cu_seqlens, int max_suffix_length) -> {triple}",
+        "surrogate_vjp_masked": "rosa_soft::surrogate_vjp_masked(Tensor query, Tensor key, "
+        "Tensor value, Tensor grad_output, Tensor packed_query_symbols, "
+        "Tensor packed_key_symbols, Tensor dropout_seed, int max_suffix_length, float scale, "
+        f"float dropout_p, float mismatch_scale, int gradient_mask) -> {grads}",
+        "surrogate_vjp_varlen_masked": "rosa_soft::surrogate_vjp_varlen_masked(Tensor query, "
+        "Tensor key, Tensor value, Tensor cu_seqlens, Tensor grad_output, "
+        "Tensor packed_query_symbols, Tensor packed_key_symbols, Tensor dropout_seed, "
+        "int max_suffix_length, float scale, float dropout_p, float mismatch_scale, "
+        f"int gradient_mask) -> {grads}",
+    }
+    for name, schema in expected.items():
+        assert str(getattr(torch.ops.rosa_soft, name).default._schema) == schema
+        assert torch._C._dispatch_has_kernel_for_dispatch_key(f"rosa_soft::{name}", "CUDA")
+    source = open(os.path.join(ROOT, "rosa_soft_amd", "csrc", "rosa_dispatch.cpp")).read()
+    assert len(re.findall(r"\bm\.def\(", source)) == 4
+
+
+def test_public_signatures():
+    # reference tests/test_soft_cuda.py:1072-1086
+    import inspect
+
+    signature = inspect.signature(rosa_soft_amd.rosa_soft)
+    assert list(signature.parameters) == [
+        "query", "key", "value", "max_suffix_length", "scale", "dropout_p", "mismatch_scale",
+    ]
+    for name in ("max_suffix_length", "scale", "dropout_p", "mismatch_scale"):
+        assert signature.parameters[name].kind is inspect.Parameter.KEYWORD_ONLY
+    assert signature.parameters["max_suffix_length"].default == 32
+    packed = inspect.signature(rosa_soft_amd.rosa_soft_varlen)
+    assert list(packed.parameters)[:4] == ["query", "key", "value", "cu_seqlens"]
+
+
+def test_fake_tensor_shapes():
+    # reference tests/test_soft_cuda.py:100-111
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        query = torch.empty(2, 5, 4, 8, device="cuda", dtype=torch.bfloat16)
+        value = torch.empty(2, 5, 2, 3, device="cuda", dtype=torch.bfloat16)
+        out, pq, pk = torch.ops.rosa_soft.hard_forward(query, query, value, 3)
+        assert out.shape == (2, 5, 4, 3) and out.dtype == torch.bfloat16
+        assert pq.shape == pk.shape == (2, 4, 5) and pq.dtype == torch.int32
+        assert pq.stride() == (20, 5, 1)
+        grads = torch.ops.rosa_soft.surrogate_vjp_masked(
+            query, query, value, out, pq, pk, torch.empty(0, dtype=torch.int64, device="cuda"),
+            3, 1.0, 0.0, 3.0, 5,
+        )
+        assert grads[0].shape == query.shape and grads[0].dtype == torch.float32
+        assert grads[1].shape == (0,) and grads[2].shape == value.shape
+        tokens = torch.empty(7, 4, 8, device="cuda")
+        packed_value = torch.empty(7, 2, 3, device="cuda")
+        offsets = torch.empty(3, dtype=torch.int32, device="cuda")
+        out, pq, _ = torch.ops.rosa_soft.hard_forward_varlen(tokens, tokens, packed_value, offsets, 3)
+        assert out.shape == (7, 4, 3) and pq.shape == (4, 7)
+
+
+def test_cpu_tensors_are_rejected_before_any_launch():
+    # reference rosa_soft/soft.py:47-54
+    tensor = torch.ones(1, 3, 1, 1)
+    with pytest.raises(ValueError, match="CUDA"):
+        rosa_soft_amd.rosa_soft(tensor, tensor, tensor)
+    packed = torch.ones(3, 1, 1)
+    with pytest.raises(ValueError, match="CUDA"):
+        rosa_soft_amd.rosa_soft_varlen(packed, packed, packed, torch.tensor([0, 3], dtype=torch.int32))
+
+
+def test_c_abi_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "rosa_soft_hip.h")).read()
+    declared = set(re.findall(r"\b(rosa_hip_[a-z_]+)\s*\(", header))
+    assert declared == set(cabi.EXPORTED_SYMBOLS)
+    library = ctypes.CDLL(cabi.LIBRARY_PATH)
+    for symbol in declared:
+        assert hasattr(library, symbol), symbol
+    loaded = cabi.load()
+    assert loaded.rosa_hip_version() >= 100
+    assert loaded.rosa_hip_target() == b"rocm-gfx950"
+    # host-side arithmetic only: workspace sizes and argument rejection
+    problem = cabi.RosaProblem(dtype=0, B=2, T=128, N=256, S=0, H=4, D=8, Hv=2, Dv=8, W=16)
+    assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) >= 256 * 4 * 4
+    assert loaded.rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0) > 0
+    problem.D = 33
+    assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) == 0
+    assert b"[1, 32]" in loaded.rosa_hip_last_error()
+
+
+def test_no_product_module_imports_the_oracle():
+    package = os.path.join(ROOT, "rosa_soft_amd")
+    for name in os.listdir(package):
+        if name.endswith(".py"):
+            text = open(os.path.join(package, name)).read()
+            assert "import oracle" not in text and "from oracle" not in text, name

@@ -1,0 +1,324 @@
+"""Parity of the HIP path against the CPU oracle (needs a real MI355X).
+
+The kernels are driven through the C ABI (``rosa_soft_amd.cabi``); the last
+section goes through the public operators and the dispatcher.  Bars:
+
+* hard forward, packed symbols and route indices: bit-exact;
+* gradients: ``|got - want| <= 1e-4 * |want| + 1e-5 * max|want|`` against the
+  float64 streamed oracle for every input dtype at the C-ABI level (the
+  kernels compute in float32 whatever the input type), and the reference's own
+  half-precision bars ``(3e-3, 3e-3)`` / ``(2e-2, 2e-2)`` after the public
+  operator has cast gradients to float16 / bfloat16.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from tests.conftest import nonzero_randn
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from rosa_soft_amd import cabi as module
+
+    module.load()
+    return module
+
+
+def assert_gradients_close(got, want, label="", slack=1.0):
+    got = got.detach().cpu().double()
+    want = want.double()
+    assert torch.isfinite(got).all(), label
+    tolerance = slack * (1e-4 * want.abs() + 1e-5 * want.abs().max())
+    excess = ((got - want).abs() - tolerance).max().item()
+    assert excess <= 0.0, f"{label}: exceeds tolerance by {excess:.3e} (max|want| {want.abs().max():.3e})"
+
+
+def make_case(B, T, H, D, Hv, Dv, dtype=torch.float32, seed=0, pattern="random"):
+    query = nonzero_randn((B, T, H, D), seed=seed + 1).to(dtype)
+    key = nonzero_randn((B, T, H, D), seed=seed + 2).to(dtype)
+    value = nonzero_randn((B, T, Hv, Dv), seed=seed + 3).to(dtype)
+    grad_output = nonzero_randn((B, T, H, Dv), seed=seed + 4, floor=0.0).to(dtype)
+    if pattern == "shifted":  # long near-exact matches along one diagonal
+        key = query.roll(3, dims=1).clone()
+        key[:, ::7] = -key[:, ::7]
+    elif pattern == "all_match":
+        query = torch.ones_like(query)
+        key = torch.ones_like(key)
+    elif pattern == "periodic":
+        period = nonzero_randn((B, 5, H, D), seed=seed + 9).to(dtype)
+        reps = (T + 4) // 5
+        key = period.repeat(1, reps, 1, 1)[:, :T].clone()
+        query = key.clone()
+    return query, key, value, grad_output
+
+
+def run_device(cabi, query, key, value, grad_output, W, scale=1.0, p=0.0, ms=3.0, seed=None,
+               mask=7, cu_seqlens=None):
+    q, k, v, go = (t.to(DEVICE).contiguous() for t in (query, key, value, grad_output))
+    offsets = None if cu_seqlens is None else torch.tensor(cu_seqlens, dtype=torch.int32, device=DEVICE)
+    out, pq, pk, routes = cabi.hard_forward(q, k, v, W, offsets)
+    seed_tensor = None if seed is None else torch.tensor(seed, dtype=torch.int64, device=DEVICE)
+    grads = cabi.surrogate_vjp(q, k, v, go, pq, pk, seed_tensor, W, scale, p, ms, mask, offsets)
+    torch.cuda.synchronize()
+    return out, pq, pk, routes, grads
+
+
+# --------------------------------------------------------------------------- forward
+
+FORWARD_CASES = [
+    # B, T, H, D, Hv, Dv, W, dtype, pattern
+    (1, 1, 1, 1, 1, 1, 1, torch.float32, "random"),
+    (2, 33, 2, 4, 1, 5, 8, torch.float32, "random"),
+    (1, 64, 2, 2, 2, 3, 64, torch.float32, "random"),
+    (1, 65, 1, 1, 1, 7, 1000, torch.float16, "random"),
+    (2, 257, 4, 3, 2, 12, 16, torch.bfloat16, "random"),
+    (1, 200, 2, 5, 1, 9, 31, torch.float32, "shifted"),
+    (1, 300, 2, 32, 2, 4, 40, torch.float32, "shifted"),
+    (1, 193, 1, 8, 1, 8, 128, torch.float32, "all_match"),
+    (1, 150, 2, 7, 1, 70, 9, torch.float16, "periodic"),
+    (1, 700, 3, 2, 3, 33, 64, torch.bfloat16, "random"),
+]
+
+
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,dtype,pattern", FORWARD_CASES)
+def test_hard_forward_is_bit_exact(cabi, c_oracle, B, T, H, D, Hv, Dv, W, dtype, pattern):
+    query, key, value, _ = make_case(B, T, H, D, Hv, Dv, dtype, seed=T, pattern=pattern)
+    q, k, v = (t.to(DEVICE) for t in (query, key, value))
+    out, pq, pk, routes = cabi.hard_forward(q, k, v, W)
+    torch.cuda.synchronize()
+    want_out, want_routes, _ = c_oracle.hard_forward(query, key, value, W)
+    assert out.dtype == dtype and out.shape == (B, T, H, Dv)
+    assert torch.equal(out.cpu().float(), want_out.float())
+    assert torch.equal(routes.cpu(), want_routes)
+    # packed symbols: bit i = x[..., i] > 0, head-major [B, H, T] (reference
+    # tests/test_soft_cuda.py:80-98)
+    weights = 1 << torch.arange(D, dtype=torch.int64)
+    want_pq = ((query > 0).long() * weights).sum(-1).permute(0, 2, 1)
+    want_pk = ((key > 0).long() * weights).sum(-1).permute(0, 2, 1)
+    assert pq.shape == (B, H, T) and pq.stride() == (H * T, T, 1) and pq.dtype == torch.int32
+    assert torch.equal(pq.cpu().long() & 0xFFFFFFFF, want_pq)
+    assert torch.equal(pk.cpu().long() & 0xFFFFFFFF, want_pk)
+    assert set(out.cpu().float().unique().tolist()) <= {-1.0, 0.0, 1.0}
+
+
+def test_sign_policy_for_zero_and_non_finite_inputs(cabi, c_oracle):
+    # zeros, -0, NaN and -inf quantise to -1, +inf to +1 (reference
+    # docs/CONCEPT.md:27-33, tests/test_soft_cuda.py:570-611)
+    query = nonzero_randn((1, 40, 1, 4), seed=1)
+    key = query.roll(1, dims=1).clone()
+    specials = torch.tensor([0.0, -0.0, float("nan"), float("-inf"), float("inf")])
+    query[0, 5:10, 0, 0] = specials
+    key[0, 6:11, 0, 1] = specials
+    value = nonzero_randn((1, 40, 1, 3), seed=2)
+    value[0, 7, 0] = torch.tensor([0.0, float("nan"), float("inf")])
+    out, _, _, routes = cabi.hard_forward(query.to(DEVICE), key.to(DEVICE), value.to(DEVICE), 8)
+    want_out, want_routes, _ = c_oracle.hard_forward(query, key, value, 8)
+    assert torch.equal(out.cpu(), want_out) and torch.equal(routes.cpu(), want_routes)
+
+
+# --------------------------------------------------------------------------- gradients
+
+VJP_CASES = [
+    # B, T, H, D, Hv, Dv, W, scale, p, ms, dtype, pattern
+    (1, 33, 2, 16, 1, 5, 16, 1.0, 0.0, 3.0, torch.float32, "random"),
+    (2, 130, 4, 8, 2, 8, 16, 1.0, 0.0, 3.0, torch.float32, "random"),
+    (1, 257, 2, 3, 2, 12, 300, 1.3, 0.0, 2.0, torch.float32, "random"),
+    (1, 160, 1, 1, 1, 4, 160, 1.0, 0.0, 3.0, torch.float32, "random"),
+    (2, 200, 4, 8, 2, 8, 16, 1.0, 0.25, 3.0, torch.float32, "random"),
+    (1, 96, 2, 4, 1, 6, 12, 0.25, 0.9, 1.0, torch.float32, "random"),
+    (1, 700, 2, 2, 1, 40, 64, 1.0, 0.0, 3.0, torch.float32, "shifted"),
+    (1, 300, 2, 1, 1, 4, 300, 1.0, 0.0, 3.0, torch.float32, "shifted"),
+    (1, 600, 1, 8, 1, 8, 128, 1.0, 0.0, 3.0, torch.float32, "all_match"),
+    (1, 260, 2, 6, 2, 17, 40, 0.7, 0.1, 9.0, torch.float32, "periodic"),
+    (1, 160, 1, 16, 1, 33, 32, 4.0, 0.1, 9.0, torch.bfloat16, "random"),
+    (2, 140, 2, 32, 2, 64, 24, 1.0, 0.0, 3.0, torch.float16, "shifted"),
+    (1, 1200, 2, 8, 1, 8, 128, 1.0, 0.1, 3.0, torch.float32, "random"),
+    (1, 180, 2, 8, 2, 8, 32, 10.0, 0.0, 3.0, torch.float32, "shifted"),   # row-maximum pass
+    (1, 120, 1, 4, 1, 4, 120, 30.0, 0.2, 0.5, torch.float32, "periodic"),  # row-maximum pass
+]
+
+
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,scale,p,ms,dtype,pattern", VJP_CASES)
+def test_surrogate_vjp_matches_oracle(cabi, c_oracle, B, T, H, D, Hv, Dv, W, scale, p, ms, dtype,
+                                      pattern):
+    query, key, value, grad_output = make_case(B, T, H, D, Hv, Dv, dtype, seed=7 * T + D, pattern=pattern)
+    seed = 0x5DEECE66D1234567 if p > 0 else None
+    out, _, _, _, grads = run_device(cabi, query, key, value, grad_output, W, scale, p, ms, seed)
+    want = c_oracle.surrogate_vjp(
+        query, key, value, grad_output, max_suffix_length=W, scale=scale, dropout_p=p,
+        mismatch_scale=ms, seed=seed,
+    )
+    # float32 logits of magnitude scale * U(W) carry an absolute rounding error of
+    # about 2^-24 of that magnitude into the exponent, so the bar widens with it
+    # once it passes ~10 (the float32 reference kernels have the same limit)
+    longest_logit = scale * 2.4142 * ((1.0 + min(W, T)) ** 0.5 - 1.0)
+    slack = max(1.0, longest_logit / 10.0)
+    for name, got, expected in zip(("grad_query", "grad_key", "grad_value"), grads, want):
+        assert got.dtype == torch.float32 and got.shape == expected.shape
+        assert_gradients_close(got, expected, name, slack)
+    # structural zeros (first query row, last key row, first value row)
+    assert torch.count_nonzero(grads[0][:, 0]) == 0
+    assert torch.count_nonzero(grads[1][:, -1]) == 0
+    assert torch.count_nonzero(grads[2][:, 0]) == 0
+
+
+@pytest.mark.parametrize("mask", range(1, 8))
+def test_gradient_masks(cabi, c_oracle, mask):
+    # reference tests/test_soft_cuda.py:510-567
+    query, key, value, grad_output = make_case(1, 70, 2, 5, 1, 6, seed=mask)
+    seed = 4242 + mask
+    _, _, _, _, grads = run_device(cabi, query, key, value, grad_output, 9, 1.0, 0.3, 3.0, seed, mask)
+    want = c_oracle.surrogate_vjp(
+        query, key, value, grad_output, max_suffix_length=9, dropout_p=0.3, seed=seed
+    )
+    for bit, got, expected in zip((1, 2, 4), grads, want):
+        if mask & bit:
+            assert_gradients_close(got, expected)
+        else:
+            assert got is None
+
+
+def test_dropout_seed_halves_and_replay(cabi):
+    query, key, value, grad_output = make_case(1, 90, 2, 4, 2, 4, seed=3)
+    low = run_device(cabi, query, key, value, grad_output, 8, p=0.5, seed=7)[4]
+    again = run_device(cabi, query, key, value, grad_output, 8, p=0.5, seed=7)[4]
+    high = run_device(cabi, query, key, value, grad_output, 8, p=0.5, seed=(1 << 32) + 7)[4]
+    for a, b in zip(low, again):  # accumulation order is free: compare to tolerance
+        torch.testing.assert_close(a, b, rtol=2e-6, atol=2e-7)
+    assert any(not torch.allclose(a, b) for a, b in zip(low, high))
+
+
+def test_every_causal_value_is_credited_and_singleton_is_zero(cabi):
+    # reference tests/test_soft_cuda.py:693-713, tests/test_soft_reference.py:436-444
+    query = torch.ones(1, 6, 2, 3)
+    key = -torch.ones(1, 6, 2, 3)
+    value = nonzero_randn((1, 6, 1, 4), seed=50)
+    out, _, _, _, grads = run_device(cabi, query, key, value, torch.ones(1, 6, 2, 4), 4)
+    assert torch.count_nonzero(out) == 0
+    assert torch.all(grads[2][:, 1:].abs().sum(dim=(0, 2, 3)) > 0)
+    ones = torch.ones(1, 1, 1, 1)
+    out, _, _, _, grads = run_device(cabi, ones, ones, ones, ones, 1)
+    assert torch.count_nonzero(out) == 0
+    assert all(torch.count_nonzero(g) == 0 for g in grads)
+
+
+# --------------------------------------------------------------------------- packed layout
+
+PACKED_CASES = [
+    # lengths, H, D, Hv, Dv, W, p, dtype
+    ([5, 0, 7, 1, 12], 2, 3, 1, 4, 4, 0.3, torch.float32),
+    ([1, 2, 127, 0, 128, 129], 2, 4, 2, 5, 160, 0.0, torch.float32),
+    ([64, 65, 63], 4, 8, 2, 8, 16, 0.2, torch.bfloat16),
+    ([300, 40, 0, 0, 513], 2, 2, 1, 33, 32, 0.1, torch.float16),
+]
+
+
+@pytest.mark.parametrize("lengths,H,D,Hv,Dv,W,p,dtype", PACKED_CASES)
+def test_packed_layout_matches_oracle(cabi, c_oracle, lengths, H, D, Hv, Dv, W, p, dtype):
+    # reference tests/test_soft_varlen.py:42-141, :392-475, :860-915
+    offsets = [0, *np.cumsum(lengths).tolist()]
+    total = offsets[-1]
+    query = nonzero_randn((total, H, D), seed=50).to(dtype)
+    key = nonzero_randn((total, H, D), seed=51).to(dtype)
+    if D <= 2:
+        key = query.roll(2, dims=0).clone()
+    value = nonzero_randn((total, Hv, Dv), seed=52).to(dtype)
+    grad_output = nonzero_randn((total, H, Dv), seed=53, floor=0.0).to(dtype)
+    seed = 987654321 if p > 0 else None
+    out, pq, pk, routes, grads = run_device(
+        cabi, query, key, value, grad_output, W, 1.0, p, 3.0, seed, 7, offsets
+    )
+    want_out, want_routes = c_oracle.varlen_hard_forward(query, key, value, offsets, W)
+    assert out.shape == (total, H, Dv) and pq.shape == (H, total)
+    assert torch.equal(out.cpu().float(), want_out.float())
+    assert torch.equal(routes.cpu(), want_routes)
+    want = c_oracle.varlen_surrogate_vjp(
+        query, key, value, offsets, grad_output, max_suffix_length=W, dropout_p=p, seed=seed
+    )
+    for got, expected in zip(grads, want):
+        assert_gradients_close(got, expected)
+    for start, end in zip(offsets[:-1], offsets[1:]):
+        if end > start:
+            assert torch.count_nonzero(grads[2][start]) == 0
+            assert torch.count_nonzero(grads[1][end - 1]) == 0
+            assert torch.count_nonzero(grads[0][start]) == 0
+
+
+def test_packed_equals_dense_batch_with_same_seed(cabi):
+    # reference tests/test_soft_varlen.py:304-389
+    B, T, H, D, Hv, Dv = 3, 70, 2, 4, 1, 5
+    query, key, value, grad_output = make_case(B, T, H, D, Hv, Dv, seed=11)
+    dense = run_device(cabi, query, key, value, grad_output, 12, p=0.4, seed=99)
+    flat = [t.reshape(B * T, *t.shape[2:]) for t in (query, key, value, grad_output)]
+    packed = run_device(cabi, *flat, 12, p=0.4, seed=99, cu_seqlens=[0, T, 2 * T, 3 * T])
+    assert torch.equal(dense[0].reshape(B * T, H, Dv), packed[0])
+    assert torch.equal(dense[3].permute(1, 0, 2).reshape(H, B * T), packed[3])
+    for a, b in zip(dense[4], packed[4]):
+        torch.testing.assert_close(a.reshape(b.shape), b, rtol=2e-5, atol=2e-6)
+
+
+def test_invalid_device_offsets_are_clamped_and_reported(cabi):
+    """Offsets the host cannot see are sanitised on the device (no fault) and
+    the violation is reported through the workspace flag."""
+
+    import ctypes
+
+    total, H, D, Dv = 40, 2, 4, 3
+    query = nonzero_randn((total, H, D), seed=1).to(DEVICE)
+    value = nonzero_randn((total, 1, Dv), seed=2).to(DEVICE)
+    library = cabi.load()
+    for offsets, bad in (([0, 10, 40], 0), ([0, 30, 20, 40], 1), ([0, 10, 50], 1), ([2, 40], 1)):
+        cu = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
+        problem = cabi.make_problem(query, value, 8, cu)
+        size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
+        workspace = torch.zeros(size, dtype=torch.uint8, device=DEVICE)
+        out = torch.empty(total, H, Dv, device=DEVICE)
+        words = torch.empty(2, H, total, dtype=torch.int32, device=DEVICE)
+        stream = torch.cuda.current_stream().cuda_stream
+        status = library.rosa_hip_hard_forward(
+            ctypes.byref(problem), query.data_ptr(), query.data_ptr(), value.data_ptr(),
+            out.data_ptr(), words[0].data_ptr(), words[1].data_ptr(), None,
+            workspace.data_ptr(), size, stream,
+        )
+        assert status == 0
+        assert library.rosa_hip_read_offset_error(workspace.data_ptr(), stream) == bad
+
+
+# --------------------------------------------------------------------------- golden vectors on the device
+
+def test_device_matches_reference_golden_vectors(cabi):
+    """GPU results against the vectors written by the reference's own oracle."""
+
+    import os
+
+    from tests.golden import make_reference_vectors as gold
+
+    vectors = np.load(os.path.join(os.path.dirname(gold.__file__), "reference_vectors.npz"))
+    bars = {"float32": (2e-4, 2e-6), "float16": (3e-3, 3e-3), "bfloat16": (2e-2, 2e-2)}
+    for name, case in gold.DENSE_CASES.items():
+        B, T, H, D, Hv, Dv, W, scale, p, ms, dtype, seed = case
+        q, k, v, go = gold.dense_inputs(case)
+        out, _, _, _, grads = run_device(cabi, q, k, v, go, W, scale, p, ms, seed)
+        assert torch.equal(out.cpu().float(), torch.from_numpy(vectors[name + "/out"].astype(np.float32)))
+        rtol, atol = bars[dtype]
+        for label, got in zip(("gq", "gk", "gv"), grads):
+            want = torch.from_numpy(vectors[name + "/" + label])
+            torch.testing.assert_close(got.cpu(), want, rtol=rtol, atol=atol)
+    for name, case in gold.VARLEN_CASES.items():
+        lengths, H, D, Hv, Dv, W, scale, p, ms, dtype, _ = case
+        q, k, v, go = gold.varlen_inputs(case)
+        offsets = [0, *np.cumsum(lengths).tolist()]
+        seed = int(vectors[name + "/seed"][0])
+        out, _, _, _, grads = run_device(cabi, q, k, v, go, W, scale, p, ms, seed, 7, offsets)
+        assert torch.equal(out.cpu().float(), torch.from_numpy(vectors[name + "/out"].astype(np.float32)))
+        rtol, atol = bars[dtype]
+        for label, got in zip(("gq", "gk", "gv"), grads):
+            torch.testing.assert_close(got.cpu(), torch.from_numpy(vectors[name + "/" + label]), rtol=rtol, atol=atol)
