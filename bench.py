@@ -44,6 +44,7 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3
 #       packed -> dict(lengths, H, D, Hv, Dv, W, p, ms, dtype)
 WORKLOADS = {
     "metric": dict(B=2, T=4096, H=64, D=8, Hv=16, Dv=8, W=128, p=0.1, ms=3.0, dtype="float32"),
+    "metric_p0": dict(B=2, T=4096, H=64, D=8, Hv=16, Dv=8, W=128, p=0.0, ms=3.0, dtype="float32"),
     "config1": dict(B=1, T=256, H=4, D=4, Hv=4, Dv=8, W=16, p=0.0, ms=3.0, dtype="float32"),
     "config2": dict(B=2, T=1024, H=64, D=8, Hv=16, Dv=8, W=128, p=0.1, ms=3.0, dtype="float32"),
     "config3": dict(B=4, T=4096, H=32, D=16, Hv=32, Dv=64, W=32, p=0.0, ms=3.0, dtype="bfloat16"),

@@ -38,9 +38,8 @@ constexpr float kSqrtScale = 2.414213562373095f;  // sqrt(2) + 1
 constexpr float kLog2e = 1.4426950408889634f;
 
 constexpr int kChunk = 16;     // rows kept in registers between the forward and reverse sweeps
-constexpr int kSegment = 512;  // rows between two checkpoints kept in LDS
+constexpr int kSegment = 128;  // rows between two checkpoints kept in LDS
 constexpr int kSegChunks = kSegment / kChunk;
-constexpr int kColumnRing = 128;  // circular column accumulators (>= kChunk + 63)
 
 thread_local char g_error[512] = "";
 
@@ -801,27 +800,57 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
 // wave is above `tail_threshold` (long near-exact matches).
 //
 // Each chunk leaves its route weights d*p and gate adjoints h in LDS as
-// [row][lane] tiles, from which the three contractions are formed with one
-// output element per lane:
+// [row][lane] tiles (with zero margins), from which the three contractions
 //   dV[a, :]   += sum_t  d p(t, a) go[t, :]
 //   dK[a-1, :] += c sum_t h(t, a) z(q[t, :])
 //   dQ[t, :]   += c sum_a h(t, a) z(k[a-1, :]),   c = mismatch_scale / (2 D)
-// Column sums complete after 64 rows, so they are kept in circular LDS
-// accumulators and flushed with one global atomic per element.
-template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
-__global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
+// are formed on the matrix cores (v_mfma_f32_16x16x4_f32).  In the chunk's own
+// (row r, window column c) coordinates the pair (r, lane l) sits at
+// c = 64 - l + r, i.e. the tile read with a skew is an ordinary matrix.  The
+// window spans 80 columns = 5 MFMA tiles; a chunk completes exactly the last
+// tile (the 16 highest columns), which is flushed with global atomics, and the
+// other four shift up by one tile for the next chunk, so column sums live in
+// accumulator registers for their whole life.
+constexpr int kTilePitch = 96;   // 16 zero + 64 lanes + 16 zero
+constexpr int kWindowTiles = 5;  // 80 window columns
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ v4f mfma_16x16x4(float a, float b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float sign_of_bit(uint32_t word, int bit, int width) {
+  // +1 / -1 for symbol bits, 0 for padding columns beyond the symbol width
+  if (bit >= width) return 0.0f;
+  return ((word >> bit) & 1u) ? 1.0f : -1.0f;
+}
+
+// register budget of the gradient kernel: waves per SIMD it is compiled for
+constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
+  if (value_tiles == 1 && symbol_tiles == 1) return 3;   // 168 registers, no spills
+  if (value_tiles == 4 && symbol_tiles == 2) return 1;   // 120 accumulator registers alone
+  return 2;
+}
+
+template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
+__global__ __launch_bounds__(kWave)
+__attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
+void vjp_gradients_kernel(VjpParams P) {
+  constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
+  constexpr int GP = VT * 16;           // pitch of the staged grad_output rows
   extern __shared__ float lds[];
   float* ck_evidence = lds;                                  // [kSegChunks][64]
   int* ck_window = reinterpret_cast<int*>(lds + kSegChunks * kWave);
-  float* weight_tile = lds + 2 * kSegChunks * kWave;         // [kChunk][64]
-  float* adjoint_tile = weight_tile + kChunk * kWave;        // [kChunk][64]
-  float* grad_tile = adjoint_tile + kChunk * kWave;          // [kChunk][DVP]
-  uint32_t* key_tile = reinterpret_cast<uint32_t*>(grad_tile + kChunk * DVP);  // [kChunk + 64]
-  uint32_t* query_tile = key_tile + kChunk + kWave;          // [kChunk]
-  float* value_acc = reinterpret_cast<float*>(query_tile + kChunk);  // [kColumnRing][DVP]
-  float* key_acc = value_acc + kColumnRing * DVP;            // [kColumnRing][D]
+  float* weight_tile = lds + 2 * kSegChunks * kWave;         // [kChunk][kTilePitch]
+  float* adjoint_tile = weight_tile + kChunk * kTilePitch;   // [kChunk][kTilePitch]
+  float* grad_tile = adjoint_tile + kChunk * kTilePitch;     // [kChunk][GP]
+  uint32_t* key_tile = reinterpret_cast<uint32_t*>(grad_tile + kChunk * GP);  // [80]
+  uint32_t* query_tile = key_tile + 16 * kWindowTiles;       // [kChunk]
 
   const int lane = threadIdx.x;
+  const int li = lane & 15;   // MFMA row (A) / column (B, C) index
+  const int lg = lane >> 4;   // MFMA k index (A, B) / row group (C)
   const int W = P.L.W;
   const int D = P.L.D;
   const int Dv = P.L.Dv;
@@ -832,6 +861,12 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
   const float symbol_scale = 0.5f * P.mismatch_scale / static_cast<float>(D);
   float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
   float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
+
+  // zero the tiles once: the margins are never written again
+  for (int index = lane; index < 2 * kChunk * kTilePitch + kChunk * GP; index += kWave) {
+    weight_tile[index] = 0.0f;
+  }
+  __syncthreads();
 
   for (;;) {
     int unit_index = 0;
@@ -852,9 +887,16 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
       key.seed_high_salt = static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u;
     }
 
-    // clear the circular column accumulators
-    for (int index = lane; index < kColumnRing * DVP; index += kWave) value_acc[index] = 0.0f;
-    for (int index = lane; index < kColumnRing * D; index += kWave) key_acc[index] = 0.0f;
+    // column accumulators of the 80-column window, one MFMA tile per 16 columns
+    v4f value_acc[kWindowTiles][VT];
+    v4f key_acc[kWindowTiles][DT];
+#pragma unroll
+    for (int m = 0; m < kWindowTiles; ++m) {
+#pragma unroll
+      for (int n = 0; n < VT; ++n) value_acc[m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int n = 0; n < DT; ++n) key_acc[m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 
     const int segments = (view.steps + kSegment - 1) / kSegment;
     Band<NVW> band;
@@ -863,13 +905,14 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
       band.evidence = 0.0f;
       band.window = 0;
       load_sliding<NVW>(band, view, 0, lane, W);
-      for (int i = 0; i < (segments - 1) * kSegment; ++i) {
-        if ((i % kSegment) == 0) {
-          const int segment = i / kSegment;
-          seg_ck[(2 * segment) * kWave + lane] = band.evidence;
-          seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+      for (int segment = 0; segment < segments - 1; ++segment) {
+        seg_ck[(2 * segment) * kWave + lane] = band.evidence;
+        seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+        const int first = segment * kSegment;
+#pragma unroll 4
+        for (int r = 0; r < kSegment; ++r) {
+          forward_step<NVW>(band, view, first + r, lane, W, P.gate_log2);
         }
-        forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
       }
       const int segment = segments - 1;
       seg_ck[(2 * segment) * kWave + lane] = band.evidence;
@@ -882,6 +925,7 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
     float ring_sum = 0.0f;        // sum of b * overflow over the next W + 1 rows
     int ring_live = 0;            // rows for which the ring still holds non-zero terms
     int ring_fresh = 0;           // ring reads that must be treated as zero
+    const int last_step = view.steps - 1;
 
     for (int segment = segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * kSegment;
@@ -910,7 +954,7 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
 
       for (int chunk = chunks - 1; chunk >= 0; --chunk) {
         const int first = seg_first + chunk * kChunk;   // step index of the chunk's first row
-        const int rows = min(kChunk, seg_last - first);
+        const int rows = min(kChunk, seg_last - first); // < kChunk only for the band's last rows
         band.evidence = ck_evidence[chunk * kWave + lane];
         band.window = ck_window[chunk * kWave + lane];
         load_sliding<NVW>(band, view, first, lane, W);
@@ -920,180 +964,202 @@ __global__ __launch_bounds__(kWave) void vjp_gradients_kernel(VjpParams P) {
         float keep_gate[kChunk];
         float keep_adjoint[kChunk];   // external adjoint A of the route score
 
-        // forward replay of the chunk
+        // Forward replay of the chunk.  Rows past the end of the band (only in
+        // the band's last chunk) are computed on the clamped last row and
+        // masked, which keeps the loop free of branches.
 #pragma unroll
         for (int r = 0; r < kChunk; ++r) {
-          if (r < rows) {
-            const int i = first + r;
-            const int t = view.diag0 + 1 + i;
-            const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
-            const float4 row = view.stats[t];
-            const float shift = fmaf(row.x, kLog2e, row.w);
-            const float one_plus = 1.0f + s.evidence;
-            const float inv_root = fast_rsq(one_plus);
-            const float root = one_plus * inv_root;
-            const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
-            const float null_weight = fast_exp2((P.null_logit - row.x) * kLog2e);
-            const float inv_denominator = fast_rcp(row.y + null_weight);
-            const float probability = weight * inv_denominator;
-            float keep = 1.0f;
-            if constexpr (DROPOUT) {
-              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-              keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
-            }
-            weight_tile[r * kWave + lane] = probability * keep;
-            float adjoint = 0.0f;
-            if (want_qk) {
-              const float utility = route_utility<NVW, DVP>(
-                  band, view.grad_rows + static_cast<int64_t>(t) * DVP, view.grad_sum[t]);
-              const float expected = row.z * inv_denominator;
-              adjoint = P.scale * probability * (keep * utility - expected) *
-                        (0.5f * kSqrtScale * inv_root);
-            }
-            keep_adjoint[r] = adjoint;
-            keep_gate[r] = s.gate;
-            keep_overflow[r] = s.overflow;
-            keep_evidence[r] = s.evidence + s.overflow;
-          } else {
-            keep_adjoint[r] = 0.0f;
-            keep_gate[r] = 0.0f;
-            keep_overflow[r] = 0.0f;
-            keep_evidence[r] = 0.0f;
-            weight_tile[r * kWave + lane] = 0.0f;
+          const bool row_ok = r < rows;
+          const int i = min(first + r, last_step);
+          const int t = view.diag0 + 1 + i;
+          const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
+          const float4 row = view.stats[t];
+          const float shift = fmaf(row.x, kLog2e, row.w);
+          const float one_plus = 1.0f + s.evidence;
+          const float inv_root = fast_rsq(one_plus);
+          const float root = one_plus * inv_root;
+          const bool live = s.active && row_ok;
+          const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
+          const float null_weight = fast_exp2((P.null_logit - row.x) * kLog2e);
+          const float inv_denominator = fast_rcp(row.y + null_weight);
+          const float probability = weight * inv_denominator;
+          float keep = 1.0f;
+          if constexpr (DROPOUT) {
+            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+            keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
           }
+          weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
+          float adjoint = 0.0f;
+          if (want_qk) {
+            const float utility = route_utility<NVW, DVP>(
+                band, view.grad_rows + static_cast<int64_t>(t) * DVP, view.grad_sum[t]);
+            const float expected = row.z * inv_denominator;
+            adjoint = P.scale * probability * (keep * utility - expected) *
+                      (0.5f * kSqrtScale * inv_root);
+          }
+          // rows past the band's end run on repeated data and may hold anything,
+          // NaN included: select, never multiply by zero
+          keep_adjoint[r] = live ? adjoint : 0.0f;
+          keep_gate[r] = live ? s.gate : 0.0f;
+          keep_overflow[r] = live ? s.overflow : 0.0f;
+          keep_evidence[r] = live ? s.evidence + s.overflow : 0.0f;
         }
 
         // reverse walk of the chunk
         if (want_qk) {
 #pragma unroll
           for (int r = kChunk - 1; r >= 0; --r) {
-            if (r < rows) {
-              const int i = first + r;
-              const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
-              adjoint_carry = b;
-              gate_below = keep_gate[r];
-              const float overflow = keep_overflow[r];
-              const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
-              const bool any_term = __ballot(term != 0.0f) != 0ull;
-              if (any_term) {
-                if (ring_live == 0) ring_fresh = P.ring_rows;
-                ring_live = P.ring_rows;
-              }
-              if (ring_live > 0) {
-                const int slot = i % P.ring_rows;
-                float leaving = 0.0f;
-                if (ring_fresh > 0) {
-                  --ring_fresh;
-                } else {
-                  leaving = ring[slot * kWave + lane];
-                }
-                ring[slot * kWave + lane] = term;
-                ring_sum += term - leaving;
-                --ring_live;
-              }
-              const float h = fmaf(b, keep_evidence[r], -ring_sum);
-              if (ring_live == 0) ring_sum = 0.0f;
-              const bool active = (i + 1 - lane) >= 1;
-              adjoint_tile[r * kWave + lane] = active ? h : 0.0f;
-            } else {
-              adjoint_tile[r * kWave + lane] = 0.0f;
+            const int i = first + r;
+            const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
+            adjoint_carry = b;
+            gate_below = keep_gate[r];
+            const float overflow = keep_overflow[r];
+            const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
+            const bool any_term = __ballot(term != 0.0f) != 0ull;
+            if (any_term) {
+              if (ring_live == 0) ring_fresh = P.ring_rows;
+              ring_live = P.ring_rows;
             }
+            if (ring_live > 0) {
+              const int slot = i % P.ring_rows;
+              float leaving = 0.0f;
+              if (ring_fresh > 0) {
+                --ring_fresh;
+              } else {
+                leaving = ring[slot * kWave + lane];
+              }
+              ring[slot * kWave + lane] = term;
+              ring_sum += term - leaving;
+              --ring_live;
+            }
+            const float h = fmaf(b, keep_evidence[r], -ring_sum);
+            if (ring_live == 0) ring_sum = 0.0f;
+            const bool active = (i + 1 - lane) >= 1 && r < rows;
+            adjoint_tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
           }
         }
 
-        // stage the row data of the chunk
+        // stage the row and column data of the chunk
         const int t_first = view.diag0 + 1 + first;
         const int a_first = first + 1;  // column of lane 0 in the chunk's first row
-        for (int index = lane; index < kChunk * DVP; index += kWave) {
-          const int r = index / DVP;
-          grad_tile[index] =
-              r < rows ? view.grad_rows[static_cast<int64_t>(t_first + r) * DVP + (index % DVP)]
-                       : 0.0f;
+        if (want_v) {
+          for (int index = lane; index < kChunk * DVP; index += kWave) {
+            const int r = index / DVP;
+            const int d = index - r * DVP;
+            grad_tile[r * GP + d] =
+                r < rows ? view.grad_rows[static_cast<int64_t>(t_first + r) * DVP + d] : 0.0f;
+          }
         }
         if (lane < kChunk) query_tile[lane] = lane < rows ? view.q[t_first + lane] : 0u;
-        for (int index = lane; index < kChunk + kWave - 1; index += kWave) {
-          const int a = a_first - 63 + index;  // column; key position a - 1
+        for (int index = lane; index < 16 * kWindowTiles; index += kWave) {
+          const int a = a_first - 64 + index;  // window column; key position a - 1
           key_tile[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
         }
         __syncthreads();
 
-        const int columns = kChunk + kWave - 1;  // a = a_first - 63 + c
-        if (want_v) {
-          for (int out = lane; out < columns * DVP; out += kWave) {
-            const int c = out / DVP;
-            const int d = out - c * DVP;
-            const int a = a_first - 63 + c;
-            if (a < 1) continue;
-            // pair (row r, column a) sits in lane l = 63 - c + r
-            const int r_low = max(0, c - 63);
-            const int r_high = min(kChunk - 1, c);
-            float total = 0.0f;
-            for (int r = r_low; r <= r_high; ++r) {
-              total = fmaf(weight_tile[r * kWave + (63 - c + r)], grad_tile[r * DVP + d], total);
+        // column sums: tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
+        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r]
+        if (want_v || want_k) {
+#pragma unroll
+          for (int step = 0; step < kChunk / 4; ++step) {
+            const int r = 4 * step + lg;
+            float grad_b[VT];
+            float query_b[DT];
+#pragma unroll
+            for (int n = 0; n < VT; ++n) grad_b[n] = grad_tile[r * GP + 16 * n + li];
+            const uint32_t q_word = query_tile[r];
+#pragma unroll
+            for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
+#pragma unroll
+            for (int m = 0; m < kWindowTiles; ++m) {
+              const int offset = r * kTilePitch + 16 + 64 - (16 * m + li) + r;
+              if (want_v) {
+                const float a_value = weight_tile[offset];
+#pragma unroll
+                for (int n = 0; n < VT; ++n) {
+                  value_acc[m][n] = mfma_16x16x4(a_value, grad_b[n], value_acc[m][n]);
+                }
+              }
+              if (want_k) {
+                const float a_value = adjoint_tile[offset];
+#pragma unroll
+                for (int n = 0; n < DT; ++n) {
+                  key_acc[m][n] = mfma_16x16x4(a_value, query_b[n], key_acc[m][n]);
+                }
+              }
             }
-            value_acc[(a & (kColumnRing - 1)) * DVP + d] += total;
           }
         }
-        if (want_k) {
-          for (int out = lane; out < columns * D; out += kWave) {
-            const int c = out / D;
-            const int bit = out - c * D;
-            const int a = a_first - 63 + c;
-            if (a < 1) continue;
-            const int r_low = max(0, c - 63);
-            const int r_high = min(kChunk - 1, c);
-            float total = 0.0f;
-            for (int r = r_low; r <= r_high; ++r) {
-              const float h = adjoint_tile[r * kWave + (63 - c + r)];
-              total += ((query_tile[r] >> bit) & 1u) ? h : -h;
-            }
-            key_acc[(a & (kColumnRing - 1)) * D + bit] += total;
-          }
-        }
+        // row sums: rows are complete for this band after the chunk
         if (want_q) {
-          for (int out = lane; out < kChunk * D; out += kWave) {
-            const int r = out / D;
-            const int bit = out - r * D;
-            if (r >= rows) continue;
-            float total = 0.0f;
-            for (int l = 0; l < kWave; ++l) {
-              const float h = adjoint_tile[r * kWave + l];
-              total += ((key_tile[63 + r - l] >> bit) & 1u) ? h : -h;
-            }
-            const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
-            atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit], symbol_scale * total);
-          }
-        }
-        __syncthreads();
-        // columns a_first .. a_first + rows - 1 are complete for this band
-        if (want_v) {
-          for (int out = lane; out < rows * DVP; out += kWave) {
-            const int c = out / DVP;
-            const int d = out - c * DVP;
-            const int a = a_first + c;
-            float* slot = &value_acc[(a & (kColumnRing - 1)) * DVP + d];
-            const float total = *slot;
-            *slot = 0.0f;
-            if (d < Dv && total != 0.0f) {
-              const int64_t token = static_cast<int64_t>(u.start) + a;
-              atomicAdd(&P.grad_value[(token * P.L.Hv + hv) * Dv + d], total);
+          v4f query_acc[DT];
+#pragma unroll
+          for (int n = 0; n < DT; ++n) query_acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int step = 0; step < 4 * kWindowTiles; ++step) {
+            const int c = 4 * step + lg;
+            const float a_value = adjoint_tile[li * kTilePitch + 16 + 64 - c + li];
+            const uint32_t k_word = key_tile[c];
+#pragma unroll
+            for (int n = 0; n < DT; ++n) {
+              query_acc[n] =
+                  mfma_16x16x4(a_value, sign_of_bit(k_word, 16 * n + li, D), query_acc[n]);
             }
           }
-        }
-        if (want_k) {
-          for (int out = lane; out < rows * D; out += kWave) {
-            const int c = out / D;
-            const int bit = out - c * D;
-            const int a = a_first + c;
-            float* slot = &key_acc[(a & (kColumnRing - 1)) * D + bit];
-            const float total = *slot;
-            *slot = 0.0f;
-            if (total != 0.0f) {
-              const int64_t token = static_cast<int64_t>(u.start) + a - 1;
-              atomicAdd(&P.grad_key[(token * P.L.H + u.head) * D + bit], symbol_scale * total);
+#pragma unroll
+          for (int n = 0; n < DT; ++n) {
+            const int bit = 16 * n + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * lg + e;
+              if (bit < D && r < rows) {
+                const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
+                atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit],
+                          symbol_scale * query_acc[n][e]);
+              }
             }
           }
         }
+        // the last window tile (columns a_first .. a_first + 15) is complete: flush it,
+        // then shift the window up by one tile
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int a = a_first + 4 * lg + e;
+          if (a <= view.len - 1) {
+            const int64_t token = static_cast<int64_t>(u.start) + a;
+            if (want_v) {
+#pragma unroll
+              for (int n = 0; n < VT; ++n) {
+                const int d = 16 * n + li;
+                if (d < Dv) {
+                  atomicAdd(&P.grad_value[(token * P.L.Hv + hv) * Dv + d],
+                            value_acc[kWindowTiles - 1][n][e]);
+                }
+              }
+            }
+            if (want_k) {
+#pragma unroll
+              for (int n = 0; n < DT; ++n) {
+                const int bit = 16 * n + li;
+                if (bit < D) {
+                  atomicAdd(&P.grad_key[((token - 1) * P.L.H + u.head) * D + bit],
+                            symbol_scale * key_acc[kWindowTiles - 1][n][e]);
+                }
+              }
+            }
+          }
+        }
+#pragma unroll
+        for (int m = kWindowTiles - 1; m > 0; --m) {
+#pragma unroll
+          for (int n = 0; n < VT; ++n) value_acc[m][n] = value_acc[m - 1][n];
+#pragma unroll
+          for (int n = 0; n < DT; ++n) key_acc[m][n] = key_acc[m - 1][n];
+        }
+#pragma unroll
+        for (int n = 0; n < VT; ++n) value_acc[0][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int n = 0; n < DT; ++n) key_acc[0][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         __syncthreads();
       }
     }
@@ -1335,7 +1401,7 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   return 0;
 }
 
-template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
+template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
                       hipStream_t stream) {
   const unsigned units = static_cast<unsigned>(P.total_units);
@@ -1348,30 +1414,38 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
                      0, stream, P);
   stage_end(kStageRowStats, stream);
-  const size_t lds_floats = 2 * kSegChunks * kWave + 2 * kChunk * kWave + kChunk * DVP +
-                            (kChunk + kWave) + kChunk + kColumnRing * DVP +
-                            kColumnRing * static_cast<size_t>(P.L.D);
+  constexpr int GP = ((DVP + 15) / 16) * 16;
+  const size_t lds_floats = 2 * kSegChunks * kWave + 2 * kChunk * kTilePitch + kChunk * GP +
+                            16 * kWindowTiles + kChunk;
   const hipError_t attribute = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
+      reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
   if (attribute != hipSuccess) return fail_hip(attribute, "gradient kernel LDS size");
   stage_begin(kStageGradients, stream);
-  hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, VARLEN, DROPOUT>),
+  hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
                      dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave),
                      lds_floats * sizeof(float), stream, P);
   stage_end(kStageGradients, stream);
   return 0;
 }
 
+template <int NVW, int DVP, int DT>
+int dispatch_vjp_layout(const VjpParams& P, const VjpWorkspace& w, bool analytic, bool dropout,
+                        hipStream_t stream) {
+  if (P.L.varlen) {
+    return dropout ? launch_vjp_passes<NVW, DVP, DT, true, true>(P, w, analytic, stream)
+                   : launch_vjp_passes<NVW, DVP, DT, true, false>(P, w, analytic, stream);
+  }
+  return dropout ? launch_vjp_passes<NVW, DVP, DT, false, true>(P, w, analytic, stream)
+                 : launch_vjp_passes<NVW, DVP, DT, false, false>(P, w, analytic, stream);
+}
+
 template <int NVW, int DVP>
 int dispatch_vjp(const VjpParams& P, const VjpWorkspace& w, bool analytic, bool dropout,
                  hipStream_t stream) {
-  if (P.L.varlen) {
-    return dropout ? launch_vjp_passes<NVW, DVP, true, true>(P, w, analytic, stream)
-                   : launch_vjp_passes<NVW, DVP, true, false>(P, w, analytic, stream);
-  }
-  return dropout ? launch_vjp_passes<NVW, DVP, false, true>(P, w, analytic, stream)
-                 : launch_vjp_passes<NVW, DVP, false, false>(P, w, analytic, stream);
+  // symbol widths above 16 need two MFMA column tiles
+  return P.L.D > 16 ? dispatch_vjp_layout<NVW, DVP, 2>(P, w, analytic, dropout, stream)
+                    : dispatch_vjp_layout<NVW, DVP, 1>(P, w, analytic, dropout, stream);
 }
 
 // the analytic exponent reference is safe while it stays within 2^80 of the null weight
