@@ -38,8 +38,6 @@ constexpr float kSqrtScale = 2.414213562373095f;  // sqrt(2) + 1
 constexpr float kLog2e = 1.4426950408889634f;
 
 constexpr int kChunk = 16;     // rows kept in registers between the forward and reverse sweeps
-constexpr int kSegment = 128;  // rows between two checkpoints kept in LDS
-constexpr int kSegChunks = kSegment / kChunk;
 
 thread_local char g_error[512] = "";
 
@@ -633,36 +631,100 @@ __device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& vi
   }
 }
 
+// Everything a step needs that depends on the row only is staged in LDS for a
+// whole block of rows with one coalesced round trip (lane = row), so that the
+// recurrences themselves never wait on memory: a step reads its row with
+// wave-uniform LDS loads.  Staged words per row:
+//   0 query word of row t          1 query word of row t - W - 1
+//   2 key word entering at lane 0  3 key word of column a0 - W - 1 entering at lane 0
+//   4,5 value sign words entering  6 exponent shift of the row   7 sum of grad_output[t]
+//   8 1 / softmax denominator      9 expected dropped utility
+constexpr int kRowWords = 12;
+enum RowDetail { kRowSymbols = 0, kRowStats = 1, kRowFull = 2 };
+
+template <int NVW, int DETAIL>
+__device__ __forceinline__ void stage_rows(const BandView& view, int first, int count, int lane,
+                                           uint32_t* rows, int W, float null_logit) {
+  for (int index = lane; index < count; index += kWave) {
+    const int i = min(first + index, view.steps - 1);  // rows past the band's end repeat the last
+    const int t = view.diag0 + 1 + i;
+    const int a0 = i + 1;
+    uint4 symbols, extra, stats;
+    symbols.x = view.q[t];
+    symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+    symbols.z = view.k[a0 - 1];
+    symbols.w = (a0 - W - 2 >= 0) ? view.k[a0 - W - 2] : 0u;
+    extra.x = view.vbits[static_cast<int64_t>(a0) * NVW];
+    extra.y = NVW > 1 ? view.vbits[static_cast<int64_t>(a0) * NVW + (NVW - 1)] : 0u;
+    extra.z = 0u;
+    extra.w = 0u;
+    stats = make_uint4(0u, 0u, 0u, 0u);
+    if constexpr (DETAIL >= kRowStats) {
+      const float4 row = view.stats[t];
+      extra.z = __float_as_uint(fmaf(row.x, kLog2e, row.w));
+      extra.w = __float_as_uint(view.grad_sum[t]);
+      if constexpr (DETAIL == kRowFull) {
+        const float null_weight = fast_exp2((null_logit - row.x) * kLog2e);
+        const float inv_denominator = fast_rcp(row.y + null_weight);
+        stats.x = __float_as_uint(inv_denominator);
+        stats.y = __float_as_uint(row.z * inv_denominator);
+      }
+    }
+    uint4* dst = reinterpret_cast<uint4*>(rows + index * kRowWords);
+    dst[0] = symbols;
+    dst[1] = extra;
+    if constexpr (DETAIL == kRowFull) dst[2] = stats;
+  }
+}
+
+// grad_output rows of a block, zero for rows past the band's end; `pitch` floats per row
+template <int DVP>
+__device__ __forceinline__ void stage_grad_rows(const BandView& view, int first, int count,
+                                                int lane, float* dst, int pitch) {
+  constexpr int kQuads = DVP / 4;
+  for (int index = lane; index < count * kQuads; index += kWave) {
+    const int r = index / kQuads;
+    const int quad = index - r * kQuads;
+    const int i = first + r;
+    float4 value = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (i < view.steps) {
+      const int t = view.diag0 + 1 + i;
+      value = *reinterpret_cast<const float4*>(view.grad_rows + static_cast<int64_t>(t) * DVP +
+                                               4 * quad);
+    }
+    *reinterpret_cast<float4*>(dst + r * pitch + 4 * quad) = value;
+  }
+}
+
 struct StepOut {
   float gate;     // local match gate of this pair
   float overflow; // product of the W+1 gates ending here (0 while the window is not full)
   float evidence; // S(t, a)
+  float shift;    // exponent shift of the row (staged)
+  float grad_sum; // sum of grad_output[t] (staged)
   bool active;    // a >= 1
   int a;
 };
 
 // One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
+// `row` points at the staged words of the step's row (wave-uniform address).
 template <int NVW>
-__device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const BandView& view, int i,
+__device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const uint32_t* row, int i,
                                                 int lane, int W, float gate_log2) {
-  const int t = view.diag0 + 1 + i;
+  const uint4 symbols = *reinterpret_cast<const uint4*>(row);
+  const uint4 extra = *reinterpret_cast<const uint4*>(row + 4);
   const int a0 = i + 1;
-  const uint32_t q_word = view.q[t];
-  const uint32_t q_old = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
-  const uint32_t k_new = view.k[a0 - 1];
-  const uint32_t k_old_new = (a0 - W - 2 >= 0) ? view.k[a0 - W - 2] : 0u;
-  band.key_word = dpp_wave_shr1(k_new, band.key_word);
-  band.old_key_word = dpp_wave_shr1(k_old_new, band.old_key_word);
-#pragma unroll
-  for (int w = 0; w < NVW; ++w) {
-    const uint32_t v_new = view.vbits[static_cast<int64_t>(a0) * NVW + w];
-    band.value_bits[w] = dpp_wave_shr1(v_new, band.value_bits[w]);
-  }
+  band.key_word = dpp_wave_shr1(symbols.z, band.key_word);
+  band.old_key_word = dpp_wave_shr1(symbols.w, band.old_key_word);
+  band.value_bits[0] = dpp_wave_shr1(extra.x, band.value_bits[0]);
+  if constexpr (NVW > 1) band.value_bits[NVW - 1] = dpp_wave_shr1(extra.y, band.value_bits[NVW - 1]);
   StepOut out;
+  out.shift = __uint_as_float(extra.z);
+  out.grad_sum = __uint_as_float(extra.w);
   out.a = a0 - lane;
   out.active = out.a >= 1;
-  const int mismatches = __popc(q_word ^ band.key_word);
-  const int leaving = (out.a >= W + 2) ? __popc(q_old ^ band.old_key_word) : 0;
+  const int mismatches = __popc(symbols.x ^ band.key_word);
+  const int leaving = (out.a >= W + 2) ? __popc(symbols.y ^ band.old_key_word) : 0;
   band.window = out.active ? band.window + mismatches - leaving : 0;
   out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
   out.overflow =
@@ -679,9 +741,15 @@ __device__ __forceinline__ float route_utility(const Band<NVW>& band, const floa
   // u = sum_d go[d] * sign_d = 2 * sum_{d: bit set} go[d] - sum_d go[d]
   float picked = 0.0f;
 #pragma unroll
-  for (int d = 0; d < DVP; ++d) {
-    const int mask = static_cast<int>(band.value_bits[d >> 5] << (31 - (d & 31))) >> 31;
-    picked += __int_as_float(__float_as_int(grad_row[d]) & mask);
+  for (int q4 = 0; q4 < DVP / 4; ++q4) {
+    const float4 g = *reinterpret_cast<const float4*>(grad_row + 4 * q4);  // wave-uniform LDS read
+    const float parts[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int d = 4 * q4 + e;
+      const int mask = static_cast<int>(band.value_bits[d >> 5] << (31 - (d & 31))) >> 31;
+      picked += __int_as_float(__float_as_int(parts[e]) & mask);
+    }
   }
   return fmaf(2.0f, picked, -grad_sum);
 }
@@ -710,6 +778,7 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
 // exponent reference): raises stats[t].x to the largest logit of the row.
 template <int NVW, bool VARLEN>
 __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
+  __shared__ __attribute__((aligned(16))) uint32_t rows[kWave * kRowWords];
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -721,16 +790,22 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
   band.evidence = 0.0f;
   band.window = 0;
   load_sliding<NVW>(band, view, 0, lane, W);
-  for (int i = 0; i < view.steps; ++i) {
-    const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
-    const int t = view.diag0 + 1 + i;
-    const float root = sqrtf(1.0f + s.evidence);
-    const float logit =
-        P.scale * kSqrtScale * (root - 1.0f) - logf(static_cast<float>(t));
-    float best = s.active ? fmaxf(logit, 0.0f) : 0.0f;
-    best = wave_max_lane63(best);
-    if (lane == 63) {
-      atomicMax(reinterpret_cast<int*>(&view.stats[t].x), __float_as_int(best));
+  for (int first = 0; first < view.steps; first += kWave) {
+    const int count = min(kWave, view.steps - first);
+    __syncthreads();
+    stage_rows<NVW, kRowSymbols>(view, first, count, lane, rows, W, P.null_logit);
+    __syncthreads();
+    for (int r = 0; r < count; ++r) {
+      const int i = first + r;
+      const StepOut s = forward_step<NVW>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
+      const int t = view.diag0 + 1 + i;
+      const float root = sqrtf(1.0f + s.evidence);
+      const float logit = P.scale * kSqrtScale * (root - 1.0f) - logf(static_cast<float>(t));
+      float best = s.active ? fmaxf(logit, 0.0f) : 0.0f;
+      best = wave_max_lane63(best);
+      if (lane == 63) {
+        atomicMax(reinterpret_cast<int*>(&view.stats[t].x), __float_as_int(best));
+      }
     }
   }
 }
@@ -738,6 +813,8 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
 // Row-statistics pass: denominator and expected dropped utility of every row.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
+  __shared__ __attribute__((aligned(16))) uint32_t rows[kWave * kRowWords];
+  __shared__ __attribute__((aligned(16))) float grads[kWave * DVP];
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -758,31 +835,35 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   band.window = 0;
   load_sliding<NVW>(band, view, 0, lane, W);
   const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
-  for (int i = 0; i < view.steps; ++i) {
-    const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
-    const int t = view.diag0 + 1 + i;
-    const float4 row = view.stats[t];
-    const float shift = fmaf(row.x, kLog2e, row.w);
-    const float one_plus = 1.0f + s.evidence;
-    const float root = one_plus * fast_rsq(one_plus);
-    const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
-    float numerator = 0.0f;
-    if (needs_utility) {
-      const float utility =
-          route_utility<NVW, DVP>(band, view.grad_rows + static_cast<int64_t>(t) * DVP,
-                                  view.grad_sum[t]);
-      float keep = 1.0f;
-      if constexpr (DROPOUT) {
-        key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-        keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
+  for (int first = 0; first < view.steps; first += kWave) {
+    const int count = min(kWave, view.steps - first);
+    __syncthreads();
+    stage_rows<NVW, kRowStats>(view, first, count, lane, rows, W, P.null_logit);
+    if (needs_utility) stage_grad_rows<DVP>(view, first, count, lane, grads, DVP);
+    __syncthreads();
+    for (int r = 0; r < count; ++r) {
+      const int i = first + r;
+      const int t = view.diag0 + 1 + i;
+      const StepOut s = forward_step<NVW>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
+      const float one_plus = 1.0f + s.evidence;
+      const float root = one_plus * fast_rsq(one_plus);
+      const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
+      float numerator = 0.0f;
+      if (needs_utility) {
+        const float utility = route_utility<NVW, DVP>(band, grads + r * DVP, s.grad_sum);
+        float keep = 1.0f;
+        if constexpr (DROPOUT) {
+          key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+          keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
+        }
+        numerator = weight * keep * utility;
       }
-      numerator = weight * keep * utility;
-    }
-    const float weight_sum = wave_sum_lane63(weight);
-    const float numerator_sum = wave_sum_lane63(numerator);
-    if (lane == 63) {
-      atomicAdd(&view.stats[t].y, weight_sum);
-      if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
+      const float weight_sum = wave_sum_lane63(weight);
+      const float numerator_sum = wave_sum_lane63(numerator);
+      if (lane == 63) {
+        atomicAdd(&view.stats[t].y, weight_sum);
+        if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
+      }
     }
   }
 }
@@ -793,7 +874,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
 //   b(n) = A(n) + gate(n+1) b(n+1)
 // needs the adjoints of later rows, while S needs earlier rows.  S is
 // therefore rebuilt from checkpoints: one cheap forward sweep per band stores
-// (S, window) every kSegment rows, one per segment stores them every kChunk
+// (S, window) once per LDS-staged segment, one per segment stores them every kChunk
 // rows in LDS, and each chunk is then replayed forward into registers and
 // walked backwards.  The windowed sum of b*overflow lives in a ring of W+1
 // rows in global memory that is touched only while some overflow term of the
@@ -833,20 +914,25 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
   return 2;
 }
 
+// rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
+constexpr int gradient_segment(int dvp) { return dvp >= 64 ? 32 : 64; }
+
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr int GP = VT * 16;           // pitch of the staged grad_output rows
+  constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
+  constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds[];
-  float* ck_evidence = lds;                                  // [kSegChunks][64]
-  int* ck_window = reinterpret_cast<int*>(lds + kSegChunks * kWave);
-  float* weight_tile = lds + 2 * kSegChunks * kWave;         // [kChunk][kTilePitch]
+  float* ck_evidence = lds;                                  // [SEG_CHUNKS][64]
+  int* ck_window = reinterpret_cast<int*>(lds + SEG_CHUNKS * kWave);
+  float* weight_tile = lds + 2 * SEG_CHUNKS * kWave;         // [kChunk][kTilePitch]
   float* adjoint_tile = weight_tile + kChunk * kTilePitch;   // [kChunk][kTilePitch]
-  float* grad_tile = adjoint_tile + kChunk * kTilePitch;     // [kChunk][GP]
-  uint32_t* key_tile = reinterpret_cast<uint32_t*>(grad_tile + kChunk * GP);  // [80]
-  uint32_t* query_tile = key_tile + 16 * kWindowTiles;       // [kChunk]
+  float* grad_rows_lds = adjoint_tile + kChunk * kTilePitch; // [SEG][GP]
+  uint32_t* rows = reinterpret_cast<uint32_t*>(grad_rows_lds + SEG * GP);  // [SEG][kRowWords]
+  uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -863,7 +949,7 @@ void vjp_gradients_kernel(VjpParams P) {
   float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
 
   // zero the tiles once: the margins are never written again
-  for (int index = lane; index < 2 * kChunk * kTilePitch + kChunk * GP; index += kWave) {
+  for (int index = lane; index < 2 * kChunk * kTilePitch + SEG * GP; index += kWave) {
     weight_tile[index] = 0.0f;
   }
   __syncthreads();
@@ -898,7 +984,7 @@ void vjp_gradients_kernel(VjpParams P) {
       for (int n = 0; n < DT; ++n) key_acc[m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    const int segments = (view.steps + kSegment - 1) / kSegment;
+    const int segments = (view.steps + SEG - 1) / SEG;
     Band<NVW> band;
     // band-level forward sweep: checkpoint (S, window) before the first row of every segment
     if (segments > 1) {
@@ -908,10 +994,13 @@ void vjp_gradients_kernel(VjpParams P) {
       for (int segment = 0; segment < segments - 1; ++segment) {
         seg_ck[(2 * segment) * kWave + lane] = band.evidence;
         seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
-        const int first = segment * kSegment;
+        const int first = segment * SEG;
+        __syncthreads();
+        stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W, P.null_logit);
+        __syncthreads();
 #pragma unroll 4
-        for (int r = 0; r < kSegment; ++r) {
-          forward_step<NVW>(band, view, first + r, lane, W, P.gate_log2);
+        for (int r = 0; r < SEG; ++r) {
+          forward_step<NVW>(band, rows + r * kRowWords, first + r, lane, W, P.gate_log2);
         }
       }
       const int segment = segments - 1;
@@ -928,8 +1017,8 @@ void vjp_gradients_kernel(VjpParams P) {
     const int last_step = view.steps - 1;
 
     for (int segment = segments - 1; segment >= 0; --segment) {
-      const int seg_first = segment * kSegment;
-      const int seg_last = min(view.steps, seg_first + kSegment);
+      const int seg_first = segment * SEG;
+      const int seg_last = min(view.steps, seg_first + SEG);
       if (segments > 1) {
         band.evidence = seg_ck[(2 * segment) * kWave + lane];
         band.window = __float_as_int(seg_ck[(2 * segment + 1) * kWave + lane]);
@@ -938,26 +1027,38 @@ void vjp_gradients_kernel(VjpParams P) {
         band.window = 0;
       }
       load_sliding<NVW>(band, view, seg_first, lane, W);
+      // one round trip brings in everything the segment needs
+      __syncthreads();
+      stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W, P.null_logit);
+      stage_grad_rows<DVP>(view, seg_first, SEG, lane, grad_rows_lds, GP);
+      for (int index = lane; index < SEG + kWave; index += kWave) {
+        const int a = seg_first - 63 + index;  // column; key position a - 1
+        key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
+      }
+      __syncthreads();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
       // segment-level forward sweep: checkpoint before every chunk
       for (int chunk = 0; chunk < chunks; ++chunk) {
         ck_evidence[chunk * kWave + lane] = band.evidence;
         ck_window[chunk * kWave + lane] = band.window;
         if (chunk + 1 < chunks) {
-          const int first = seg_first + chunk * kChunk;
+          const int local = chunk * kChunk;
 #pragma unroll 4
           for (int r = 0; r < kChunk; ++r) {
-            forward_step<NVW>(band, view, first + r, lane, W, P.gate_log2);
+            forward_step<NVW>(band, rows + (local + r) * kRowWords, seg_first + local + r, lane, W,
+                              P.gate_log2);
           }
         }
       }
 
       for (int chunk = chunks - 1; chunk >= 0; --chunk) {
-        const int first = seg_first + chunk * kChunk;   // step index of the chunk's first row
-        const int rows = min(kChunk, seg_last - first); // < kChunk only for the band's last rows
+        const int local = chunk * kChunk;               // first row of the chunk inside the segment
+        const int first = seg_first + local;            // step index of the chunk's first row
+        const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
         band.evidence = ck_evidence[chunk * kWave + lane];
         band.window = ck_window[chunk * kWave + lane];
         load_sliding<NVW>(band, view, first, lane, W);
+        const float* grad_tile = grad_rows_lds + local * GP;
 
         float keep_evidence[kChunk];  // S + overflow
         float keep_overflow[kChunk];
@@ -965,23 +1066,22 @@ void vjp_gradients_kernel(VjpParams P) {
         float keep_adjoint[kChunk];   // external adjoint A of the route score
 
         // Forward replay of the chunk.  Rows past the end of the band (only in
-        // the band's last chunk) are computed on the clamped last row and
-        // masked, which keeps the loop free of branches.
+        // the band's last chunk) repeat the last row's data and are masked,
+        // which keeps the loop free of branches.
 #pragma unroll
         for (int r = 0; r < kChunk; ++r) {
-          const bool row_ok = r < rows;
+          const bool row_ok = r < rows_here;
           const int i = min(first + r, last_step);
           const int t = view.diag0 + 1 + i;
-          const StepOut s = forward_step<NVW>(band, view, i, lane, W, P.gate_log2);
-          const float4 row = view.stats[t];
-          const float shift = fmaf(row.x, kLog2e, row.w);
+          const uint32_t* row = rows + (local + r) * kRowWords;
+          const StepOut s = forward_step<NVW>(band, row, i, lane, W, P.gate_log2);
+          const float inv_denominator = __uint_as_float(row[8]);
+          const float expected = __uint_as_float(row[9]);
           const float one_plus = 1.0f + s.evidence;
           const float inv_root = fast_rsq(one_plus);
           const float root = one_plus * inv_root;
           const bool live = s.active && row_ok;
-          const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
-          const float null_weight = fast_exp2((P.null_logit - row.x) * kLog2e);
-          const float inv_denominator = fast_rcp(row.y + null_weight);
+          const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
           const float probability = weight * inv_denominator;
           float keep = 1.0f;
           if constexpr (DROPOUT) {
@@ -991,9 +1091,7 @@ void vjp_gradients_kernel(VjpParams P) {
           weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
           float adjoint = 0.0f;
           if (want_qk) {
-            const float utility = route_utility<NVW, DVP>(
-                band, view.grad_rows + static_cast<int64_t>(t) * DVP, view.grad_sum[t]);
-            const float expected = row.z * inv_denominator;
+            const float utility = route_utility<NVW, DVP>(band, grad_tile + r * GP, s.grad_sum);
             adjoint = P.scale * probability * (keep * utility - expected) *
                       (0.5f * kSqrtScale * inv_root);
           }
@@ -1034,27 +1132,14 @@ void vjp_gradients_kernel(VjpParams P) {
             }
             const float h = fmaf(b, keep_evidence[r], -ring_sum);
             if (ring_live == 0) ring_sum = 0.0f;
-            const bool active = (i + 1 - lane) >= 1 && r < rows;
+            const bool active = (i + 1 - lane) >= 1 && r < rows_here;
             adjoint_tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
           }
         }
 
-        // stage the row and column data of the chunk
         const int t_first = view.diag0 + 1 + first;
         const int a_first = first + 1;  // column of lane 0 in the chunk's first row
-        if (want_v) {
-          for (int index = lane; index < kChunk * DVP; index += kWave) {
-            const int r = index / DVP;
-            const int d = index - r * DVP;
-            grad_tile[r * GP + d] =
-                r < rows ? view.grad_rows[static_cast<int64_t>(t_first + r) * DVP + d] : 0.0f;
-          }
-        }
-        if (lane < kChunk) query_tile[lane] = lane < rows ? view.q[t_first + lane] : 0u;
-        for (int index = lane; index < 16 * kWindowTiles; index += kWave) {
-          const int a = a_first - 64 + index;  // window column; key position a - 1
-          key_tile[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
-        }
+        const uint32_t* key_tile = key_window + local;  // window column c <-> a = a_first - 64 + c
         __syncthreads();
 
         // column sums: tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
@@ -1067,7 +1152,7 @@ void vjp_gradients_kernel(VjpParams P) {
             float query_b[DT];
 #pragma unroll
             for (int n = 0; n < VT; ++n) grad_b[n] = grad_tile[r * GP + 16 * n + li];
-            const uint32_t q_word = query_tile[r];
+            const uint32_t q_word = r < rows_here ? rows[(local + r) * kRowWords] : 0u;
 #pragma unroll
             for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
 #pragma unroll
@@ -1112,7 +1197,7 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int r = 4 * lg + e;
-              if (bit < D && r < rows) {
+              if (bit < D && r < rows_here) {
                 const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
                 atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit],
                           symbol_scale * query_acc[n][e]);
@@ -1307,13 +1392,14 @@ VjpWorkspace carve_vjp(const ProblemView& v) {
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
-  const int max_segments = (longest + kSegment - 1) / kSegment + 1;
+  const int segment_rows = gradient_segment(dvp);
+  const int max_segments = (longest + segment_rows - 1) / segment_rows + 1;
   w.block_scratch_floats =
       static_cast<int64_t>(w.ring_rows) * kWave + static_cast<int64_t>(max_segments) * 2 * kWave;
   const int64_t units = static_cast<int64_t>(v.L.slots) * v.L.H;
   w.resident_blocks = static_cast<int>(std::min<int64_t>(units, kMaxResidentBlocks));
-  // keep the ring pool below 1 GiB by running fewer resident blocks for huge windows
-  const int64_t budget_floats = (int64_t(1) << 30) / 4;
+  // keep the scratch pool below 2 GiB by running fewer resident blocks for huge windows
+  const int64_t budget_floats = (int64_t(1) << 31) / 4;
   while (w.resident_blocks > 64 &&
          static_cast<int64_t>(w.resident_blocks) * w.block_scratch_floats > budget_floats) {
     w.resident_blocks /= 2;
@@ -1415,8 +1501,9 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
                      0, stream, P);
   stage_end(kStageRowStats, stream);
   constexpr int GP = ((DVP + 15) / 16) * 16;
-  const size_t lds_floats = 2 * kSegChunks * kWave + 2 * kChunk * kTilePitch + kChunk * GP +
-                            16 * kWindowTiles + kChunk;
+  constexpr int SEG = gradient_segment(DVP);
+  const size_t lds_floats = 2 * (SEG / kChunk) * kWave + 2 * kChunk * kTilePitch + SEG * GP +
+                            SEG * kRowWords + SEG + kWave;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
