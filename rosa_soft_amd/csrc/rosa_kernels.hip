@@ -177,9 +177,15 @@ struct DropoutKey {
   uint32_t seed_high_salt;  // seed_high ^ 0x9e3779b9
 };
 
-__device__ __forceinline__ float dropout_multiplier(const DropoutKey& key, int route,
+// first hash round: depends on the route only, so a band computes it once per
+// column (for the column entering at lane 0) and slides it with the columns
+__device__ __forceinline__ uint32_t route_hash_of(int route) {
+  return mix32(static_cast<uint32_t>(route) ^ 0x68e31da4u);
+}
+
+__device__ __forceinline__ float dropout_multiplier(const DropoutKey& key, uint32_t route_hash,
                                                     float dropout_p, float inverse_keep) {
-  uint32_t s = mix32(static_cast<uint32_t>(route) ^ 0x68e31da4u);
+  uint32_t s = route_hash;
   s = mix32(s ^ key.row_salt);
   s = mix32(s ^ key.head_salt);
   s = mix32(s ^ key.batch_salt);
@@ -200,8 +206,21 @@ struct Layout {
   const int32_t* seq_start;
   const int32_t* seq_len;
   const int32_t* block_prefix;  // [S+1] prefix sums of ceil(len / 64)
+  const int64_t* step_prefix;   // [S+1] prefix sums of band_steps_total(len)
   int slots;                    // number of 64-row block slots over all sequences (upper bound)
 };
+
+// number of (row, band) steps of one (sequence, head) of length `len`, and the
+// number that precede band j: the index space of the cached keep masks
+__host__ __device__ inline int64_t band_steps_total(int len) {
+  if (len < 2) return 0;
+  const int64_t bands = (len - 2) / 64 + 1;
+  return bands * (len - 1) - 32 * bands * (bands - 1);
+}
+
+__host__ __device__ inline int64_t band_steps_before(int len, int band) {
+  return static_cast<int64_t>(band) * (len - 1) - 32 * static_cast<int64_t>(band) * (band - 1);
+}
 
 struct Unit {
   int seq;     // batch index (dense) or packed sequence index
@@ -254,6 +273,8 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
                                          int32_t* __restrict__ seq_start,
                                          int32_t* __restrict__ seq_len,
                                          int32_t* __restrict__ block_prefix,
+                                         int64_t* __restrict__ step_prefix, int H,
+                                         int64_t mask_capacity,
                                          int32_t* __restrict__ header) {
   // single block; offsets are clamped into [previous, N] so that no later
   // kernel can index outside the tensors, and any violation is recorded.
@@ -292,6 +313,17 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
     }
     block_prefix[S] = running;
     header[0] = bad;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && step_prefix != nullptr) {
+    // index space of the cached keep masks; they are used only if they fit
+    int64_t steps = 0;
+    for (int s = 0; s < S; ++s) {
+      step_prefix[s] = steps;
+      steps += band_steps_total(seq_len[s]);
+    }
+    step_prefix[S] = steps;
+    header[2] = steps * H <= mask_capacity ? 1 : 0;
   }
   __syncthreads();
   int running = partial[threadIdx.x];
@@ -494,6 +526,8 @@ struct VjpParams {
   float* grad_key;
   float* grad_value;
   int32_t* work_counter;
+  const int32_t* header;        // [0] offsets flag, [1] work counter, [2] keep masks fit
+  unsigned long long* keep_masks;  // one 64-lane keep ballot per (band, row) step, or NULL
   float* block_scratch;         // per resident block: ring + segment checkpoints
   int64_t block_scratch_floats;
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
@@ -613,6 +647,7 @@ struct BandView {
   const float* grad_rows;  // [t][dvp]
   const float* grad_sum;   // [t]
   float4* stats;           // [t]
+  const unsigned long long* masks;  // cached keep ballots of this band (step i), or NULL
   int len;
   int diag0;               // first diagonal of the band
   int steps;               // rows of the band: t = diag0 + 1 + i
@@ -668,6 +703,11 @@ __device__ __forceinline__ void stage_rows(const BandView& view, int first, int 
         const float inv_denominator = fast_rcp(row.y + null_weight);
         stats.x = __float_as_uint(inv_denominator);
         stats.y = __float_as_uint(row.z * inv_denominator);
+        if (view.masks != nullptr) {
+          const unsigned long long ballot = view.masks[i];
+          stats.z = static_cast<uint32_t>(ballot);
+          stats.w = static_cast<uint32_t>(ballot >> 32);
+        }
       }
     }
     uint4* dst = reinterpret_cast<uint4*>(rows + index * kRowWords);
@@ -771,6 +811,17 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
   view.grad_rows = P.grad_rows + u.word_base * P.dvp;
   view.grad_sum = P.grad_row_sum + u.word_base;
   view.stats = P.stats + u.word_base;
+  view.masks = nullptr;
+  if (P.keep_masks != nullptr) {
+    int64_t base;
+    if constexpr (VARLEN) {
+      base = P.L.step_prefix[u.seq] * P.L.H + u.head * band_steps_total(u.len);
+    } else {
+      base = (static_cast<int64_t>(u.seq) * P.L.H + u.head) * band_steps_total(u.len);
+    }
+    const bool fits = !VARLEN || P.header[2] != 0;
+    if (fits) view.masks = P.keep_masks + base + band_steps_before(u.len, u.block);
+  }
   return true;
 }
 
@@ -835,6 +886,8 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   band.window = 0;
   load_sliding<NVW>(band, view, 0, lane, W);
   const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
+  unsigned long long* mask_out = const_cast<unsigned long long*>(view.masks);
+  uint32_t route_hash = route_hash_of(-lane);
   for (int first = 0; first < view.steps; first += kWave) {
     const int count = min(kWave, view.steps - first);
     __syncthreads();
@@ -849,13 +902,21 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       const float root = one_plus * fast_rsq(one_plus);
       const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
       float numerator = 0.0f;
+      float keep = 1.0f;
+      if constexpr (DROPOUT) {
+        route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
+        if (needs_utility || mask_out != nullptr) {
+          key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+          keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+          if (mask_out != nullptr) {
+            // the gradient pass reads the decisions back instead of hashing again
+            const unsigned long long ballot = __ballot(keep != 0.0f);
+            if (lane == 0) mask_out[i] = ballot;
+          }
+        }
+      }
       if (needs_utility) {
         const float utility = route_utility<NVW, DVP>(band, grads + r * DVP, s.grad_sum);
-        float keep = 1.0f;
-        if constexpr (DROPOUT) {
-          key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-          keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
-        }
         numerator = weight * keep * utility;
       }
       const float weight_sum = wave_sum_lane63(weight);
@@ -1059,6 +1120,10 @@ void vjp_gradients_kernel(VjpParams P) {
         band.window = ck_window[chunk * kWave + lane];
         load_sliding<NVW>(band, view, first, lane, W);
         const float* grad_tile = grad_rows_lds + local * GP;
+        uint32_t route_hash = 0u;
+        if constexpr (DROPOUT) {
+          if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
+        }
 
         float keep_evidence[kChunk];  // S + overflow
         float keep_overflow[kChunk];
@@ -1085,8 +1150,15 @@ void vjp_gradients_kernel(VjpParams P) {
           const float probability = weight * inv_denominator;
           float keep = 1.0f;
           if constexpr (DROPOUT) {
-            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-            keep = dropout_multiplier(key, s.a, P.dropout_p, P.inverse_keep);
+            if (view.masks != nullptr) {
+              const unsigned long long ballot =
+                  (static_cast<unsigned long long>(row[11]) << 32) | row[10];
+              keep = ((ballot >> lane) & 1ull) ? P.inverse_keep : 0.0f;
+            } else {
+              route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
+              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+              keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+            }
           }
           weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
           float adjoint = 0.0f;
@@ -1366,8 +1438,9 @@ int padded_value_width(int Dv) {
 }
 
 struct VjpWorkspace {
-  size_t header, seq_start, seq_len, block_prefix, stats, grad_rows, grad_sum, value_bits,
-      block_scratch, total;
+  size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows, grad_sum,
+      value_bits, keep_masks, block_scratch, total;
+  int64_t mask_capacity;  // 64-lane keep ballots that fit in the workspace (0: none kept)
   int resident_blocks;
   int64_t block_scratch_floats;
   int ring_rows;
@@ -1375,7 +1448,7 @@ struct VjpWorkspace {
 
 constexpr int kMaxResidentBlocks = 2048;
 
-VjpWorkspace carve_vjp(const ProblemView& v) {
+VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   VjpWorkspace w;
   size_t cursor = 0;
   w.header = cursor; cursor += align_up(256);
@@ -1383,6 +1456,7 @@ VjpWorkspace carve_vjp(const ProblemView& v) {
   w.seq_start = cursor; cursor += align_up(sizeof(int32_t) * s);
   w.seq_len = cursor; cursor += align_up(sizeof(int32_t) * s);
   w.block_prefix = cursor; cursor += align_up(sizeof(int32_t) * (s + 1));
+  w.step_prefix = cursor; cursor += align_up(sizeof(int64_t) * (s + 1));
   const size_t rows = static_cast<size_t>(v.symbol_rows);
   const int dvp = padded_value_width(v.L.Dv);
   w.stats = cursor; cursor += align_up(sizeof(float) * 4 * rows);
@@ -1390,6 +1464,21 @@ VjpWorkspace carve_vjp(const ProblemView& v) {
   w.grad_sum = cursor; cursor += align_up(sizeof(float) * rows);
   w.value_bits = cursor;
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
+  // Keep decisions of the dropout hash, one 64-lane ballot per (band, row)
+  // step (1 bit per pair): written by the row-statistics pass, read back by
+  // the gradient pass.  A packed batch is sized for its worst case (a single
+  // sequence) up to a budget; the device checks whether the real batch fits
+  // and otherwise hashes again.
+  w.keep_masks = cursor;
+  w.mask_capacity = 0;
+  if (dropout) {
+    const int64_t budget = (int64_t(3) << 29) / 8;  // 1.5 GiB of ballots
+    const int64_t wanted = v.L.varlen
+        ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
+        : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
+    w.mask_capacity = v.L.varlen ? std::min(wanted, budget) : (wanted <= 2 * budget ? wanted : 0);
+    cursor += align_up(sizeof(uint64_t) * static_cast<size_t>(w.mask_capacity));
+  }
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
   const int segment_rows = gradient_segment(dvp);
@@ -1422,14 +1511,17 @@ unsigned blocks_for(int64_t items, int threads) {
 
 int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, size_t seq_start,
                              size_t seq_len, size_t block_prefix, size_t header,
-                             hipStream_t stream) {
+                             hipStream_t stream, int64_t* step_prefix = nullptr,
+                             int64_t mask_capacity = 0) {
   if (!L.varlen) return 0;
   L.seq_start = at<int32_t>(workspace, seq_start);
   L.seq_len = at<int32_t>(workspace, seq_len);
   L.block_prefix = at<int32_t>(workspace, block_prefix);
+  L.step_prefix = step_prefix;
   hipLaunchKernelGGL(prepare_sequences_kernel, dim3(1), dim3(256), 0, stream, p->cu_seqlens, L.S,
                      L.N, at<int32_t>(workspace, seq_start), at<int32_t>(workspace, seq_len),
-                     at<int32_t>(workspace, block_prefix), at<int32_t>(workspace, header));
+                     at<int32_t>(workspace, block_prefix), step_prefix, L.H, mask_capacity,
+                     at<int32_t>(workspace, header));
   return 0;
 }
 
@@ -1550,9 +1642,9 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
             float inverse_keep, float mismatch_scale, int gradient_mask, float* grad_query,
             float* grad_key, float* grad_value, void* workspace, hipStream_t stream) {
   Layout L = view.L;
-  const VjpWorkspace w = carve_vjp(view);
+  const VjpWorkspace w = carve_vjp(view, dropout_p > 0.0f);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
-                           stream);
+                           stream, at<int64_t>(workspace, w.step_prefix), w.mask_capacity);
   const int dvp = padded_value_width(L.Dv);
   const int nvw = value_words(L.Dv);
   const int64_t symbol_elements = view.symbol_rows * L.D;
@@ -1620,6 +1712,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   P.grad_key = grad_key;
   P.grad_value = grad_value;
   P.work_counter = counter;
+  P.header = at<int32_t>(workspace, w.header);
+  P.keep_masks = w.mask_capacity > 0 ? at<unsigned long long>(workspace, w.keep_masks) : nullptr;
   P.block_scratch = at<float>(workspace, w.block_scratch);
   P.block_scratch_floats = w.block_scratch_floats;
   P.ring_rows = w.ring_rows;
@@ -1670,10 +1764,9 @@ size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_ma
                                     int dropout) {
   (void)gradient_mask;
   (void)scale;
-  (void)dropout;
   ProblemView view;
   if (check_problem(problem, &view) != 0) return 0;
-  return carve_vjp(view).total;
+  return carve_vjp(view, dropout != 0).total;
 }
 
 int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const void* key,
@@ -1724,7 +1817,8 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const
     return fail(2, "surrogate_vjp: dropout_seed must be given exactly when dropout_p > 0");
   if (problem->Dv > 64)
     return fail(4, "surrogate_vjp: value dimension above 64 is not supported by this build");
-  if (workspace_bytes < carve_vjp(view).total) return fail(3, "surrogate_vjp: workspace too small");
+  if (workspace_bytes < carve_vjp(view, dropout_p > 0.0f).total)
+    return fail(3, "surrogate_vjp: workspace too small");
   if (!(gradient_mask & ROSA_GRAD_QUERY)) grad_query = nullptr;
   if (!(gradient_mask & ROSA_GRAD_KEY)) grad_key = nullptr;
   if (!(gradient_mask & ROSA_GRAD_VALUE)) grad_value = nullptr;
