@@ -748,7 +748,10 @@ struct StepOut {
 
 // One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
 // `row` points at the staged words of the step's row (wave-uniform address).
-template <int NVW>
+// STEADY: every lane of the wave is past its diagonal's first W + 1 rows, so no
+// lane needs masking (true for all but the first W + 64 rows of a band).
+// VALUES: also slide the value sign bits (not needed by evidence-only sweeps).
+template <int NVW, bool STEADY = false, bool VALUES = true>
 __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const uint32_t* row, int i,
                                                 int lane, int W, float gate_log2) {
   const uint4 symbols = *reinterpret_cast<const uint4*>(row);
@@ -756,23 +759,52 @@ __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const uint32_t*
   const int a0 = i + 1;
   band.key_word = dpp_wave_shr1(symbols.z, band.key_word);
   band.old_key_word = dpp_wave_shr1(symbols.w, band.old_key_word);
-  band.value_bits[0] = dpp_wave_shr1(extra.x, band.value_bits[0]);
-  if constexpr (NVW > 1) band.value_bits[NVW - 1] = dpp_wave_shr1(extra.y, band.value_bits[NVW - 1]);
+  if constexpr (VALUES) {
+    band.value_bits[0] = dpp_wave_shr1(extra.x, band.value_bits[0]);
+    if constexpr (NVW > 1) {
+      band.value_bits[NVW - 1] = dpp_wave_shr1(extra.y, band.value_bits[NVW - 1]);
+    }
+  }
   StepOut out;
   out.shift = __uint_as_float(extra.z);
   out.grad_sum = __uint_as_float(extra.w);
   out.a = a0 - lane;
-  out.active = out.a >= 1;
   const int mismatches = __popc(symbols.x ^ band.key_word);
-  const int leaving = (out.a >= W + 2) ? __popc(symbols.y ^ band.old_key_word) : 0;
-  band.window = out.active ? band.window + mismatches - leaving : 0;
-  out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
-  out.overflow =
-      (out.a >= W + 1) ? fast_exp2(-gate_log2 * static_cast<float>(band.window)) : 0.0f;
-  const float next = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
-  band.evidence = out.active ? next : 0.0f;
+  if constexpr (STEADY) {
+    out.active = true;
+    band.window += mismatches - __popc(symbols.y ^ band.old_key_word);
+    out.gate = fast_exp2(-gate_log2 * static_cast<float>(mismatches));
+    out.overflow = fast_exp2(-gate_log2 * static_cast<float>(band.window));
+    band.evidence = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
+  } else {
+    out.active = out.a >= 1;
+    const int leaving = (out.a >= W + 2) ? __popc(symbols.y ^ band.old_key_word) : 0;
+    band.window = out.active ? band.window + mismatches - leaving : 0;
+    out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
+    out.overflow =
+        (out.a >= W + 1) ? fast_exp2(-gate_log2 * static_cast<float>(band.window)) : 0.0f;
+    const float next = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
+    band.evidence = out.active ? next : 0.0f;
+  }
   out.evidence = band.evidence;
   return out;
+}
+
+// Evidence-only sweep over `count` staged rows starting at step `first`.
+template <int NVW>
+__device__ __forceinline__ void sweep_rows(Band<NVW>& band, const uint32_t* rows, int first,
+                                           int count, int lane, int W, float gate_log2) {
+  if (first >= W + kWave) {  // steady state: all 64 lanes are past their window fill
+#pragma unroll 4
+    for (int r = 0; r < count; ++r) {
+      forward_step<NVW, true, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+    }
+  } else {
+#pragma unroll 4
+    for (int r = 0; r < count; ++r) {
+      forward_step<NVW, false, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+    }
+  }
 }
 
 template <int NVW, int DVP>
@@ -894,37 +926,46 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
     stage_rows<NVW, kRowStats>(view, first, count, lane, rows, W, P.null_logit);
     if (needs_utility) stage_grad_rows<DVP>(view, first, count, lane, grads, DVP);
     __syncthreads();
-    for (int r = 0; r < count; ++r) {
-      const int i = first + r;
-      const int t = view.diag0 + 1 + i;
-      const StepOut s = forward_step<NVW>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
-      const float one_plus = 1.0f + s.evidence;
-      const float root = one_plus * fast_rsq(one_plus);
-      const float weight = s.active ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
-      float numerator = 0.0f;
-      float keep = 1.0f;
-      if constexpr (DROPOUT) {
-        route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-        if (needs_utility || mask_out != nullptr) {
-          key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-          keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-          if (mask_out != nullptr) {
-            // the gradient pass reads the decisions back instead of hashing again
-            const unsigned long long ballot = __ballot(keep != 0.0f);
-            if (lane == 0) mask_out[i] = ballot;
+    // compiled twice: once every lane is past its window fill no masking is needed
+    auto run_block = [&](auto steady_tag) {
+      constexpr bool STEADY = decltype(steady_tag)::value;
+      for (int r = 0; r < count; ++r) {
+        const int i = first + r;
+        const int t = view.diag0 + 1 + i;
+        const StepOut s = forward_step<NVW, STEADY, true>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
+        const float one_plus = 1.0f + s.evidence;
+        const float root = one_plus * fast_rsq(one_plus);
+        const float weight = (STEADY || s.active) ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
+        float numerator = 0.0f;
+        float keep = 1.0f;
+        if constexpr (DROPOUT) {
+          route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
+          if (needs_utility || mask_out != nullptr) {
+            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+            keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+            if (mask_out != nullptr) {
+              // the gradient pass reads the decisions back instead of hashing again
+              const unsigned long long ballot = __ballot(keep != 0.0f);
+              if (lane == 0) mask_out[i] = ballot;
+            }
           }
         }
+        if (needs_utility) {
+          const float utility = route_utility<NVW, DVP>(band, grads + r * DVP, s.grad_sum);
+          numerator = weight * keep * utility;
+        }
+        const float weight_sum = wave_sum_lane63(weight);
+        const float numerator_sum = wave_sum_lane63(numerator);
+        if (lane == 63) {
+          atomicAdd(&view.stats[t].y, weight_sum);
+          if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
+        }
       }
-      if (needs_utility) {
-        const float utility = route_utility<NVW, DVP>(band, grads + r * DVP, s.grad_sum);
-        numerator = weight * keep * utility;
-      }
-      const float weight_sum = wave_sum_lane63(weight);
-      const float numerator_sum = wave_sum_lane63(numerator);
-      if (lane == 63) {
-        atomicAdd(&view.stats[t].y, weight_sum);
-        if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
-      }
+    };
+    if (first >= W + kWave) {
+      run_block(std::true_type{});
+    } else {
+      run_block(std::false_type{});
     }
   }
 }
@@ -1059,10 +1100,7 @@ void vjp_gradients_kernel(VjpParams P) {
         __syncthreads();
         stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W, P.null_logit);
         __syncthreads();
-#pragma unroll 4
-        for (int r = 0; r < SEG; ++r) {
-          forward_step<NVW>(band, rows + r * kRowWords, first + r, lane, W, P.gate_log2);
-        }
+        sweep_rows<NVW>(band, rows, first, SEG, lane, W, P.gate_log2);
       }
       const int segment = segments - 1;
       seg_ck[(2 * segment) * kWave + lane] = band.evidence;
@@ -1104,11 +1142,8 @@ void vjp_gradients_kernel(VjpParams P) {
         ck_window[chunk * kWave + lane] = band.window;
         if (chunk + 1 < chunks) {
           const int local = chunk * kChunk;
-#pragma unroll 4
-          for (int r = 0; r < kChunk; ++r) {
-            forward_step<NVW>(band, rows + (local + r) * kRowWords, seg_first + local + r, lane, W,
-                              P.gate_log2);
-          }
+          sweep_rows<NVW>(band, rows + local * kRowWords, seg_first + local, kChunk, lane, W,
+                          P.gate_log2);
         }
       }
 
@@ -1125,88 +1160,99 @@ void vjp_gradients_kernel(VjpParams P) {
           if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
         }
 
-        float keep_evidence[kChunk];  // S + overflow
-        float keep_overflow[kChunk];
-        float keep_gate[kChunk];
-        float keep_adjoint[kChunk];   // external adjoint A of the route score
+        // The replay is compiled twice: the steady-state form (all lanes past
+        // their window fill, full chunk) needs no masking at all.
+        auto replay = [&](auto steady_tag) {
+          constexpr bool STEADY = decltype(steady_tag)::value;
+          float keep_evidence[kChunk];  // S + overflow
+          float keep_overflow[kChunk];
+          float keep_gate[kChunk];
+          float keep_adjoint[kChunk];   // external adjoint A of the route score
 
-        // Forward replay of the chunk.  Rows past the end of the band (only in
-        // the band's last chunk) repeat the last row's data and are masked,
-        // which keeps the loop free of branches.
-#pragma unroll
-        for (int r = 0; r < kChunk; ++r) {
-          const bool row_ok = r < rows_here;
-          const int i = min(first + r, last_step);
-          const int t = view.diag0 + 1 + i;
-          const uint32_t* row = rows + (local + r) * kRowWords;
-          const StepOut s = forward_step<NVW>(band, row, i, lane, W, P.gate_log2);
-          const float inv_denominator = __uint_as_float(row[8]);
-          const float expected = __uint_as_float(row[9]);
-          const float one_plus = 1.0f + s.evidence;
-          const float inv_root = fast_rsq(one_plus);
-          const float root = one_plus * inv_root;
-          const bool live = s.active && row_ok;
-          const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
-          const float probability = weight * inv_denominator;
-          float keep = 1.0f;
-          if constexpr (DROPOUT) {
-            if (view.masks != nullptr) {
-              const unsigned long long ballot =
-                  (static_cast<unsigned long long>(row[11]) << 32) | row[10];
-              keep = ((ballot >> lane) & 1ull) ? P.inverse_keep : 0.0f;
-            } else {
-              route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-              keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-            }
-          }
-          weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
-          float adjoint = 0.0f;
-          if (want_qk) {
-            const float utility = route_utility<NVW, DVP>(band, grad_tile + r * GP, s.grad_sum);
-            adjoint = P.scale * probability * (keep * utility - expected) *
-                      (0.5f * kSqrtScale * inv_root);
-          }
-          // rows past the band's end run on repeated data and may hold anything,
-          // NaN included: select, never multiply by zero
-          keep_adjoint[r] = live ? adjoint : 0.0f;
-          keep_gate[r] = live ? s.gate : 0.0f;
-          keep_overflow[r] = live ? s.overflow : 0.0f;
-          keep_evidence[r] = live ? s.evidence + s.overflow : 0.0f;
-        }
-
-        // reverse walk of the chunk
-        if (want_qk) {
-#pragma unroll
-          for (int r = kChunk - 1; r >= 0; --r) {
-            const int i = first + r;
-            const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
-            adjoint_carry = b;
-            gate_below = keep_gate[r];
-            const float overflow = keep_overflow[r];
-            const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
-            const bool any_term = __ballot(term != 0.0f) != 0ull;
-            if (any_term) {
-              if (ring_live == 0) ring_fresh = P.ring_rows;
-              ring_live = P.ring_rows;
-            }
-            if (ring_live > 0) {
-              const int slot = i % P.ring_rows;
-              float leaving = 0.0f;
-              if (ring_fresh > 0) {
-                --ring_fresh;
+          // Forward replay of the chunk.  Rows past the end of the band (only in
+          // the band's last chunk) repeat the last row's data and are masked,
+          // which keeps the loop free of branches.
+  #pragma unroll
+          for (int r = 0; r < kChunk; ++r) {
+            const bool row_ok = r < rows_here;
+            const int i = min(first + r, last_step);
+            const int t = view.diag0 + 1 + i;
+            const uint32_t* row = rows + (local + r) * kRowWords;
+            const StepOut s = forward_step<NVW, STEADY, true>(band, row, i, lane, W, P.gate_log2);
+            const float inv_denominator = __uint_as_float(row[8]);
+            const float expected = __uint_as_float(row[9]);
+            const float one_plus = 1.0f + s.evidence;
+            const float inv_root = fast_rsq(one_plus);
+            const float root = one_plus * inv_root;
+            const bool live = STEADY || (s.active && row_ok);
+            const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
+            const float probability = weight * inv_denominator;
+            float keep = 1.0f;
+            if constexpr (DROPOUT) {
+              if (view.masks != nullptr) {
+                const unsigned long long ballot =
+                    (static_cast<unsigned long long>(row[11]) << 32) | row[10];
+                keep = ((ballot >> lane) & 1ull) ? P.inverse_keep : 0.0f;
               } else {
-                leaving = ring[slot * kWave + lane];
+                route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
+                key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+                keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
               }
-              ring[slot * kWave + lane] = term;
-              ring_sum += term - leaving;
-              --ring_live;
             }
-            const float h = fmaf(b, keep_evidence[r], -ring_sum);
-            if (ring_live == 0) ring_sum = 0.0f;
-            const bool active = (i + 1 - lane) >= 1 && r < rows_here;
-            adjoint_tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
+            weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
+            float adjoint = 0.0f;
+            if (want_qk) {
+              const float utility = route_utility<NVW, DVP>(band, grad_tile + r * GP, s.grad_sum);
+              adjoint = P.scale * probability * (keep * utility - expected) *
+                        (0.5f * kSqrtScale * inv_root);
+            }
+            // rows past the band's end run on repeated data and may hold anything,
+            // NaN included: select, never multiply by zero
+            keep_adjoint[r] = live ? adjoint : 0.0f;
+            keep_gate[r] = live ? s.gate : 0.0f;
+            keep_overflow[r] = live ? s.overflow : 0.0f;
+            keep_evidence[r] = live ? s.evidence + s.overflow : 0.0f;
           }
+
+          // reverse walk of the chunk
+          if (want_qk) {
+  #pragma unroll
+            for (int r = kChunk - 1; r >= 0; --r) {
+              const int i = first + r;
+              const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
+              adjoint_carry = b;
+              gate_below = keep_gate[r];
+              const float overflow = keep_overflow[r];
+              const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
+              const bool any_term = __ballot(term != 0.0f) != 0ull;
+              if (any_term) {
+                if (ring_live == 0) ring_fresh = P.ring_rows;
+                ring_live = P.ring_rows;
+              }
+              if (ring_live > 0) {
+                const int slot = i % P.ring_rows;
+                float leaving = 0.0f;
+                if (ring_fresh > 0) {
+                  --ring_fresh;
+                } else {
+                  leaving = ring[slot * kWave + lane];
+                }
+                ring[slot * kWave + lane] = term;
+                ring_sum += term - leaving;
+                --ring_live;
+              }
+              const float h = fmaf(b, keep_evidence[r], -ring_sum);
+              if (ring_live == 0) ring_sum = 0.0f;
+              const bool active = STEADY || ((i + 1 - lane) >= 1 && r < rows_here);
+              adjoint_tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
+            }
+          }
+
+        };
+        if (first >= W + kWave && rows_here == kChunk) {
+          replay(std::true_type{});
+        } else {
+          replay(std::false_type{});
         }
 
         const int t_first = view.diag0 + 1 + first;
