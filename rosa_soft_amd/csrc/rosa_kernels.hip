@@ -512,7 +512,6 @@ struct VjpParams {
   const uint32_t* packed_key;
   const uint32_t* value_bits;   // [value_words_total][NVW], head-major over value heads
   const float* grad_rows;       // [head-major row][DVP] float32, zero padded
-  const float* grad_row_sum;    // [head-major row]
   float4* stats;                // [head-major row] (reference logit, denominator, numerator, base)
   const int64_t* dropout_seed;
   float scale, dropout_p, inverse_keep, mismatch_scale;
@@ -534,12 +533,11 @@ struct VjpParams {
   int total_units;
 };
 
-// grad_output -> float32 head-major rows padded to DVP, plus the row sums
+// grad_output -> float32 head-major rows padded to DVP
 template <int DTYPE>
 __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
-    const void* __restrict__ grad_output, float* __restrict__ grad_rows,
-    float* __restrict__ grad_row_sum, int64_t rows, int H, int Dv, int dvp, int T, int N,
-    int varlen) {
+    const void* __restrict__ grad_output, float* __restrict__ grad_rows, int64_t rows, int H,
+    int Dv, int dvp, int T, int N, int varlen) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (row >= rows) return;  // row = token * H + h (token-major)
   const int64_t token = row / H;
@@ -551,14 +549,9 @@ __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
     const int64_t b = token / T;
     dst = (b * H + h) * T + (token - b * T);
   }
-  float total = 0.0f;
   for (int d = 0; d < dvp; ++d) {
-    float g = 0.0f;
-    if (d < Dv) g = load_as_float<DTYPE>(grad_output, row * Dv + d);
-    grad_rows[dst * dvp + d] = g;
-    total += g;
+    grad_rows[dst * dvp + d] = d < Dv ? load_as_float<DTYPE>(grad_output, row * Dv + d) : 0.0f;
   }
-  grad_row_sum[dst] = total;
 }
 
 // value sign bits, head-major over value heads: word index (seq, hv, t) like the symbol words
@@ -634,7 +627,6 @@ struct Band {
   // sliding per-column registers (lane l holds the column a = a0 - l)
   uint32_t key_word;      // key word of column a     (key position a - 1)
   uint32_t old_key_word;  // key word of column a - W - 1, leaving the window
-  uint32_t value_bits[NVW];
   // per-diagonal state
   float evidence;   // S of the previous row on this diagonal
   int window;       // mismatching bits over the last min(n, W + 1) gates
@@ -645,7 +637,6 @@ struct BandView {
   const uint32_t* k;
   const uint32_t* vbits;   // value sign words of this (sequence, value head), NVW per token
   const float* grad_rows;  // [t][dvp]
-  const float* grad_sum;   // [t]
   float4* stats;           // [t]
   const unsigned long long* masks;  // cached keep ballots of this band (step i), or NULL
   int len;
@@ -660,10 +651,6 @@ __device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& vi
   const int a = i - lane;  // column held before the shift
   band.key_word = (a >= 1) ? view.k[a - 1] : 0u;
   band.old_key_word = (a - W - 2 >= 0) ? view.k[a - W - 2] : 0u;
-#pragma unroll
-  for (int w = 0; w < NVW; ++w) {
-    band.value_bits[w] = (a >= 1) ? view.vbits[static_cast<int64_t>(a) * NVW + w] : 0u;
-  }
 }
 
 // Everything a step needs that depends on the row only is staged in LDS for a
@@ -672,8 +659,9 @@ __device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& vi
 // wave-uniform LDS loads.  Staged words per row:
 //   0 query word of row t          1 query word of row t - W - 1
 //   2 key word entering at lane 0  3 key word of column a0 - W - 1 entering at lane 0
-//   4,5 value sign words entering  6 exponent shift of the row   7 sum of grad_output[t]
-//   8 1 / softmax denominator      9 expected dropped utility
+//   4 exponent shift of the row    5 1 / softmax denominator
+//   6 expected dropped utility     7 unused
+//   8,9 cached dropout keep ballot of the step (lanes 0-31, 32-63)
 constexpr int kRowWords = 12;
 enum RowDetail { kRowSymbols = 0, kRowStats = 1, kRowFull = 2 };
 
@@ -684,36 +672,42 @@ __device__ __forceinline__ void stage_rows(const BandView& view, int first, int 
     const int i = min(first + index, view.steps - 1);  // rows past the band's end repeat the last
     const int t = view.diag0 + 1 + i;
     const int a0 = i + 1;
-    uint4 symbols, extra, stats;
+    uint4 symbols;
     symbols.x = view.q[t];
     symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
     symbols.z = view.k[a0 - 1];
     symbols.w = (a0 - W - 2 >= 0) ? view.k[a0 - W - 2] : 0u;
-    extra.x = view.vbits[static_cast<int64_t>(a0) * NVW];
-    extra.y = NVW > 1 ? view.vbits[static_cast<int64_t>(a0) * NVW + (NVW - 1)] : 0u;
-    extra.z = 0u;
-    extra.w = 0u;
-    stats = make_uint4(0u, 0u, 0u, 0u);
+    uint4* dst = reinterpret_cast<uint4*>(rows + index * kRowWords);
+    dst[0] = symbols;
     if constexpr (DETAIL >= kRowStats) {
       const float4 row = view.stats[t];
-      extra.z = __float_as_uint(fmaf(row.x, kLog2e, row.w));
-      extra.w = __float_as_uint(view.grad_sum[t]);
+      uint4 extra = make_uint4(__float_as_uint(fmaf(row.x, kLog2e, row.w)), 0u, 0u, 0u);
       if constexpr (DETAIL == kRowFull) {
         const float null_weight = fast_exp2((null_logit - row.x) * kLog2e);
         const float inv_denominator = fast_rcp(row.y + null_weight);
-        stats.x = __float_as_uint(inv_denominator);
-        stats.y = __float_as_uint(row.z * inv_denominator);
+        extra.y = __float_as_uint(inv_denominator);
+        extra.z = __float_as_uint(row.z * inv_denominator);
         if (view.masks != nullptr) {
           const unsigned long long ballot = view.masks[i];
-          stats.z = static_cast<uint32_t>(ballot);
-          stats.w = static_cast<uint32_t>(ballot >> 32);
+          dst[2] = make_uint4(static_cast<uint32_t>(ballot), static_cast<uint32_t>(ballot >> 32),
+                              0u, 0u);
         }
       }
+      dst[1] = extra;
     }
-    uint4* dst = reinterpret_cast<uint4*>(rows + index * kRowWords);
-    dst[0] = symbols;
-    dst[1] = extra;
-    if constexpr (DETAIL == kRowFull) dst[2] = stats;
+  }
+}
+
+// Value sign words of the window columns of a block of rows: entry `index`
+// holds column a = first - 63 + index (zero outside 1 .. len-1).
+template <int NVW>
+__device__ __forceinline__ void stage_value_columns(const BandView& view, int first, int count,
+                                                    int lane, uint32_t* dst) {
+  for (int index = lane; index < count * NVW; index += kWave) {
+    const int column = index / NVW;
+    const int a = first - 63 + column;
+    dst[index] = (a >= 1 && a <= view.len - 1)
+        ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
   }
 }
 
@@ -740,8 +734,6 @@ struct StepOut {
   float gate;     // local match gate of this pair
   float overflow; // product of the W+1 gates ending here (0 while the window is not full)
   float evidence; // S(t, a)
-  float shift;    // exponent shift of the row (staged)
-  float grad_sum; // sum of grad_output[t] (staged)
   bool active;    // a >= 1
   int a;
 };
@@ -750,24 +742,14 @@ struct StepOut {
 // `row` points at the staged words of the step's row (wave-uniform address).
 // STEADY: every lane of the wave is past its diagonal's first W + 1 rows, so no
 // lane needs masking (true for all but the first W + 64 rows of a band).
-// VALUES: also slide the value sign bits (not needed by evidence-only sweeps).
-template <int NVW, bool STEADY = false, bool VALUES = true>
+template <int NVW, bool STEADY = false>
 __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const uint32_t* row, int i,
                                                 int lane, int W, float gate_log2) {
   const uint4 symbols = *reinterpret_cast<const uint4*>(row);
-  const uint4 extra = *reinterpret_cast<const uint4*>(row + 4);
   const int a0 = i + 1;
   band.key_word = dpp_wave_shr1(symbols.z, band.key_word);
   band.old_key_word = dpp_wave_shr1(symbols.w, band.old_key_word);
-  if constexpr (VALUES) {
-    band.value_bits[0] = dpp_wave_shr1(extra.x, band.value_bits[0]);
-    if constexpr (NVW > 1) {
-      band.value_bits[NVW - 1] = dpp_wave_shr1(extra.y, band.value_bits[NVW - 1]);
-    }
-  }
   StepOut out;
-  out.shift = __uint_as_float(extra.z);
-  out.grad_sum = __uint_as_float(extra.w);
   out.a = a0 - lane;
   const int mismatches = __popc(symbols.x ^ band.key_word);
   if constexpr (STEADY) {
@@ -797,33 +779,54 @@ __device__ __forceinline__ void sweep_rows(Band<NVW>& band, const uint32_t* rows
   if (first >= W + kWave) {  // steady state: all 64 lanes are past their window fill
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, true, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+      forward_step<NVW, true>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
     }
   } else {
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, false, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+      forward_step<NVW, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
     }
   }
 }
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ v4f mfma_16x16x4(float a, float b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+// Utilities u(t, a) = sum_d grad_output[t, d] * sign(v[a, d]) of 16 rows against
+// their 80 window columns on the matrix cores, written in (row r, lane l)
+// coordinates: out[r * pitch + l] for the pair on diagonal lane l, whose window
+// column is c = 64 - l + r.  `grad_tile` holds the 16 grad_output rows
+// (`grad_pitch` floats each, zero beyond Dv), `value_columns` the sign words of
+// the window columns (NVW per column).
 template <int NVW, int DVP>
-__device__ __forceinline__ float route_utility(const Band<NVW>& band, const float* grad_row,
-                                               float grad_sum) {
-  // u = sum_d go[d] * sign_d = 2 * sum_{d: bit set} go[d] - sum_d go[d]
-  float picked = 0.0f;
+__device__ __forceinline__ void utility_tile(const float* grad_tile, int grad_pitch,
+                                             const uint32_t* value_columns, float* out,
+                                             int pitch, int lane) {
+  const int li = lane & 15;
+  const int lg = lane >> 4;
 #pragma unroll
-  for (int q4 = 0; q4 < DVP / 4; ++q4) {
-    const float4 g = *reinterpret_cast<const float4*>(grad_row + 4 * q4);  // wave-uniform LDS read
-    const float parts[4] = {g.x, g.y, g.z, g.w};
+  for (int m = 0; m < 5; ++m) {
+    uint32_t words[NVW];
+#pragma unroll
+    for (int w = 0; w < NVW; ++w) words[w] = value_columns[(16 * m + li) * NVW + w];
+    v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < DVP / 4; ++ks) {
+      const int d = 4 * ks + lg;
+      const float a_value = grad_tile[li * grad_pitch + d];
+      const float b_value = ((words[(4 * ks) >> 5] >> (d & 31)) & 1u) ? 1.0f : -1.0f;
+      acc = mfma_16x16x4(a_value, b_value, acc);
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int d = 4 * q4 + e;
-      const int mask = static_cast<int>(band.value_bits[d >> 5] << (31 - (d & 31))) >> 31;
-      picked += __int_as_float(__float_as_int(parts[e]) & mask);
+      const int r = 4 * lg + e;
+      const int l = 64 - (16 * m + li) + r;
+      if (l >= 0 && l < kWave) out[r * pitch + l] = acc[e];
     }
   }
-  return fmaf(2.0f, picked, -grad_sum);
 }
 
 template <int NVW, bool VARLEN>
@@ -841,7 +844,6 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
       : (static_cast<int64_t>(u.seq) * P.L.Hv + value_head) * P.L.T;
   view.vbits = P.value_bits + value_base * NVW;
   view.grad_rows = P.grad_rows + u.word_base * P.dvp;
-  view.grad_sum = P.grad_row_sum + u.word_base;
   view.stats = P.stats + u.word_base;
   view.masks = nullptr;
   if (P.keep_masks != nullptr) {
@@ -898,6 +900,8 @@ template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   __shared__ __attribute__((aligned(16))) uint32_t rows[kWave * kRowWords];
   __shared__ __attribute__((aligned(16))) float grads[kWave * DVP];
+  __shared__ uint32_t value_columns[2 * kWave * NVW];
+  __shared__ float utilities[kChunk * kWave];
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -924,48 +928,59 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
     const int count = min(kWave, view.steps - first);
     __syncthreads();
     stage_rows<NVW, kRowStats>(view, first, count, lane, rows, W, P.null_logit);
-    if (needs_utility) stage_grad_rows<DVP>(view, first, count, lane, grads, DVP);
-    __syncthreads();
-    // compiled twice: once every lane is past its window fill no masking is needed
-    auto run_block = [&](auto steady_tag) {
-      constexpr bool STEADY = decltype(steady_tag)::value;
-      for (int r = 0; r < count; ++r) {
-        const int i = first + r;
-        const int t = view.diag0 + 1 + i;
-        const StepOut s = forward_step<NVW, STEADY, true>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
-        const float one_plus = 1.0f + s.evidence;
-        const float root = one_plus * fast_rsq(one_plus);
-        const float weight = (STEADY || s.active) ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
-        float numerator = 0.0f;
-        float keep = 1.0f;
-        if constexpr (DROPOUT) {
-          route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-          if (needs_utility || mask_out != nullptr) {
-            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-            keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-            if (mask_out != nullptr) {
-              // the gradient pass reads the decisions back instead of hashing again
-              const unsigned long long ballot = __ballot(keep != 0.0f);
-              if (lane == 0) mask_out[i] = ballot;
+    if (needs_utility) {
+      stage_grad_rows<DVP>(view, first, kWave, lane, grads, DVP);
+      stage_value_columns<NVW>(view, first, 2 * kWave, lane, value_columns);
+    }
+    for (int local = 0; local < count; local += kChunk) {
+      const int rows_here = min(kChunk, count - local);
+      __syncthreads();
+      if (needs_utility) {
+        utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
+                               kWave, lane);
+        __syncthreads();
+      }
+      // compiled twice: once every lane is past its window fill no masking is needed
+      auto run_rows = [&](auto steady_tag) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+        for (int r = 0; r < rows_here; ++r) {
+          const int i = first + local + r;
+          const int t = view.diag0 + 1 + i;
+          const uint32_t* row = rows + (local + r) * kRowWords;
+          const StepOut s = forward_step<NVW, STEADY>(band, row, i, lane, W, P.gate_log2);
+          const float shift = __uint_as_float(row[4]);
+          const float one_plus = 1.0f + s.evidence;
+          const float root = one_plus * fast_rsq(one_plus);
+          const float weight =
+              (STEADY || s.active) ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
+          float numerator = 0.0f;
+          float keep = 1.0f;
+          if constexpr (DROPOUT) {
+            route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
+            if (needs_utility || mask_out != nullptr) {
+              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+              keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+              if (mask_out != nullptr) {
+                // the gradient pass reads the decisions back instead of hashing again
+                const unsigned long long ballot = __ballot(keep != 0.0f);
+                if (lane == 0) mask_out[i] = ballot;
+              }
             }
           }
+          if (needs_utility) numerator = weight * keep * utilities[r * kWave + lane];
+          const float weight_sum = wave_sum_lane63(weight);
+          const float numerator_sum = wave_sum_lane63(numerator);
+          if (lane == 63) {
+            atomicAdd(&view.stats[t].y, weight_sum);
+            if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
+          }
         }
-        if (needs_utility) {
-          const float utility = route_utility<NVW, DVP>(band, grads + r * DVP, s.grad_sum);
-          numerator = weight * keep * utility;
-        }
-        const float weight_sum = wave_sum_lane63(weight);
-        const float numerator_sum = wave_sum_lane63(numerator);
-        if (lane == 63) {
-          atomicAdd(&view.stats[t].y, weight_sum);
-          if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
-        }
+      };
+      if (first + local >= W + kWave) {
+        run_rows(std::true_type{});
+      } else {
+        run_rows(std::false_type{});
       }
-    };
-    if (first >= W + kWave) {
-      run_block(std::true_type{});
-    } else {
-      run_block(std::false_type{});
     }
   }
 }
@@ -996,12 +1011,6 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
 // accumulator registers for their whole life.
 constexpr int kTilePitch = 96;   // 16 zero + 64 lanes + 16 zero
 constexpr int kWindowTiles = 5;  // 80 window columns
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ v4f mfma_16x16x4(float a, float b, v4f c) {
-  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-}
 
 __device__ __forceinline__ float sign_of_bit(uint32_t word, int bit, int width) {
   // +1 / -1 for symbol bits, 0 for padding columns beyond the symbol width
@@ -1035,6 +1044,7 @@ void vjp_gradients_kernel(VjpParams P) {
   float* grad_rows_lds = adjoint_tile + kChunk * kTilePitch; // [SEG][GP]
   uint32_t* rows = reinterpret_cast<uint32_t*>(grad_rows_lds + SEG * GP);  // [SEG][kRowWords]
   uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
+  uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1134,6 +1144,7 @@ void vjp_gradients_kernel(VjpParams P) {
         const int a = seg_first - 63 + index;  // column; key position a - 1
         key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
       }
+      if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
       __syncthreads();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
       // segment-level forward sweep: checkpoint before every chunk
@@ -1155,6 +1166,12 @@ void vjp_gradients_kernel(VjpParams P) {
         band.window = ck_window[chunk * kWave + lane];
         load_sliding<NVW>(band, view, first, lane, W);
         const float* grad_tile = grad_rows_lds + local * GP;
+        // utilities of the chunk, left where the gate adjoints will replace them
+        if (want_qk) {
+          utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, adjoint_tile + 16,
+                                 kTilePitch, lane);
+          __syncthreads();
+        }
         uint32_t route_hash = 0u;
         if constexpr (DROPOUT) {
           if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
@@ -1178,21 +1195,22 @@ void vjp_gradients_kernel(VjpParams P) {
             const int i = min(first + r, last_step);
             const int t = view.diag0 + 1 + i;
             const uint32_t* row = rows + (local + r) * kRowWords;
-            const StepOut s = forward_step<NVW, STEADY, true>(band, row, i, lane, W, P.gate_log2);
-            const float inv_denominator = __uint_as_float(row[8]);
-            const float expected = __uint_as_float(row[9]);
+            const StepOut s = forward_step<NVW, STEADY>(band, row, i, lane, W, P.gate_log2);
+            const float shift = __uint_as_float(row[4]);
+            const float inv_denominator = __uint_as_float(row[5]);
+            const float expected = __uint_as_float(row[6]);
             const float one_plus = 1.0f + s.evidence;
             const float inv_root = fast_rsq(one_plus);
             const float root = one_plus * inv_root;
             const bool live = STEADY || (s.active && row_ok);
-            const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -s.shift)) : 0.0f;
+            const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
             const float probability = weight * inv_denominator;
             float keep = 1.0f;
             if constexpr (DROPOUT) {
               if (view.masks != nullptr) {
-                const unsigned long long ballot =
-                    (static_cast<unsigned long long>(row[11]) << 32) | row[10];
-                keep = ((ballot >> lane) & 1ull) ? P.inverse_keep : 0.0f;
+                const uint32_t ballot_half = lane >= 32 ? row[9] : row[8];
+                const int kept = __builtin_amdgcn_sbfe(static_cast<int>(ballot_half), lane & 31, 1);
+                keep = __int_as_float(__float_as_int(P.inverse_keep) & kept);
               } else {
                 route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
                 key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
@@ -1202,7 +1220,7 @@ void vjp_gradients_kernel(VjpParams P) {
             weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
             float adjoint = 0.0f;
             if (want_qk) {
-              const float utility = route_utility<NVW, DVP>(band, grad_tile + r * GP, s.grad_sum);
+              const float utility = adjoint_tile[r * kTilePitch + 16 + lane];
               adjoint = P.scale * probability * (keep * utility - expected) *
                         (0.5f * kSqrtScale * inv_root);
             }
@@ -1484,7 +1502,7 @@ int padded_value_width(int Dv) {
 }
 
 struct VjpWorkspace {
-  size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows, grad_sum,
+  size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows,
       value_bits, keep_masks, block_scratch, total;
   int64_t mask_capacity;  // 64-lane keep ballots that fit in the workspace (0: none kept)
   int resident_blocks;
@@ -1507,7 +1525,6 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   const int dvp = padded_value_width(v.L.Dv);
   w.stats = cursor; cursor += align_up(sizeof(float) * 4 * rows);
   w.grad_rows = cursor; cursor += align_up(sizeof(float) * rows * dvp);
-  w.grad_sum = cursor; cursor += align_up(sizeof(float) * rows);
   w.value_bits = cursor;
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
   // Keep decisions of the dropout hash, one 64-lane ballot per (band, row)
@@ -1641,7 +1658,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int GP = ((DVP + 15) / 16) * 16;
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + 2 * kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + SEG + kWave;
+                            SEG * kRowWords + (SEG + kWave) * (1 + NVW);
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
@@ -1706,13 +1723,12 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
 
   float4* stats = at<float4>(workspace, w.stats);
   float* grad_rows = at<float>(workspace, w.grad_rows);
-  float* grad_sum = at<float>(workspace, w.grad_sum);
   uint32_t* value_bits = at<uint32_t>(workspace, w.value_bits);
   int32_t* counter = at<int32_t>(workspace, w.header) + 1;
   const bool analytic = analytic_reference_is_safe(L, scale);
 
   hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>, dim3(blocks_for(view.symbol_rows, 256)),
-                     dim3(256), 0, stream, grad_output, grad_rows, grad_sum, view.symbol_rows,
+                     dim3(256), 0, stream, grad_output, grad_rows, view.symbol_rows,
                      L.H, L.Dv, dvp, L.T, L.N, L.varlen);
   hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
                      dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
@@ -1734,7 +1750,6 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   P.packed_key = reinterpret_cast<const uint32_t*>(packed_key);
   P.value_bits = value_bits;
   P.grad_rows = grad_rows;
-  P.grad_row_sum = grad_sum;
   P.stats = stats;
   P.dropout_seed = dropout_seed;
   P.scale = scale;
