@@ -1026,22 +1026,21 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
 }
 
 // rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
-constexpr int gradient_segment(int dvp) { return dvp >= 64 ? 32 : 64; }
+constexpr int kGradientSegment = 32;
 
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
-  constexpr int GP = VT * 16;           // pitch of the staged grad_output rows
-  constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
+  constexpr int GP = DVP;               // pitch of the staged grad_output rows
+  constexpr int SEG = kGradientSegment; // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds[];
   float* ck_evidence = lds;                                  // [SEG_CHUNKS][64]
   int* ck_window = reinterpret_cast<int*>(lds + SEG_CHUNKS * kWave);
-  float* weight_tile = lds + 2 * SEG_CHUNKS * kWave;         // [kChunk][kTilePitch]
-  float* adjoint_tile = weight_tile + kChunk * kTilePitch;   // [kChunk][kTilePitch]
-  float* grad_rows_lds = adjoint_tile + kChunk * kTilePitch; // [SEG][GP]
+  float* tile = lds + 2 * SEG_CHUNKS * kWave;                // [kChunk][kTilePitch]
+  float* grad_rows_lds = tile + kChunk * kTilePitch;         // [SEG][GP]
   uint32_t* rows = reinterpret_cast<uint32_t*>(grad_rows_lds + SEG * GP);  // [SEG][kRowWords]
   uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
   uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
@@ -1060,10 +1059,8 @@ void vjp_gradients_kernel(VjpParams P) {
   float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
   float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
 
-  // zero the tiles once: the margins are never written again
-  for (int index = lane; index < 2 * kChunk * kTilePitch + SEG * GP; index += kWave) {
-    weight_tile[index] = 0.0f;
-  }
+  // zero the tile once: its margins are never written again
+  for (int index = lane; index < kChunk * kTilePitch; index += kWave) tile[index] = 0.0f;
   __syncthreads();
 
   for (;;) {
@@ -1166,30 +1163,33 @@ void vjp_gradients_kernel(VjpParams P) {
         band.window = ck_window[chunk * kWave + lane];
         load_sliding<NVW>(band, view, first, lane, W);
         const float* grad_tile = grad_rows_lds + local * GP;
-        // utilities of the chunk, left where the gate adjoints will replace them
+        const int t_first = view.diag0 + 1 + first;
+        const int a_first = first + 1;  // column of lane 0 in the chunk's first row
+        const uint32_t* key_tile = key_window + local;  // window column c <-> a = a_first - 64 + c
+        // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
+        // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
-          utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, adjoint_tile + 16,
-                                 kTilePitch, lane);
+          utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, tile + 16, kTilePitch,
+                                 lane);
           __syncthreads();
         }
         uint32_t route_hash = 0u;
         if constexpr (DROPOUT) {
           if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
         }
+        float keep_evidence[kChunk];  // S + overflow
+        float keep_overflow[kChunk];
+        float keep_gate[kChunk];
+        float keep_adjoint[kChunk];   // external adjoint A of the route score
 
-        // The replay is compiled twice: the steady-state form (all lanes past
-        // their window fill, full chunk) needs no masking at all.
+        // Forward replay of the chunk, compiled twice: the steady-state form (all
+        // lanes past their window fill, full chunk) needs no masking at all.  In
+        // the general form rows past the end of the band (only in the band's last
+        // chunk) repeat the last row's data and are masked, which keeps the loop
+        // free of branches.
         auto replay = [&](auto steady_tag) {
           constexpr bool STEADY = decltype(steady_tag)::value;
-          float keep_evidence[kChunk];  // S + overflow
-          float keep_overflow[kChunk];
-          float keep_gate[kChunk];
-          float keep_adjoint[kChunk];   // external adjoint A of the route score
-
-          // Forward replay of the chunk.  Rows past the end of the band (only in
-          // the band's last chunk) repeat the last row's data and are masked,
-          // which keeps the loop free of branches.
-  #pragma unroll
+#pragma unroll
           for (int r = 0; r < kChunk; ++r) {
             const bool row_ok = r < rows_here;
             const int i = min(first + r, last_step);
@@ -1217,13 +1217,14 @@ void vjp_gradients_kernel(VjpParams P) {
                 keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
               }
             }
-            weight_tile[r * kTilePitch + 16 + lane] = live ? probability * keep : 0.0f;
+            float* slot = tile + r * kTilePitch + 16 + lane;
             float adjoint = 0.0f;
             if (want_qk) {
-              const float utility = adjoint_tile[r * kTilePitch + 16 + lane];
+              const float utility = *slot;
               adjoint = P.scale * probability * (keep * utility - expected) *
                         (0.5f * kSqrtScale * inv_root);
             }
+            *slot = live ? probability * keep : 0.0f;
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
             keep_adjoint[r] = live ? adjoint : 0.0f;
@@ -1231,78 +1232,83 @@ void vjp_gradients_kernel(VjpParams P) {
             keep_overflow[r] = live ? s.overflow : 0.0f;
             keep_evidence[r] = live ? s.evidence + s.overflow : 0.0f;
           }
-
-          // reverse walk of the chunk
-          if (want_qk) {
-  #pragma unroll
-            for (int r = kChunk - 1; r >= 0; --r) {
-              const int i = first + r;
-              const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
-              adjoint_carry = b;
-              gate_below = keep_gate[r];
-              const float overflow = keep_overflow[r];
-              const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
-              const bool any_term = __ballot(term != 0.0f) != 0ull;
-              if (any_term) {
-                if (ring_live == 0) ring_fresh = P.ring_rows;
-                ring_live = P.ring_rows;
-              }
-              if (ring_live > 0) {
-                const int slot = i % P.ring_rows;
-                float leaving = 0.0f;
-                if (ring_fresh > 0) {
-                  --ring_fresh;
-                } else {
-                  leaving = ring[slot * kWave + lane];
-                }
-                ring[slot * kWave + lane] = term;
-                ring_sum += term - leaving;
-                --ring_live;
-              }
-              const float h = fmaf(b, keep_evidence[r], -ring_sum);
-              if (ring_live == 0) ring_sum = 0.0f;
-              const bool active = STEADY || ((i + 1 - lane) >= 1 && r < rows_here);
-              adjoint_tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
-            }
-          }
-
         };
-        if (first >= W + kWave && rows_here == kChunk) {
+        const bool steady = first >= W + kWave && rows_here == kChunk;
+        if (steady) {
           replay(std::true_type{});
         } else {
           replay(std::false_type{});
         }
-
-        const int t_first = view.diag0 + 1 + first;
-        const int a_first = first + 1;  // column of lane 0 in the chunk's first row
-        const uint32_t* key_tile = key_window + local;  // window column c <-> a = a_first - 64 + c
         __syncthreads();
 
-        // column sums: tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
-        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r]
-        if (want_v || want_k) {
+        // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
+        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r].
+        if (want_v) {
 #pragma unroll
           for (int step = 0; step < kChunk / 4; ++step) {
             const int r = 4 * step + lg;
             float grad_b[VT];
-            float query_b[DT];
 #pragma unroll
-            for (int n = 0; n < VT; ++n) grad_b[n] = grad_tile[r * GP + 16 * n + li];
-            const uint32_t q_word = r < rows_here ? rows[(local + r) * kRowWords] : 0u;
-#pragma unroll
-            for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
+            for (int n = 0; n < VT; ++n) {
+              grad_b[n] = (16 * n + li < DVP) ? grad_tile[r * GP + 16 * n + li] : 0.0f;
+            }
 #pragma unroll
             for (int m = 0; m < kWindowTiles; ++m) {
-              const int offset = r * kTilePitch + 16 + 64 - (16 * m + li) + r;
-              if (want_v) {
-                const float a_value = weight_tile[offset];
+              const float a_value = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
 #pragma unroll
-                for (int n = 0; n < VT; ++n) {
-                  value_acc[m][n] = mfma_16x16x4(a_value, grad_b[n], value_acc[m][n]);
-                }
+              for (int n = 0; n < VT; ++n) {
+                value_acc[m][n] = mfma_16x16x4(a_value, grad_b[n], value_acc[m][n]);
               }
-              if (want_k) {
-                const float a_value = adjoint_tile[offset];
+            }
+          }
+        }
+
+        if (want_qk) {
+          __syncthreads();
+          // reverse walk of the chunk: gate adjoints replace the weights
+#pragma unroll
+          for (int r = kChunk - 1; r >= 0; --r) {
+            const int i = first + r;
+            const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
+            adjoint_carry = b;
+            gate_below = keep_gate[r];
+            const float overflow = keep_overflow[r];
+            const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
+            const bool any_term = __ballot(term != 0.0f) != 0ull;
+            if (any_term) {
+              if (ring_live == 0) ring_fresh = P.ring_rows;
+              ring_live = P.ring_rows;
+            }
+            if (ring_live > 0) {
+              const int slot = i % P.ring_rows;
+              float leaving = 0.0f;
+              if (ring_fresh > 0) {
+                --ring_fresh;
+              } else {
+                leaving = ring[slot * kWave + lane];
+              }
+              ring[slot * kWave + lane] = term;
+              ring_sum += term - leaving;
+              --ring_live;
+            }
+            const float h = fmaf(b, keep_evidence[r], -ring_sum);
+            if (ring_live == 0) ring_sum = 0.0f;
+            const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
+            tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
+          }
+          __syncthreads();
+
+          if (want_k) {
+#pragma unroll
+            for (int step = 0; step < kChunk / 4; ++step) {
+              const int r = 4 * step + lg;
+              float query_b[DT];
+              const uint32_t q_word = r < rows_here ? rows[(local + r) * kRowWords] : 0u;
+#pragma unroll
+              for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
+#pragma unroll
+              for (int m = 0; m < kWindowTiles; ++m) {
+                const float a_value = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
 #pragma unroll
                 for (int n = 0; n < DT; ++n) {
                   key_acc[m][n] = mfma_16x16x4(a_value, query_b[n], key_acc[m][n]);
@@ -1310,33 +1316,33 @@ void vjp_gradients_kernel(VjpParams P) {
               }
             }
           }
-        }
-        // row sums: rows are complete for this band after the chunk
-        if (want_q) {
-          v4f query_acc[DT];
+          // row sums: rows are complete for this band after the chunk
+          if (want_q) {
+            v4f query_acc[DT];
 #pragma unroll
-          for (int n = 0; n < DT; ++n) query_acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int n = 0; n < DT; ++n) query_acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-          for (int step = 0; step < 4 * kWindowTiles; ++step) {
-            const int c = 4 * step + lg;
-            const float a_value = adjoint_tile[li * kTilePitch + 16 + 64 - c + li];
-            const uint32_t k_word = key_tile[c];
+            for (int step = 0; step < 4 * kWindowTiles; ++step) {
+              const int c = 4 * step + lg;
+              const float a_value = tile[li * kTilePitch + 16 + 64 - c + li];
+              const uint32_t k_word = key_tile[c];
+#pragma unroll
+              for (int n = 0; n < DT; ++n) {
+                query_acc[n] =
+                    mfma_16x16x4(a_value, sign_of_bit(k_word, 16 * n + li, D), query_acc[n]);
+              }
+            }
 #pragma unroll
             for (int n = 0; n < DT; ++n) {
-              query_acc[n] =
-                  mfma_16x16x4(a_value, sign_of_bit(k_word, 16 * n + li, D), query_acc[n]);
-            }
-          }
+              const int bit = 16 * n + li;
 #pragma unroll
-          for (int n = 0; n < DT; ++n) {
-            const int bit = 16 * n + li;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int r = 4 * lg + e;
-              if (bit < D && r < rows_here) {
-                const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
-                atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit],
-                          symbol_scale * query_acc[n][e]);
+              for (int e = 0; e < 4; ++e) {
+                const int r = 4 * lg + e;
+                if (bit < D && r < rows_here) {
+                  const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
+                  atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit],
+                            symbol_scale * query_acc[n][e]);
+                }
               }
             }
           }
@@ -1510,7 +1516,7 @@ struct VjpWorkspace {
   int ring_rows;
 };
 
-constexpr int kMaxResidentBlocks = 2048;
+constexpr int kMaxResidentBlocks = 4096;
 
 VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   VjpWorkspace w;
@@ -1544,7 +1550,7 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   }
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
-  const int segment_rows = gradient_segment(dvp);
+  const int segment_rows = kGradientSegment;
   const int max_segments = (longest + segment_rows - 1) / segment_rows + 1;
   w.block_scratch_floats =
       static_cast<int64_t>(w.ring_rows) * kWave + static_cast<int64_t>(max_segments) * 2 * kWave;
@@ -1655,9 +1661,9 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
                      0, stream, P);
   stage_end(kStageRowStats, stream);
-  constexpr int GP = ((DVP + 15) / 16) * 16;
-  constexpr int SEG = gradient_segment(DVP);
-  const size_t lds_floats = 2 * (SEG / kChunk) * kWave + 2 * kChunk * kTilePitch + SEG * GP +
+  constexpr int GP = DVP;
+  constexpr int SEG = kGradientSegment;
+  const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
                             SEG * kRowWords + (SEG + kWave) * (1 + NVW);
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
