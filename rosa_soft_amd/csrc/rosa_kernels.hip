@@ -100,6 +100,30 @@ __device__ __forceinline__ float dpp_add(float acc, float src) {
 }
 
 // Sum over the 64 lanes; the total is valid in lane 63 only.
+// lane `lane_index` (0..15, a constant after unrolling) of the result takes the
+// wave-uniform `value`, the others keep `old`
+__device__ __forceinline__ uint32_t write_lane(uint32_t value, int lane_index, uint32_t old) {
+#define ROSA_WRITE_LANE(n) \
+  case n: asm volatile("v_writelane_b32 %0, %1, " #n : "+v"(old) : "s"(value)); break;
+  switch (lane_index) {
+    ROSA_WRITE_LANE(0) ROSA_WRITE_LANE(1) ROSA_WRITE_LANE(2) ROSA_WRITE_LANE(3)
+    ROSA_WRITE_LANE(4) ROSA_WRITE_LANE(5) ROSA_WRITE_LANE(6) ROSA_WRITE_LANE(7)
+    ROSA_WRITE_LANE(8) ROSA_WRITE_LANE(9) ROSA_WRITE_LANE(10) ROSA_WRITE_LANE(11)
+    ROSA_WRITE_LANE(12) ROSA_WRITE_LANE(13) ROSA_WRITE_LANE(14) ROSA_WRITE_LANE(15)
+    default: break;
+  }
+#undef ROSA_WRITE_LANE
+  return old;
+}
+
+// The collector moves down by one lane and takes lane 63 of `total` at the top: after
+// 16 calls lane 48 + r holds the lane-63 value of call r.
+__device__ __forceinline__ float collect_lane63(float total, float collector) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(total),
+                                                    __float_as_int(collector), 0x130, 0xf, 0xf,
+                                                    false));  // wave_shl:1
+}
+
 __device__ __forceinline__ float wave_sum_lane63(float v) {
   v = dpp_add<0x111, 0xf>(v, v);  // row_shr:1
   v = dpp_add<0x112, 0xf>(v, v);  // row_shr:2
@@ -222,6 +246,15 @@ __host__ __device__ inline int64_t band_steps_before(int len, int band) {
   return static_cast<int64_t>(band) * (len - 1) - 32 * static_cast<int64_t>(band) * (band - 1);
 }
 
+// The row-statistics pass leaves (S, window) of every diagonal before each 16th row of a
+// band; chunk c of the band with global step offset `steps_before` and global band
+// number `bands_before` owns slot steps_before / 16 + bands_before + c (distinct for all
+// chunks of all bands, because a band of n steps has fewer than n / 16 + 2 chunks).
+constexpr int kCheckpointFloats = 128;  // [S | window][64 lanes]
+__host__ __device__ inline int64_t checkpoint_slots(int64_t steps, int64_t bands) {
+  return steps / 16 + bands + 1;
+}
+
 struct Unit {
   int seq;     // batch index (dense) or packed sequence index
   int block;   // 64-row block / 64-diagonal band index inside the sequence
@@ -274,7 +307,7 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
                                          int32_t* __restrict__ seq_len,
                                          int32_t* __restrict__ block_prefix,
                                          int64_t* __restrict__ step_prefix, int H,
-                                         int64_t mask_capacity,
+                                         int64_t mask_capacity, int64_t checkpoint_capacity,
                                          int32_t* __restrict__ header) {
   // single block; offsets are clamped into [previous, N] so that no later
   // kernel can index outside the tensors, and any violation is recorded.
@@ -324,6 +357,8 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
     }
     step_prefix[S] = steps;
     header[2] = steps * H <= mask_capacity ? 1 : 0;
+    header[3] = checkpoint_slots(steps * H, static_cast<int64_t>(block_prefix[S]) * H) <=
+                        checkpoint_capacity ? 1 : 0;
   }
   __syncthreads();
   int running = partial[threadIdx.x];
@@ -525,8 +560,9 @@ struct VjpParams {
   float* grad_key;
   float* grad_value;
   int32_t* work_counter;
-  const int32_t* header;        // [0] offsets flag, [1] work counter, [2] keep masks fit
+  const int32_t* header;        // [0] offsets flag, [1] work counter, [2] keep masks fit, [3] checkpoints fit
   unsigned long long* keep_masks;  // one 64-lane keep ballot per (band, row) step, or NULL
+  float* checkpoints;           // kCheckpointFloats per (band, 16-row chunk), or NULL
   float* block_scratch;         // per resident block: ring + segment checkpoints
   int64_t block_scratch_floats;
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
@@ -639,6 +675,7 @@ struct BandView {
   const float* grad_rows;  // [t][dvp]
   float4* stats;           // [t]
   const unsigned long long* masks;  // cached keep ballots of this band (step i), or NULL
+  float* checkpoints;      // (S, window) before every 16th row of this band, or NULL
   int len;
   int diag0;               // first diagonal of the band
   int steps;               // rows of the band: t = diag0 + 1 + i
@@ -659,15 +696,17 @@ __device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& vi
 // wave-uniform LDS loads.  Staged words per row:
 //   0 query word of row t          1 query word of row t - W - 1
 //   2 key word entering at lane 0  3 key word of column a0 - W - 1 entering at lane 0
-//   4 exponent shift of the row    5 1 / softmax denominator
-//   6 expected dropped utility     7 unused
-//   8,9 cached dropout keep ballot of the step (lanes 0-31, 32-63)
-constexpr int kRowWords = 12;
+//   4 exponent shift of the row    5 expected dropped utility
+//   6,7 cached dropout keep ballot of the step (lanes 0-31, 32-63)
+// In the row-statistics pass the shift is that of the raw weight; in the gradient
+// pass the row records are final and the shift includes log2 of the denominator,
+// so that exp2 gives the route probability directly.
+constexpr int kRowWords = 8;
 enum RowDetail { kRowSymbols = 0, kRowStats = 1, kRowFull = 2 };
 
 template <int NVW, int DETAIL>
 __device__ __forceinline__ void stage_rows(const BandView& view, int first, int count, int lane,
-                                           uint32_t* rows, int W, float null_logit) {
+                                           uint32_t* rows, int W) {
   for (int index = lane; index < count; index += kWave) {
     const int i = min(first + index, view.steps - 1);  // rows past the band's end repeat the last
     const int t = view.diag0 + 1 + i;
@@ -679,19 +718,16 @@ __device__ __forceinline__ void stage_rows(const BandView& view, int first, int 
     symbols.w = (a0 - W - 2 >= 0) ? view.k[a0 - W - 2] : 0u;
     uint4* dst = reinterpret_cast<uint4*>(rows + index * kRowWords);
     dst[0] = symbols;
-    if constexpr (DETAIL >= kRowStats) {
+    if constexpr (DETAIL == kRowStats) {
       const float4 row = view.stats[t];
-      uint4 extra = make_uint4(__float_as_uint(fmaf(row.x, kLog2e, row.w)), 0u, 0u, 0u);
-      if constexpr (DETAIL == kRowFull) {
-        const float null_weight = fast_exp2((null_logit - row.x) * kLog2e);
-        const float inv_denominator = fast_rcp(row.y + null_weight);
-        extra.y = __float_as_uint(inv_denominator);
-        extra.z = __float_as_uint(row.z * inv_denominator);
-        if (view.masks != nullptr) {
-          const unsigned long long ballot = view.masks[i];
-          dst[2] = make_uint4(static_cast<uint32_t>(ballot), static_cast<uint32_t>(ballot >> 32),
-                              0u, 0u);
-        }
+      dst[1] = make_uint4(__float_as_uint(fmaf(row.x, kLog2e, row.w)), 0u, 0u, 0u);
+    } else if constexpr (DETAIL == kRowFull) {
+      const uint4 record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
+      uint4 extra = make_uint4(record.y, record.z, 0u, 0u);
+      if (view.masks != nullptr) {
+        const unsigned long long ballot = view.masks[i];
+        extra.z = static_cast<uint32_t>(ballot);
+        extra.w = static_cast<uint32_t>(ballot >> 32);
       }
       dst[1] = extra;
     }
@@ -738,29 +774,40 @@ struct StepOut {
   int a;
 };
 
+// the four symbol words a step needs, all wave-uniform
+struct RowSymbols {
+  uint32_t query;      // q[t]
+  uint32_t old_query;  // q[t - W - 1]
+  uint32_t key;        // key word of column a0 = i + 1, entering at lane 0
+  uint32_t old_key;    // key word of column a0 - W - 1, entering at lane 0
+};
+
+__device__ __forceinline__ RowSymbols staged_symbols(const uint32_t* row) {
+  const uint4 words = *reinterpret_cast<const uint4*>(row);
+  return RowSymbols{words.x, words.y, words.z, words.w};
+}
+
 // One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
-// `row` points at the staged words of the step's row (wave-uniform address).
 // STEADY: every lane of the wave is past its diagonal's first W + 1 rows, so no
 // lane needs masking (true for all but the first W + 64 rows of a band).
 template <int NVW, bool STEADY = false>
-__device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const uint32_t* row, int i,
+__device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbols& symbols, int i,
                                                 int lane, int W, float gate_log2) {
-  const uint4 symbols = *reinterpret_cast<const uint4*>(row);
   const int a0 = i + 1;
-  band.key_word = dpp_wave_shr1(symbols.z, band.key_word);
-  band.old_key_word = dpp_wave_shr1(symbols.w, band.old_key_word);
+  band.key_word = dpp_wave_shr1(symbols.key, band.key_word);
+  band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
   StepOut out;
   out.a = a0 - lane;
-  const int mismatches = __popc(symbols.x ^ band.key_word);
+  const int mismatches = __popc(symbols.query ^ band.key_word);
   if constexpr (STEADY) {
     out.active = true;
-    band.window += mismatches - __popc(symbols.y ^ band.old_key_word);
+    band.window += mismatches - __popc(symbols.old_query ^ band.old_key_word);
     out.gate = fast_exp2(-gate_log2 * static_cast<float>(mismatches));
     out.overflow = fast_exp2(-gate_log2 * static_cast<float>(band.window));
     band.evidence = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
   } else {
     out.active = out.a >= 1;
-    const int leaving = (out.a >= W + 2) ? __popc(symbols.y ^ band.old_key_word) : 0;
+    const int leaving = (out.a >= W + 2) ? __popc(symbols.old_query ^ band.old_key_word) : 0;
     band.window = out.active ? band.window + mismatches - leaving : 0;
     out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
     out.overflow =
@@ -779,12 +826,14 @@ __device__ __forceinline__ void sweep_rows(Band<NVW>& band, const uint32_t* rows
   if (first >= W + kWave) {  // steady state: all 64 lanes are past their window fill
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, true>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+      forward_step<NVW, true>(band, staged_symbols(rows + r * kRowWords), first + r, lane, W,
+                              gate_log2);
     }
   } else {
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, false>(band, rows + r * kRowWords, first + r, lane, W, gate_log2);
+      forward_step<NVW, false>(band, staged_symbols(rows + r * kRowWords), first + r, lane, W,
+                               gate_log2);
     }
   }
 }
@@ -845,16 +894,26 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
   view.vbits = P.value_bits + value_base * NVW;
   view.grad_rows = P.grad_rows + u.word_base * P.dvp;
   view.stats = P.stats + u.word_base;
+  // position of the band in the global (step, band) order of the cached data
+  int64_t steps_before, bands_before;
+  const int blocks = (u.len + 63) >> 6;
+  if constexpr (VARLEN) {
+    steps_before = P.L.step_prefix[u.seq] * P.L.H + u.head * band_steps_total(u.len);
+    bands_before = static_cast<int64_t>(P.L.block_prefix[u.seq]) * P.L.H + u.head * blocks;
+  } else {
+    const int64_t sequence_head = static_cast<int64_t>(u.seq) * P.L.H + u.head;
+    steps_before = sequence_head * band_steps_total(u.len);
+    bands_before = sequence_head * blocks;
+  }
+  steps_before += band_steps_before(u.len, u.block);
+  bands_before += u.block;
   view.masks = nullptr;
-  if (P.keep_masks != nullptr) {
-    int64_t base;
-    if constexpr (VARLEN) {
-      base = P.L.step_prefix[u.seq] * P.L.H + u.head * band_steps_total(u.len);
-    } else {
-      base = (static_cast<int64_t>(u.seq) * P.L.H + u.head) * band_steps_total(u.len);
-    }
-    const bool fits = !VARLEN || P.header[2] != 0;
-    if (fits) view.masks = P.keep_masks + base + band_steps_before(u.len, u.block);
+  if (P.keep_masks != nullptr && (!VARLEN || P.header[2] != 0)) {
+    view.masks = P.keep_masks + steps_before;
+  }
+  view.checkpoints = nullptr;
+  if (P.checkpoints != nullptr && (!VARLEN || P.header[3] != 0)) {
+    view.checkpoints = P.checkpoints + ((steps_before >> 4) + bands_before) * kCheckpointFloats;
   }
   return true;
 }
@@ -878,11 +937,12 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
   for (int first = 0; first < view.steps; first += kWave) {
     const int count = min(kWave, view.steps - first);
     __syncthreads();
-    stage_rows<NVW, kRowSymbols>(view, first, count, lane, rows, W, P.null_logit);
+    stage_rows<NVW, kRowSymbols>(view, first, count, lane, rows, W);
     __syncthreads();
     for (int r = 0; r < count; ++r) {
       const int i = first + r;
-      const StepOut s = forward_step<NVW>(band, rows + r * kRowWords, i, lane, W, P.gate_log2);
+      const StepOut s =
+          forward_step<NVW>(band, staged_symbols(rows + r * kRowWords), i, lane, W, P.gate_log2);
       const int t = view.diag0 + 1 + i;
       const float root = sqrtf(1.0f + s.evidence);
       const float logit = P.scale * kSqrtScale * (root - 1.0f) - logf(static_cast<float>(t));
@@ -896,12 +956,16 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
 }
 
 // Row-statistics pass: denominator and expected dropped utility of every row.
+// Rows are processed 16 at a time without any branch in between: the two row
+// sums of a chunk are parked in lanes 0..15 and leave in one atomic each, and
+// so do the keep ballots kept for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
+  constexpr int kUtilityPitch = 67;  // 4 * (pitch + 1) = 16 (mod 64): conflict-free tile writes
   __shared__ __attribute__((aligned(16))) uint32_t rows[kWave * kRowWords];
   __shared__ __attribute__((aligned(16))) float grads[kWave * DVP];
   __shared__ uint32_t value_columns[2 * kWave * NVW];
-  __shared__ float utilities[kChunk * kWave];
+  __shared__ float utilities[kChunk * kUtilityPitch];
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -924,65 +988,116 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
   unsigned long long* mask_out = const_cast<unsigned long long*>(view.masks);
   uint32_t route_hash = route_hash_of(-lane);
+  const int last_step = view.steps - 1;
+  // without symbol gradients no utilities are computed and the tile stays zero
+  for (int index = lane; index < kChunk * kUtilityPitch; index += kWave) utilities[index] = 0.0f;
   for (int first = 0; first < view.steps; first += kWave) {
     const int count = min(kWave, view.steps - first);
     __syncthreads();
-    stage_rows<NVW, kRowStats>(view, first, count, lane, rows, W, P.null_logit);
+    stage_rows<NVW, kRowStats>(view, first, kWave, lane, rows, W);
     if (needs_utility) {
       stage_grad_rows<DVP>(view, first, kWave, lane, grads, DVP);
       stage_value_columns<NVW>(view, first, 2 * kWave, lane, value_columns);
     }
     for (int local = 0; local < count; local += kChunk) {
       const int rows_here = min(kChunk, count - local);
+      const int chunk_first = first + local;
+      if (view.checkpoints != nullptr) {
+        float* slot =
+            view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * kCheckpointFloats;
+        slot[lane] = band.evidence;
+        slot[kWave + lane] = __int_as_float(band.window);
+      }
       __syncthreads();
       if (needs_utility) {
         utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
-                               kWave, lane);
+                               kUtilityPitch, lane);
         __syncthreads();
       }
+      float weight_sums = 0.0f;     // lane 48 + r: sum of the weights of row r of the chunk
+      float numerator_sums = 0.0f;  // lane 48 + r: sum of weight * keep * utility
+      uint32_t ballot_low = 0u, ballot_high = 0u;  // lane r: keep ballot of row r
       // compiled twice: once every lane is past its window fill no masking is needed
-      auto run_rows = [&](auto steady_tag) {
+      auto run_chunk = [&](auto steady_tag) {
         constexpr bool STEADY = decltype(steady_tag)::value;
-        for (int r = 0; r < rows_here; ++r) {
-          const int i = first + local + r;
+        const uint32_t* row = rows + local * kRowWords;
+        uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
+        float next_shift = __uint_as_float(row[4]);
+        float next_utility = utilities[lane];
+#pragma unroll
+        for (int r = 0; r < kChunk; ++r) {
+          const RowSymbols symbols{next_symbols.x, next_symbols.y, next_symbols.z, next_symbols.w};
+          const float shift = next_shift;
+          const float utility = next_utility;
+          if (r + 1 < kChunk) {  // the next row's words are on their way while this one runs
+            next_symbols = *reinterpret_cast<const uint4*>(row + (r + 1) * kRowWords);
+            next_shift = __uint_as_float(row[(r + 1) * kRowWords + 4]);
+            next_utility = utilities[(r + 1) * kUtilityPitch + lane];
+          }
+          const int i = min(chunk_first + r, last_step);
           const int t = view.diag0 + 1 + i;
-          const uint32_t* row = rows + (local + r) * kRowWords;
-          const StepOut s = forward_step<NVW, STEADY>(band, row, i, lane, W, P.gate_log2);
-          const float shift = __uint_as_float(row[4]);
+          const StepOut s = forward_step<NVW, STEADY>(band, symbols, i, lane, W, P.gate_log2);
           const float one_plus = 1.0f + s.evidence;
           const float root = one_plus * fast_rsq(one_plus);
-          const float weight =
-              (STEADY || s.active) ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
-          float numerator = 0.0f;
+          const bool live = STEADY || (s.active && r < rows_here);
+          const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
           float keep = 1.0f;
           if constexpr (DROPOUT) {
             route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-            if (needs_utility || mask_out != nullptr) {
-              key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-              keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-              if (mask_out != nullptr) {
-                // the gradient pass reads the decisions back instead of hashing again
-                const unsigned long long ballot = __ballot(keep != 0.0f);
-                if (lane == 0) mask_out[i] = ballot;
-              }
-            }
+            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
+            keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+            const unsigned long long ballot = __ballot(keep != 0.0f);
+            ballot_low = write_lane(static_cast<uint32_t>(ballot), r, ballot_low);
+            ballot_high =
+                write_lane(static_cast<uint32_t>(ballot >> 32), r, ballot_high);
           }
-          if (needs_utility) numerator = weight * keep * utilities[r * kWave + lane];
+          const float numerator = weight * keep * utility;
           const float weight_sum = wave_sum_lane63(weight);
           const float numerator_sum = wave_sum_lane63(numerator);
-          if (lane == 63) {
-            atomicAdd(&view.stats[t].y, weight_sum);
-            if (needs_utility) atomicAdd(&view.stats[t].z, numerator_sum);
-          }
+          weight_sums = collect_lane63(weight_sum, weight_sums);
+          numerator_sums = collect_lane63(numerator_sum, numerator_sums);
         }
       };
-      if (first + local >= W + kWave) {
-        run_rows(std::true_type{});
+      if (chunk_first >= W + kWave && rows_here == kChunk) {
+        run_chunk(std::true_type{});
       } else {
-        run_rows(std::false_type{});
+        run_chunk(std::false_type{});
+      }
+      if (lane >= 48 && lane - 48 < rows_here) {
+        float4* row_stats = view.stats + (view.diag0 + 1 + chunk_first + lane - 48);
+        atomicAdd(&row_stats->y, weight_sums);
+        if (needs_utility) atomicAdd(&row_stats->z, numerator_sums);
+      }
+      if (lane < rows_here) {
+        const int i = chunk_first + lane;
+        if constexpr (DROPOUT) {
+          // the gradient pass reads the decisions back instead of hashing again
+          if (mask_out != nullptr) {
+            mask_out[i] = (static_cast<unsigned long long>(ballot_high) << 32) | ballot_low;
+          }
+        }
       }
     }
   }
+}
+
+// After the row-statistics pass a row's float4 (reference, denominator, dropped
+// utility sum, constant logit part) is replaced by what the gradient pass reads per
+// row: (unused, exponent shift including log2 of the denominator, expected dropped
+// utility, unused).
+__global__ __launch_bounds__(256) void finalize_row_records_kernel(float4* __restrict__ stats,
+                                                                   int64_t rows,
+                                                                   float null_logit) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= rows) return;
+  const float4 row = stats[index];
+  const float denominator = row.y + fast_exp2((null_logit - row.x) * kLog2e);
+  uint4 record;
+  record.x = 0u;
+  record.y = __float_as_uint(fmaf(row.x, kLog2e, row.w) + __log2f(denominator));
+  record.z = __float_as_uint(row.z / denominator);
+  record.w = 0u;
+  reinterpret_cast<uint4*>(stats)[index] = record;
 }
 
 // Gradient pass.  Persistent blocks pull bands from a work counter.  A band is
@@ -1009,7 +1124,10 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
 // tile (the 16 highest columns), which is flushed with global atomics, and the
 // other four shift up by one tile for the next chunk, so column sums live in
 // accumulator registers for their whole life.
-constexpr int kTilePitch = 96;   // 16 zero + 64 lanes + 16 zero
+// 16 zero + 64 lanes + 16 zero, padded to 99: with 4 * (pitch + 1) = 16 (mod 64) the
+// skewed reads of the column sums (k slice lg <-> row step + 4 lg) and of the row sums
+// (row li, stride pitch + 1 = 36 (mod 64)) both touch 64 different LDS banks.
+constexpr int kTilePitch = 99;
 constexpr int kWindowTiles = 5;  // 80 window columns
 
 __device__ __forceinline__ float sign_of_bit(uint32_t word, int bit, int width) {
@@ -1020,7 +1138,7 @@ __device__ __forceinline__ float sign_of_bit(uint32_t word, int bit, int width) 
 
 // register budget of the gradient kernel: waves per SIMD it is compiled for
 constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
-  if (value_tiles == 1 && symbol_tiles == 1) return 3;   // 168 registers, no spills
+  if (value_tiles == 1 && symbol_tiles == 1) return 2;
   if (value_tiles == 4 && symbol_tiles == 2) return 1;   // 120 accumulator registers alone
   return 2;
 }
@@ -1044,6 +1162,7 @@ void vjp_gradients_kernel(VjpParams P) {
   uint32_t* rows = reinterpret_cast<uint32_t*>(grad_rows_lds + SEG * GP);  // [SEG][kRowWords]
   uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
   uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
+  uint32_t* query_rows = value_window + (SEG + kWave) * NVW; // [SEG] query words of the rows
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1095,8 +1214,10 @@ void vjp_gradients_kernel(VjpParams P) {
 
     const int segments = (view.steps + SEG - 1) / SEG;
     Band<NVW> band;
-    // band-level forward sweep: checkpoint (S, window) before the first row of every segment
-    if (segments > 1) {
+    // Without stored checkpoints, a band-level forward sweep leaves (S, window) before the
+    // first row of every segment and a segment-level one before every chunk.
+    const bool stored = view.checkpoints != nullptr;
+    if (!stored && segments > 1) {
       band.evidence = 0.0f;
       band.window = 0;
       load_sliding<NVW>(band, view, 0, lane, W);
@@ -1105,7 +1226,7 @@ void vjp_gradients_kernel(VjpParams P) {
         seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
         const int first = segment * SEG;
         __syncthreads();
-        stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W, P.null_logit);
+        stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W);
         __syncthreads();
         sweep_rows<NVW>(band, rows, first, SEG, lane, W, P.gate_log2);
       }
@@ -1125,17 +1246,23 @@ void vjp_gradients_kernel(VjpParams P) {
     for (int segment = segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * SEG;
       const int seg_last = min(view.steps, seg_first + SEG);
-      if (segments > 1) {
-        band.evidence = seg_ck[(2 * segment) * kWave + lane];
-        band.window = __float_as_int(seg_ck[(2 * segment + 1) * kWave + lane]);
-      } else {
-        band.evidence = 0.0f;
-        band.window = 0;
+      if (!stored) {
+        if (segments > 1) {
+          band.evidence = seg_ck[(2 * segment) * kWave + lane];
+          band.window = __float_as_int(seg_ck[(2 * segment + 1) * kWave + lane]);
+        } else {
+          band.evidence = 0.0f;
+          band.window = 0;
+        }
+        load_sliding<NVW>(band, view, seg_first, lane, W);
       }
-      load_sliding<NVW>(band, view, seg_first, lane, W);
       // one round trip brings in everything the segment needs
       __syncthreads();
-      stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W, P.null_logit);
+      stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W);
+      if (lane < SEG) {
+        const int i = seg_first + lane;
+        query_rows[lane] = i < view.steps ? view.q[view.diag0 + 1 + i] : 0u;
+      }
       stage_grad_rows<DVP>(view, seg_first, SEG, lane, grad_rows_lds, GP);
       for (int index = lane; index < SEG + kWave; index += kWave) {
         const int a = seg_first - 63 + index;  // column; key position a - 1
@@ -1145,7 +1272,7 @@ void vjp_gradients_kernel(VjpParams P) {
       __syncthreads();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
       // segment-level forward sweep: checkpoint before every chunk
-      for (int chunk = 0; chunk < chunks; ++chunk) {
+      for (int chunk = 0; !stored && chunk < chunks; ++chunk) {
         ck_evidence[chunk * kWave + lane] = band.evidence;
         ck_window[chunk * kWave + lane] = band.window;
         if (chunk + 1 < chunks) {
@@ -1159,8 +1286,15 @@ void vjp_gradients_kernel(VjpParams P) {
         const int local = chunk * kChunk;               // first row of the chunk inside the segment
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
-        band.evidence = ck_evidence[chunk * kWave + lane];
-        band.window = ck_window[chunk * kWave + lane];
+        if (stored) {
+          const float* slot =
+              view.checkpoints + static_cast<int64_t>(first / kChunk) * kCheckpointFloats;
+          band.evidence = slot[lane];
+          band.window = __float_as_int(slot[kWave + lane]);
+        } else {
+          band.evidence = ck_evidence[chunk * kWave + lane];
+          band.window = ck_window[chunk * kWave + lane];
+        }
         load_sliding<NVW>(band, view, first, lane, W);
         const float* grad_tile = grad_rows_lds + local * GP;
         const int t_first = view.diag0 + 1 + first;
@@ -1177,6 +1311,10 @@ void vjp_gradients_kernel(VjpParams P) {
         if constexpr (DROPOUT) {
           if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
         }
+        if (!want_qk) {  // no utilities were written: the replay must still read finite values
+#pragma unroll
+          for (int r = 0; r < kChunk; ++r) tile[r * kTilePitch + 16 + lane] = 0.0f;
+        }
         float keep_evidence[kChunk];  // S + overflow
         float keep_overflow[kChunk];
         float keep_gate[kChunk];
@@ -1187,28 +1325,42 @@ void vjp_gradients_kernel(VjpParams P) {
         // the general form rows past the end of the band (only in the band's last
         // chunk) repeat the last row's data and are masked, which keeps the loop
         // free of branches.
-        auto replay = [&](auto steady_tag) {
+        auto replay = [&](auto steady_tag, auto cached_tag) {
           constexpr bool STEADY = decltype(steady_tag)::value;
+          constexpr bool CACHED = decltype(cached_tag)::value;  // keep decisions are read back
+          const uint32_t* row = rows + local * kRowWords;
+          const float* slot = tile + 16 + lane;
+          uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
+          uint4 next_extra = *reinterpret_cast<const uint4*>(row + 4);
+          float next_utility = *slot;
 #pragma unroll
           for (int r = 0; r < kChunk; ++r) {
+            const RowSymbols symbols{next_symbols.x, next_symbols.y, next_symbols.z,
+                                     next_symbols.w};
+            const uint4 extra = next_extra;
+            // the slot holds the pair's utility (anything finite when no symbol
+            // gradient is wanted, in which case the adjoint is never used)
+            const float utility = next_utility;
+            if (r + 1 < kChunk) {  // the next row's words are on their way while this one runs
+              next_symbols = *reinterpret_cast<const uint4*>(row + (r + 1) * kRowWords);
+              next_extra = *reinterpret_cast<const uint4*>(row + (r + 1) * kRowWords + 4);
+              next_utility = slot[(r + 1) * kTilePitch];
+            }
             const bool row_ok = r < rows_here;
             const int i = min(first + r, last_step);
             const int t = view.diag0 + 1 + i;
-            const uint32_t* row = rows + (local + r) * kRowWords;
-            const StepOut s = forward_step<NVW, STEADY>(band, row, i, lane, W, P.gate_log2);
-            const float shift = __uint_as_float(row[4]);
-            const float inv_denominator = __uint_as_float(row[5]);
-            const float expected = __uint_as_float(row[6]);
+            const float shift = __uint_as_float(extra.x);
+            const float expected = __uint_as_float(extra.y);
+            const StepOut s = forward_step<NVW, STEADY>(band, symbols, i, lane, W, P.gate_log2);
             const float one_plus = 1.0f + s.evidence;
             const float inv_root = fast_rsq(one_plus);
             const float root = one_plus * inv_root;
             const bool live = STEADY || (s.active && row_ok);
-            const float weight = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
-            const float probability = weight * inv_denominator;
+            const float probability = live ? fast_exp2(fmaf(root, P.logit_gain, -shift)) : 0.0f;
             float keep = 1.0f;
             if constexpr (DROPOUT) {
-              if (view.masks != nullptr) {
-                const uint32_t ballot_half = lane >= 32 ? row[9] : row[8];
+              if constexpr (CACHED) {
+                const uint32_t ballot_half = lane >= 32 ? extra.w : extra.z;
                 const int kept = __builtin_amdgcn_sbfe(static_cast<int>(ballot_half), lane & 31, 1);
                 keep = __int_as_float(__float_as_int(P.inverse_keep) & kept);
               } else {
@@ -1217,14 +1369,9 @@ void vjp_gradients_kernel(VjpParams P) {
                 keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
               }
             }
-            float* slot = tile + r * kTilePitch + 16 + lane;
-            float adjoint = 0.0f;
-            if (want_qk) {
-              const float utility = *slot;
-              adjoint = P.scale * probability * (keep * utility - expected) *
-                        (0.5f * kSqrtScale * inv_root);
-            }
-            *slot = live ? probability * keep : 0.0f;
+            const float adjoint = P.scale * probability * (keep * utility - expected) *
+                                  (0.5f * kSqrtScale * inv_root);
+            tile[r * kTilePitch + 16 + lane] = probability * keep;
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
             keep_adjoint[r] = live ? adjoint : 0.0f;
@@ -1234,10 +1381,13 @@ void vjp_gradients_kernel(VjpParams P) {
           }
         };
         const bool steady = first >= W + kWave && rows_here == kChunk;
+        const bool cached = DROPOUT && view.masks != nullptr;
         if (steady) {
-          replay(std::true_type{});
+          if (cached) replay(std::true_type{}, std::true_type{});
+          else replay(std::true_type{}, std::false_type{});
         } else {
-          replay(std::false_type{});
+          if (cached) replay(std::false_type{}, std::true_type{});
+          else replay(std::false_type{}, std::false_type{});
         }
         __syncthreads();
 
@@ -1246,7 +1396,7 @@ void vjp_gradients_kernel(VjpParams P) {
         if (want_v) {
 #pragma unroll
           for (int step = 0; step < kChunk / 4; ++step) {
-            const int r = 4 * step + lg;
+            const int r = step + 4 * lg;
             float grad_b[VT];
 #pragma unroll
             for (int n = 0; n < VT; ++n) {
@@ -1301,9 +1451,9 @@ void vjp_gradients_kernel(VjpParams P) {
           if (want_k) {
 #pragma unroll
             for (int step = 0; step < kChunk / 4; ++step) {
-              const int r = 4 * step + lg;
+              const int r = step + 4 * lg;
               float query_b[DT];
-              const uint32_t q_word = r < rows_here ? rows[(local + r) * kRowWords] : 0u;
+              const uint32_t q_word = query_rows[local + r];
 #pragma unroll
               for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
 #pragma unroll
@@ -1511,6 +1661,8 @@ struct VjpWorkspace {
   size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows,
       value_bits, keep_masks, block_scratch, total;
   int64_t mask_capacity;  // 64-lane keep ballots that fit in the workspace (0: none kept)
+  size_t checkpoints;
+  int64_t checkpoint_capacity;  // checkpoint slots that fit in the workspace (0: none kept)
   int resident_blocks;
   int64_t block_scratch_floats;
   int ring_rows;
@@ -1548,6 +1700,19 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
     w.mask_capacity = v.L.varlen ? std::min(wanted, budget) : (wanted <= 2 * budget ? wanted : 0);
     cursor += align_up(sizeof(uint64_t) * static_cast<size_t>(w.mask_capacity));
   }
+  // (S, window) checkpoints written by the row-statistics pass for the gradient pass,
+  // which otherwise rebuilds them with forward sweeps of its own
+  w.checkpoints = cursor;
+  {
+    const int64_t budget = (int64_t(1) << 32) / (sizeof(float) * kCheckpointFloats);  // 4 GiB
+    const int64_t steps = v.L.varlen
+        ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
+        : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
+    const int64_t wanted = checkpoint_slots(steps, static_cast<int64_t>(v.L.slots) * v.L.H);
+    w.checkpoint_capacity = v.L.varlen ? std::min(wanted, budget) : (wanted <= budget ? wanted : 0);
+    cursor += align_up(sizeof(float) * kCheckpointFloats *
+                       static_cast<size_t>(w.checkpoint_capacity));
+  }
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
   const int segment_rows = kGradientSegment;
@@ -1581,7 +1746,7 @@ unsigned blocks_for(int64_t items, int threads) {
 int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, size_t seq_start,
                              size_t seq_len, size_t block_prefix, size_t header,
                              hipStream_t stream, int64_t* step_prefix = nullptr,
-                             int64_t mask_capacity = 0) {
+                             int64_t mask_capacity = 0, int64_t checkpoint_capacity = 0) {
   if (!L.varlen) return 0;
   L.seq_start = at<int32_t>(workspace, seq_start);
   L.seq_len = at<int32_t>(workspace, seq_len);
@@ -1590,7 +1755,7 @@ int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, 
   hipLaunchKernelGGL(prepare_sequences_kernel, dim3(1), dim3(256), 0, stream, p->cu_seqlens, L.S,
                      L.N, at<int32_t>(workspace, seq_start), at<int32_t>(workspace, seq_len),
                      at<int32_t>(workspace, block_prefix), step_prefix, L.H, mask_capacity,
-                     at<int32_t>(workspace, header));
+                     checkpoint_capacity, at<int32_t>(workspace, header));
   return 0;
 }
 
@@ -1660,11 +1825,16 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   stage_begin(kStageRowStats, stream);
   hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
                      0, stream, P);
+  {
+    const int64_t rows = static_cast<int64_t>(P.L.N) * P.L.H;
+    hipLaunchKernelGGL(finalize_row_records_kernel, dim3(blocks_for(rows, 256)), dim3(256), 0,
+                       stream, P.stats, rows, P.null_logit);
+  }
   stage_end(kStageRowStats, stream);
   constexpr int GP = DVP;
   constexpr int SEG = kGradientSegment;
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (1 + NVW);
+                            SEG * kRowWords + (SEG + kWave) * (1 + NVW) + SEG;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
@@ -1713,7 +1883,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   Layout L = view.L;
   const VjpWorkspace w = carve_vjp(view, dropout_p > 0.0f);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
-                           stream, at<int64_t>(workspace, w.step_prefix), w.mask_capacity);
+                           stream, at<int64_t>(workspace, w.step_prefix), w.mask_capacity,
+                           w.checkpoint_capacity);
   const int dvp = padded_value_width(L.Dv);
   const int nvw = value_words(L.Dv);
   const int64_t symbol_elements = view.symbol_rows * L.D;
@@ -1781,6 +1952,7 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   P.work_counter = counter;
   P.header = at<int32_t>(workspace, w.header);
   P.keep_masks = w.mask_capacity > 0 ? at<unsigned long long>(workspace, w.keep_masks) : nullptr;
+  P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
   P.block_scratch = at<float>(workspace, w.block_scratch);
   P.block_scratch_floats = w.block_scratch_floats;
   P.ring_rows = w.ring_rows;
