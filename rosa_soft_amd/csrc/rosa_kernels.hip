@@ -1144,7 +1144,7 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
 }
 
 // rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
-constexpr int kGradientSegment = 32;
+constexpr int gradient_segment(int dvp) { return dvp >= 64 ? 32 : 64; }
 
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
@@ -1152,7 +1152,7 @@ __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr int GP = DVP;               // pitch of the staged grad_output rows
-  constexpr int SEG = kGradientSegment; // rows staged in LDS at a time
+  constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds[];
   float* ck_evidence = lds;                                  // [SEG_CHUNKS][64]
@@ -1715,7 +1715,7 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   }
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
-  const int segment_rows = kGradientSegment;
+  const int segment_rows = gradient_segment(dvp);
   const int max_segments = (longest + segment_rows - 1) / segment_rows + 1;
   w.block_scratch_floats =
       static_cast<int64_t>(w.ring_rows) * kWave + static_cast<int64_t>(max_segments) * 2 * kWave;
@@ -1832,7 +1832,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   }
   stage_end(kStageRowStats, stream);
   constexpr int GP = DVP;
-  constexpr int SEG = kGradientSegment;
+  constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
                             SEG * kRowWords + (SEG + kWave) * (1 + NVW) + SEG;
   const hipError_t attribute = hipFuncSetAttribute(
