@@ -98,6 +98,12 @@ def pair_count(config) -> int:
     return config["B"] * config["H"] * config["T"] * (config["T"] - 1) // 2
 
 
+# HBM bytes per launch of vjp_gradients_kernel, measured with `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs of this script (scaled by what the same counters read for
+# `--copy-calibration 1024`); only the metric workload has been measured.
+MEASURED_TRAFFIC_BYTES = {"metric": 2.87e9}
+
+
 def token_count(config) -> int:
     return sum(config["lengths"]) if "lengths" in config else config["B"] * config["T"]
 
@@ -188,6 +194,11 @@ def main() -> None:
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--workload", default="metric", choices=sorted(WORKLOADS))
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument(
+        "--copy-calibration", type=int, default=0, metavar="MIB",
+        help="only run a plain device copy of MIB mebibytes three times (reference point for "
+             "scaling the FETCH_SIZE / WRITE_SIZE counters of rocprofv3) and exit",
+    )
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(
@@ -196,6 +207,16 @@ def main() -> None:
             file=sys.stderr,
         )
         sys.exit(2)
+
+    if args.copy_calibration > 0:
+        source = torch.ones(args.copy_calibration << 18, dtype=torch.float32, device="cuda:0")
+        target = torch.empty_like(source)
+        for _ in range(3):
+            target.copy_(source)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": source.numel() * 4, "copy_bytes_written": source.numel() * 4,
+                          "launches": 3}))
+        return
 
     import rosa_soft_amd
     from rosa_soft_amd import cabi
@@ -293,8 +314,10 @@ def main() -> None:
             "peak": FP32_MATRIX_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved_tflops / FP32_MATRIX_PEAK_TFLOPS,
-            "traffic": None,
-            "note": "algorithmic flops 2*pairs*(3D+2Dv) over the kernel's mean launch time",
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "note": "algorithmic flops 2*pairs*(3D+2Dv) over the kernel's mean launch time; "
+                    "traffic = HBM bytes per launch of this kernel from rocprofv3 FETCH_SIZE + "
+                    "WRITE_SIZE runs of this command, scaled by a 1 GiB device copy",
         },
         "kernels": kernels,
     }
