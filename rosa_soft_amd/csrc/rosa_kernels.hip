@@ -1416,6 +1416,22 @@ void vjp_gradients_kernel(VjpParams P) {
         if (want_qk) {
           __syncthreads();
           // reverse walk of the chunk: gate adjoints replace the weights
+          float peak_overflow = keep_overflow[0];
+#pragma unroll
+          for (int r = 1; r < kChunk; ++r) peak_overflow = fmaxf(peak_overflow, keep_overflow[r]);
+          const bool quiet = steady && ring_live == 0 &&
+                             __ballot(peak_overflow >= P.tail_threshold) == 0ull;
+          if (quiet) {
+            // no overflow term of the chunk can move a gradient and the ring is empty:
+            // h = b (S + o), nothing to mask
+#pragma unroll
+            for (int r = kChunk - 1; r >= 0; --r) {
+              const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
+              adjoint_carry = b;
+              gate_below = keep_gate[r];
+              tile[r * kTilePitch + 16 + lane] = b * keep_evidence[r];
+            }
+          } else {
 #pragma unroll
           for (int r = kChunk - 1; r >= 0; --r) {
             const int i = first + r;
@@ -1445,6 +1461,7 @@ void vjp_gradients_kernel(VjpParams P) {
             if (ring_live == 0) ring_sum = 0.0f;
             const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
             tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
+          }
           }
           __syncthreads();
 
@@ -1668,7 +1685,7 @@ struct VjpWorkspace {
   int ring_rows;
 };
 
-constexpr int kMaxResidentBlocks = 4096;
+constexpr int kMaxResidentBlocks = 2048;
 
 VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   VjpWorkspace w;
