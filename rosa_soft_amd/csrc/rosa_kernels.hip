@@ -116,12 +116,12 @@ __device__ __forceinline__ uint32_t write_lane(uint32_t value, int lane_index, u
   return old;
 }
 
-// The collector moves down by one lane and takes lane 63 of `total` at the top: after
-// 16 calls lane 48 + r holds the lane-63 value of call r.
-__device__ __forceinline__ float collect_lane63(float total, float collector) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(total),
-                                                    __float_as_int(collector), 0x130, 0xf, 0xf,
-                                                    false));  // wave_shl:1
+// The band kernels run one wavefront per block.  LDS instructions of one wave execute in
+// order, so data written by one lane is visible to another lane's later read without a
+// barrier; what is needed is that the compiler keeps the order, and nothing else: a full
+// __syncthreads() would also wait for every outstanding global store and atomic.
+__device__ __forceinline__ void wave_lds_fence() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 }
 
 __device__ __forceinline__ float wave_sum_lane63(float v) {
@@ -936,9 +936,9 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
   load_sliding<NVW>(band, view, 0, lane, W);
   for (int first = 0; first < view.steps; first += kWave) {
     const int count = min(kWave, view.steps - first);
-    __syncthreads();
+    wave_lds_fence();
     stage_rows<NVW, kRowSymbols>(view, first, count, lane, rows, W);
-    __syncthreads();
+    wave_lds_fence();
     for (int r = 0; r < count; ++r) {
       const int i = first + r;
       const StepOut s =
@@ -955,17 +955,40 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
   }
 }
 
+// Sum of every row of a [16][pitch] LDS tile over its 64 columns: each lane adds four
+// neighbouring columns (one 16-byte read), and the matrix cores add the 16 partial sums
+// of a row (the partial sums times a matrix of ones).  `pitch` is a multiple of 4 floats.
+// Lane (li, lg) = (lane & 15, lane >> 4) returns with the sums of rows 4 lg + e in
+// element e, whatever li.
+__device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, int lane) {
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  v4f sums = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    const float4 part =
+        *reinterpret_cast<const float4*>(tile_rows + li * pitch + 16 * ks + 4 * lg);
+    sums = mfma_16x16x4((part.x + part.y) + (part.z + part.w), 1.0f, sums);
+  }
+  return sums;
+}
+
 // Row-statistics pass: denominator and expected dropped utility of every row.
-// Rows are processed 16 at a time without any branch in between: the two row
-// sums of a chunk are parked in lanes 0..15 and leave in one atomic each, and
-// so do the keep ballots kept for the gradient pass.
+// Rows are processed 16 at a time without any branch in between.  A chunk leaves
+// its route weights and its dropped weighted utilities as two [row][lane] tiles
+// in LDS; their row sums are formed on the matrix cores and leave in one atomic
+// each from 16 lanes, and the 16 keep ballots kept for the gradient pass leave
+// as one store.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
-  constexpr int kUtilityPitch = 67;  // 4 * (pitch + 1) = 16 (mod 64): conflict-free tile writes
-  __shared__ __attribute__((aligned(16))) uint32_t rows[kWave * kRowWords];
-  __shared__ __attribute__((aligned(16))) float grads[kWave * DVP];
-  __shared__ uint32_t value_columns[2 * kWave * NVW];
-  __shared__ float utilities[kChunk * kUtilityPitch];
+  constexpr int kBlockRows = 32;     // rows staged in LDS at a time
+  constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
+  constexpr int kWeightPitch = 68;
+  __shared__ __attribute__((aligned(16))) uint32_t rows[kBlockRows * kRowWords];
+  __shared__ __attribute__((aligned(16))) float grads[kBlockRows * DVP];
+  __shared__ uint32_t value_columns[(kBlockRows + kWave) * NVW];
+  __shared__ __attribute__((aligned(16))) float utilities[kChunk * kUtilityPitch];  // u, then e d u
+  __shared__ __attribute__((aligned(16))) float weights[kChunk * kWeightPitch];     // e
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -991,13 +1014,13 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   const int last_step = view.steps - 1;
   // without symbol gradients no utilities are computed and the tile stays zero
   for (int index = lane; index < kChunk * kUtilityPitch; index += kWave) utilities[index] = 0.0f;
-  for (int first = 0; first < view.steps; first += kWave) {
-    const int count = min(kWave, view.steps - first);
-    __syncthreads();
-    stage_rows<NVW, kRowStats>(view, first, kWave, lane, rows, W);
+  for (int first = 0; first < view.steps; first += kBlockRows) {
+    const int count = min(kBlockRows, view.steps - first);
+    wave_lds_fence();
+    stage_rows<NVW, kRowStats>(view, first, kBlockRows, lane, rows, W);
     if (needs_utility) {
-      stage_grad_rows<DVP>(view, first, kWave, lane, grads, DVP);
-      stage_value_columns<NVW>(view, first, 2 * kWave, lane, value_columns);
+      stage_grad_rows<DVP>(view, first, kBlockRows, lane, grads, DVP);
+      stage_value_columns<NVW>(view, first, kBlockRows + kWave, lane, value_columns);
     }
     for (int local = 0; local < count; local += kChunk) {
       const int rows_here = min(kChunk, count - local);
@@ -1008,14 +1031,12 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
         slot[lane] = band.evidence;
         slot[kWave + lane] = __int_as_float(band.window);
       }
-      __syncthreads();
+      wave_lds_fence();
       if (needs_utility) {
         utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
                                kUtilityPitch, lane);
-        __syncthreads();
+        wave_lds_fence();
       }
-      float weight_sums = 0.0f;     // lane 48 + r: sum of the weights of row r of the chunk
-      float numerator_sums = 0.0f;  // lane 48 + r: sum of weight * keep * utility
       uint32_t ballot_low = 0u, ballot_high = 0u;  // lane r: keep ballot of row r
       // compiled twice: once every lane is past its window fill no masking is needed
       auto run_chunk = [&](auto steady_tag) {
@@ -1048,14 +1069,10 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
             keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
             const unsigned long long ballot = __ballot(keep != 0.0f);
             ballot_low = write_lane(static_cast<uint32_t>(ballot), r, ballot_low);
-            ballot_high =
-                write_lane(static_cast<uint32_t>(ballot >> 32), r, ballot_high);
+            ballot_high = write_lane(static_cast<uint32_t>(ballot >> 32), r, ballot_high);
           }
-          const float numerator = weight * keep * utility;
-          const float weight_sum = wave_sum_lane63(weight);
-          const float numerator_sum = wave_sum_lane63(numerator);
-          weight_sums = collect_lane63(weight_sum, weight_sums);
-          numerator_sums = collect_lane63(numerator_sum, numerator_sums);
+          weights[r * kWeightPitch + lane] = weight;
+          utilities[r * kUtilityPitch + lane] = weight * keep * utility;
         }
       };
       if (chunk_first >= W + kWave && rows_here == kChunk) {
@@ -1063,18 +1080,28 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       } else {
         run_chunk(std::false_type{});
       }
-      if (lane >= 48 && lane - 48 < rows_here) {
-        float4* row_stats = view.stats + (view.diag0 + 1 + chunk_first + lane - 48);
-        atomicAdd(&row_stats->y, weight_sums);
-        if (needs_utility) atomicAdd(&row_stats->z, numerator_sums);
+      wave_lds_fence();
+      {
+        const v4f weight_sums = tile_row_sums(weights, kWeightPitch, lane);
+        const v4f numerator_sums = tile_row_sums(utilities, kUtilityPitch, lane);
+        // lanes 0..3 of every 16-lane group write the four rows of their group
+        const int e = lane & 15;
+        const int r = 4 * (lane >> 4) + e;
+        if (e < 4 && r < rows_here) {
+          const float weight_sum = e == 0 ? weight_sums[0] : e == 1 ? weight_sums[1]
+                                 : e == 2 ? weight_sums[2] : weight_sums[3];
+          const float numerator_sum = e == 0 ? numerator_sums[0] : e == 1 ? numerator_sums[1]
+                                    : e == 2 ? numerator_sums[2] : numerator_sums[3];
+          float4* row_stats = view.stats + (view.diag0 + 1 + chunk_first + r);
+          atomicAdd(&row_stats->y, weight_sum);
+          if (needs_utility) atomicAdd(&row_stats->z, numerator_sum);
+        }
       }
-      if (lane < rows_here) {
-        const int i = chunk_first + lane;
-        if constexpr (DROPOUT) {
-          // the gradient pass reads the decisions back instead of hashing again
-          if (mask_out != nullptr) {
-            mask_out[i] = (static_cast<unsigned long long>(ballot_high) << 32) | ballot_low;
-          }
+      if constexpr (DROPOUT) {
+        // the gradient pass reads the decisions back instead of hashing again
+        if (lane < rows_here && mask_out != nullptr) {
+          mask_out[chunk_first + lane] =
+              (static_cast<unsigned long long>(ballot_high) << 32) | ballot_low;
         }
       }
     }
@@ -1180,7 +1207,7 @@ void vjp_gradients_kernel(VjpParams P) {
 
   // zero the tile once: its margins are never written again
   for (int index = lane; index < kChunk * kTilePitch; index += kWave) tile[index] = 0.0f;
-  __syncthreads();
+  wave_lds_fence();
 
   for (;;) {
     int unit_index = 0;
@@ -1225,9 +1252,9 @@ void vjp_gradients_kernel(VjpParams P) {
         seg_ck[(2 * segment) * kWave + lane] = band.evidence;
         seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
         const int first = segment * SEG;
-        __syncthreads();
+        wave_lds_fence();
         stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W);
-        __syncthreads();
+        wave_lds_fence();
         sweep_rows<NVW>(band, rows, first, SEG, lane, W, P.gate_log2);
       }
       const int segment = segments - 1;
@@ -1257,7 +1284,7 @@ void vjp_gradients_kernel(VjpParams P) {
         load_sliding<NVW>(band, view, seg_first, lane, W);
       }
       // one round trip brings in everything the segment needs
-      __syncthreads();
+      wave_lds_fence();
       stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W);
       if (lane < SEG) {
         const int i = seg_first + lane;
@@ -1269,7 +1296,7 @@ void vjp_gradients_kernel(VjpParams P) {
         key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
       }
       if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
-      __syncthreads();
+      wave_lds_fence();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
       // segment-level forward sweep: checkpoint before every chunk
       for (int chunk = 0; !stored && chunk < chunks; ++chunk) {
@@ -1305,7 +1332,7 @@ void vjp_gradients_kernel(VjpParams P) {
         if (want_qk) {
           utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, tile + 16, kTilePitch,
                                  lane);
-          __syncthreads();
+          wave_lds_fence();
         }
         uint32_t route_hash = 0u;
         if constexpr (DROPOUT) {
@@ -1389,7 +1416,7 @@ void vjp_gradients_kernel(VjpParams P) {
           if (cached) replay(std::false_type{}, std::true_type{});
           else replay(std::false_type{}, std::false_type{});
         }
-        __syncthreads();
+        wave_lds_fence();
 
         // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
         // element (column c, row r) of the skewed matrix is tile[r][64 - c + r].
@@ -1414,7 +1441,7 @@ void vjp_gradients_kernel(VjpParams P) {
         }
 
         if (want_qk) {
-          __syncthreads();
+          wave_lds_fence();
           // reverse walk of the chunk: gate adjoints replace the weights
           float peak_overflow = keep_overflow[0];
 #pragma unroll
@@ -1463,7 +1490,7 @@ void vjp_gradients_kernel(VjpParams P) {
             tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
           }
           }
-          __syncthreads();
+          wave_lds_fence();
 
           if (want_k) {
 #pragma unroll
@@ -1554,7 +1581,7 @@ void vjp_gradients_kernel(VjpParams P) {
         for (int n = 0; n < VT; ++n) value_acc[0][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int n = 0; n < DT; ++n) key_acc[0][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        __syncthreads();
+        wave_lds_fence();
       }
     }
   }
