@@ -844,36 +844,45 @@ __device__ __forceinline__ v4f mfma_16x16x4(float a, float b, v4f c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// +1.0f where bit 31 of `x` is clear, -1.0f where it is set
+__device__ __forceinline__ float sign_from_bit31(uint32_t x) {
+  return __uint_as_float((x & 0x80000000u) | 0x3f800000u);
+}
+
 // Utilities u(t, a) = sum_d grad_output[t, d] * sign(v[a, d]) of 16 rows against
 // their 80 window columns on the matrix cores, written in (row r, lane l)
 // coordinates: out[r * pitch + l] for the pair on diagonal lane l, whose window
 // column is c = 64 - l + r.  `grad_tile` holds the 16 grad_output rows
 // (`grad_pitch` floats each, zero beyond Dv), `value_columns` the sign words of
-// the window columns (NVW per column).
+// the window columns (NVW per column).  Elements of the first and last column
+// tile that belong to no lane go to `discard` (one float per lane).
 template <int NVW, int DVP>
 __device__ __forceinline__ void utility_tile(const float* grad_tile, int grad_pitch,
                                              const uint32_t* value_columns, float* out,
-                                             int pitch, int lane) {
+                                             int pitch, float* discard, int lane) {
   const int li = lane & 15;
   const int lg = lane >> 4;
 #pragma unroll
   for (int m = 0; m < 5; ++m) {
+    // inverted and moved down by lg: bit 4 ks of a word is the inverted sign bit 4 ks + lg
     uint32_t words[NVW];
 #pragma unroll
-    for (int w = 0; w < NVW; ++w) words[w] = value_columns[(16 * m + li) * NVW + w];
+    for (int w = 0; w < NVW; ++w) words[w] = ~value_columns[(16 * m + li) * NVW + w] >> lg;
     v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int ks = 0; ks < DVP / 4; ++ks) {
-      const int d = 4 * ks + lg;
-      const float a_value = grad_tile[li * grad_pitch + d];
-      const float b_value = ((words[(4 * ks) >> 5] >> (d & 31)) & 1u) ? 1.0f : -1.0f;
+      const float a_value = grad_tile[li * grad_pitch + 4 * ks + lg];
+      const float b_value = sign_from_bit31(words[(4 * ks) >> 5] << (31 - ((4 * ks) & 31)));
       acc = mfma_16x16x4(a_value, b_value, acc);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int r = 4 * lg + e;
       const int l = 64 - (16 * m + li) + r;
-      if (l >= 0 && l < kWave) out[r * pitch + l] = acc[e];
+      float* target = out + r * pitch + l;
+      if (m == 0) target = l < kWave ? target : discard + lane;
+      if (m == 4) target = l >= 0 ? target : discard + lane;
+      *target = acc[e];
     }
   }
 }
@@ -989,6 +998,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   __shared__ uint32_t value_columns[(kBlockRows + kWave) * NVW];
   __shared__ __attribute__((aligned(16))) float utilities[kChunk * kUtilityPitch];  // u, then e d u
   __shared__ __attribute__((aligned(16))) float weights[kChunk * kWeightPitch];     // e
+  __shared__ float discard[kWave];
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -1034,7 +1044,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       wave_lds_fence();
       if (needs_utility) {
         utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
-                               kUtilityPitch, lane);
+                               kUtilityPitch, discard, lane);
         wave_lds_fence();
       }
       uint32_t ballot_low = 0u, ballot_high = 0u;  // lane r: keep ballot of row r
@@ -1157,10 +1167,11 @@ __global__ __launch_bounds__(256) void finalize_row_records_kernel(float4* __res
 constexpr int kTilePitch = 99;
 constexpr int kWindowTiles = 5;  // 80 window columns
 
-__device__ __forceinline__ float sign_of_bit(uint32_t word, int bit, int width) {
-  // +1 / -1 for symbol bits, 0 for padding columns beyond the symbol width
-  if (bit >= width) return 0.0f;
-  return ((word >> bit) & 1u) ? 1.0f : -1.0f;
+// -1.0f where symbol bit `bit` of `word` is set, +1.0f where it is clear: the negated
+// symbol, two instructions; callers fold the sign into their output scale.  Columns
+// beyond the symbol width produce values nobody stores.
+__device__ __forceinline__ float negated_symbol(uint32_t word, int bit) {
+  return sign_from_bit31(word << (31 - bit));
 }
 
 // register budget of the gradient kernel: waves per SIMD it is compiled for
@@ -1190,6 +1201,7 @@ void vjp_gradients_kernel(VjpParams P) {
   uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
   uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
   uint32_t* query_rows = value_window + (SEG + kWave) * NVW; // [SEG] query words of the rows
+  float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1201,7 +1213,8 @@ void vjp_gradients_kernel(VjpParams P) {
   const bool want_k = (P.gradient_mask & ROSA_GRAD_KEY) != 0;
   const bool want_v = (P.gradient_mask & ROSA_GRAD_VALUE) != 0;
   const bool want_qk = want_q || want_k;
-  const float symbol_scale = 0.5f * P.mismatch_scale / static_cast<float>(D);
+  // the contractions run on negated symbols
+  const float symbol_scale = -0.5f * P.mismatch_scale / static_cast<float>(D);
   float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
   float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
 
@@ -1331,7 +1344,7 @@ void vjp_gradients_kernel(VjpParams P) {
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
           utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, tile + 16, kTilePitch,
-                                 lane);
+                                 discard, lane);
           wave_lds_fence();
         }
         uint32_t route_hash = 0u;
@@ -1499,7 +1512,7 @@ void vjp_gradients_kernel(VjpParams P) {
               float query_b[DT];
               const uint32_t q_word = query_rows[local + r];
 #pragma unroll
-              for (int n = 0; n < DT; ++n) query_b[n] = sign_of_bit(q_word, 16 * n + li, D);
+              for (int n = 0; n < DT; ++n) query_b[n] = negated_symbol(q_word, 16 * n + li);
 #pragma unroll
               for (int m = 0; m < kWindowTiles; ++m) {
                 const float a_value = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
@@ -1515,15 +1528,26 @@ void vjp_gradients_kernel(VjpParams P) {
             v4f query_acc[DT];
 #pragma unroll
             for (int n = 0; n < DT; ++n) query_acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            // k slice lg of step s <-> window column 20 lg + s: every lane reads 20
+            // consecutive key words
+            uint32_t key_words[4 * kWindowTiles];
+#pragma unroll
+            for (int quad = 0; quad < kWindowTiles; ++quad) {
+              const uint4 four =
+                  *reinterpret_cast<const uint4*>(key_tile + 4 * kWindowTiles * lg + 4 * quad);
+              key_words[4 * quad] = four.x;
+              key_words[4 * quad + 1] = four.y;
+              key_words[4 * quad + 2] = four.z;
+              key_words[4 * quad + 3] = four.w;
+            }
 #pragma unroll
             for (int step = 0; step < 4 * kWindowTiles; ++step) {
-              const int c = 4 * step + lg;
+              const int c = 4 * kWindowTiles * lg + step;
               const float a_value = tile[li * kTilePitch + 16 + 64 - c + li];
-              const uint32_t k_word = key_tile[c];
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
-                query_acc[n] =
-                    mfma_16x16x4(a_value, sign_of_bit(k_word, 16 * n + li, D), query_acc[n]);
+                query_acc[n] = mfma_16x16x4(a_value, negated_symbol(key_words[step], 16 * n + li),
+                                            query_acc[n]);
               }
             }
 #pragma unroll
@@ -1878,7 +1902,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int GP = DVP;
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (1 + NVW) + SEG;
+                            SEG * kRowWords + (SEG + kWave) * (1 + NVW) + SEG + kWave;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
