@@ -100,22 +100,6 @@ __device__ __forceinline__ float dpp_add(float acc, float src) {
 }
 
 // Sum over the 64 lanes; the total is valid in lane 63 only.
-// lane `lane_index` (0..15, a constant after unrolling) of the result takes the
-// wave-uniform `value`, the others keep `old`
-__device__ __forceinline__ uint32_t write_lane(uint32_t value, int lane_index, uint32_t old) {
-#define ROSA_WRITE_LANE(n) \
-  case n: asm volatile("v_writelane_b32 %0, %1, " #n : "+v"(old) : "s"(value)); break;
-  switch (lane_index) {
-    ROSA_WRITE_LANE(0) ROSA_WRITE_LANE(1) ROSA_WRITE_LANE(2) ROSA_WRITE_LANE(3)
-    ROSA_WRITE_LANE(4) ROSA_WRITE_LANE(5) ROSA_WRITE_LANE(6) ROSA_WRITE_LANE(7)
-    ROSA_WRITE_LANE(8) ROSA_WRITE_LANE(9) ROSA_WRITE_LANE(10) ROSA_WRITE_LANE(11)
-    ROSA_WRITE_LANE(12) ROSA_WRITE_LANE(13) ROSA_WRITE_LANE(14) ROSA_WRITE_LANE(15)
-    default: break;
-  }
-#undef ROSA_WRITE_LANE
-  return old;
-}
-
 // The band kernels run one wavefront per block.  LDS instructions of one wave execute in
 // order, so data written by one lane is visible to another lane's later read without a
 // barrier; what is needed is that the compiler keeps the order, and nothing else: a full
@@ -182,6 +166,8 @@ __device__ __forceinline__ void store_sign(void* base, int64_t index, int sign) 
   }
 }
 
+// One round of the counter hash.  (The two 32-bit multiplies run at quarter rate; building
+// them from 16-bit dot products, v_dot2_u32_u16, was measured slower on gfx950.)
 __device__ __forceinline__ uint32_t mix32(uint32_t s) {
   s ^= s >> 16;
   s *= 0x7feb352du;
@@ -235,7 +221,7 @@ struct Layout {
 };
 
 // number of (row, band) steps of one (sequence, head) of length `len`, and the
-// number that precede band j: the index space of the cached keep masks
+// number that precede band j: the index space of the chunk records
 __host__ __device__ inline int64_t band_steps_total(int len) {
   if (len < 2) return 0;
   const int64_t bands = (len - 2) / 64 + 1;
@@ -246,11 +232,14 @@ __host__ __device__ inline int64_t band_steps_before(int len, int band) {
   return static_cast<int64_t>(band) * (len - 1) - 32 * static_cast<int64_t>(band) * (band - 1);
 }
 
-// The row-statistics pass leaves (S, window) of every diagonal before each 16th row of a
-// band; chunk c of the band with global step offset `steps_before` and global band
-// number `bands_before` owns slot steps_before / 16 + bands_before + c (distinct for all
+// The row-statistics pass leaves a record per 16-row chunk of a band for the gradient
+// pass: (S, window) of every diagonal before the chunk's first row and, with dropout,
+// the keep decisions of the chunk (bit r of lane l's 16-bit word = row r, diagonal l).
+// Chunk c of the band with global step offset `steps_before` and global band number
+// `bands_before` owns slot steps_before / 16 + bands_before + c (distinct for all
 // chunks of all bands, because a band of n steps has fewer than n / 16 + 2 chunks).
 constexpr int kCheckpointFloats = 128;  // [S | window][64 lanes]
+constexpr int kKeepBitFloats = 32;      // 64 lanes x 16 bits
 __host__ __device__ inline int64_t checkpoint_slots(int64_t steps, int64_t bands) {
   return steps / 16 + bands + 1;
 }
@@ -307,7 +296,7 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
                                          int32_t* __restrict__ seq_len,
                                          int32_t* __restrict__ block_prefix,
                                          int64_t* __restrict__ step_prefix, int H,
-                                         int64_t mask_capacity, int64_t checkpoint_capacity,
+                                         int64_t checkpoint_capacity,
                                          int32_t* __restrict__ header) {
   // single block; offsets are clamped into [previous, N] so that no later
   // kernel can index outside the tensors, and any violation is recorded.
@@ -349,14 +338,13 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
   }
   __syncthreads();
   if (threadIdx.x == 0 && step_prefix != nullptr) {
-    // index space of the cached keep masks; they are used only if they fit
+    // index space of the chunk records; they are used only if they fit
     int64_t steps = 0;
     for (int s = 0; s < S; ++s) {
       step_prefix[s] = steps;
       steps += band_steps_total(seq_len[s]);
     }
     step_prefix[S] = steps;
-    header[2] = steps * H <= mask_capacity ? 1 : 0;
     header[3] = checkpoint_slots(steps * H, static_cast<int64_t>(block_prefix[S]) * H) <=
                         checkpoint_capacity ? 1 : 0;
   }
@@ -560,9 +548,9 @@ struct VjpParams {
   float* grad_key;
   float* grad_value;
   int32_t* work_counter;
-  const int32_t* header;        // [0] offsets flag, [1] work counter, [2] keep masks fit, [3] checkpoints fit
-  unsigned long long* keep_masks;  // one 64-lane keep ballot per (band, row) step, or NULL
-  float* checkpoints;           // kCheckpointFloats per (band, 16-row chunk), or NULL
+  const int32_t* header;        // [0] offsets flag, [1] work counter, [3] chunk records fit
+  float* checkpoints;           // one record per (band, 16-row chunk), or NULL
+  int record_floats;            // kCheckpointFloats (+ kKeepBitFloats with dropout)
   float* block_scratch;         // per resident block: ring + segment checkpoints
   int64_t block_scratch_floats;
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
@@ -674,8 +662,8 @@ struct BandView {
   const uint32_t* vbits;   // value sign words of this (sequence, value head), NVW per token
   const float* grad_rows;  // [t][dvp]
   float4* stats;           // [t]
-  const unsigned long long* masks;  // cached keep ballots of this band (step i), or NULL
-  float* checkpoints;      // (S, window) before every 16th row of this band, or NULL
+  float* checkpoints;      // chunk records of this band, or NULL
+  int record_floats;
   int len;
   int diag0;               // first diagonal of the band
   int steps;               // rows of the band: t = diag0 + 1 + i
@@ -697,7 +685,7 @@ __device__ __forceinline__ void load_sliding(Band<NVW>& band, const BandView& vi
 //   0 query word of row t          1 query word of row t - W - 1
 //   2 key word entering at lane 0  3 key word of column a0 - W - 1 entering at lane 0
 //   4 exponent shift of the row    5 expected dropped utility
-//   6,7 cached dropout keep ballot of the step (lanes 0-31, 32-63)
+//   6,7 unused
 // In the row-statistics pass the shift is that of the raw weight; in the gradient
 // pass the row records are final and the shift includes log2 of the denominator,
 // so that exp2 gives the route probability directly.
@@ -723,13 +711,7 @@ __device__ __forceinline__ void stage_rows(const BandView& view, int first, int 
       dst[1] = make_uint4(__float_as_uint(fmaf(row.x, kLog2e, row.w)), 0u, 0u, 0u);
     } else if constexpr (DETAIL == kRowFull) {
       const uint4 record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
-      uint4 extra = make_uint4(record.y, record.z, 0u, 0u);
-      if (view.masks != nullptr) {
-        const unsigned long long ballot = view.masks[i];
-        extra.z = static_cast<uint32_t>(ballot);
-        extra.w = static_cast<uint32_t>(ballot >> 32);
-      }
-      dst[1] = extra;
+      dst[1] = make_uint4(record.y, record.z, 0u, 0u);
     }
   }
 }
@@ -916,13 +898,10 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
   }
   steps_before += band_steps_before(u.len, u.block);
   bands_before += u.block;
-  view.masks = nullptr;
-  if (P.keep_masks != nullptr && (!VARLEN || P.header[2] != 0)) {
-    view.masks = P.keep_masks + steps_before;
-  }
   view.checkpoints = nullptr;
+  view.record_floats = P.record_floats;
   if (P.checkpoints != nullptr && (!VARLEN || P.header[3] != 0)) {
-    view.checkpoints = P.checkpoints + ((steps_before >> 4) + bands_before) * kCheckpointFloats;
+    view.checkpoints = P.checkpoints + ((steps_before >> 4) + bands_before) * P.record_floats;
   }
   return true;
 }
@@ -986,8 +965,8 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 // Rows are processed 16 at a time without any branch in between.  A chunk leaves
 // its route weights and its dropped weighted utilities as two [row][lane] tiles
 // in LDS; their row sums are formed on the matrix cores and leave in one atomic
-// each from 16 lanes, and the 16 keep ballots kept for the gradient pass leave
-// as one store.
+// each from 16 lanes; every lane keeps its 16 dropout decisions of the chunk as bits and
+// stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   constexpr int kBlockRows = 32;     // rows staged in LDS at a time
@@ -1019,7 +998,6 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   band.window = 0;
   load_sliding<NVW>(band, view, 0, lane, W);
   const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
-  unsigned long long* mask_out = const_cast<unsigned long long*>(view.masks);
   uint32_t route_hash = route_hash_of(-lane);
   const int last_step = view.steps - 1;
   // without symbol gradients no utilities are computed and the tile stays zero
@@ -1037,7 +1015,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       const int chunk_first = first + local;
       if (view.checkpoints != nullptr) {
         float* slot =
-            view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * kCheckpointFloats;
+            view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
         slot[lane] = band.evidence;
         slot[kWave + lane] = __int_as_float(band.window);
       }
@@ -1047,7 +1025,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
                                kUtilityPitch, discard, lane);
         wave_lds_fence();
       }
-      uint32_t ballot_low = 0u, ballot_high = 0u;  // lane r: keep ballot of row r
+      uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
       // compiled twice: once every lane is past its window fill no masking is needed
       auto run_chunk = [&](auto steady_tag) {
         constexpr bool STEADY = decltype(steady_tag)::value;
@@ -1077,9 +1055,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
             route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
             key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
             keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-            const unsigned long long ballot = __ballot(keep != 0.0f);
-            ballot_low = write_lane(static_cast<uint32_t>(ballot), r, ballot_low);
-            ballot_high = write_lane(static_cast<uint32_t>(ballot >> 32), r, ballot_high);
+            kept_bits |= keep != 0.0f ? (1u << r) : 0u;
           }
           weights[r * kWeightPitch + lane] = weight;
           utilities[r * kUtilityPitch + lane] = weight * keep * utility;
@@ -1109,9 +1085,11 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       }
       if constexpr (DROPOUT) {
         // the gradient pass reads the decisions back instead of hashing again
-        if (lane < rows_here && mask_out != nullptr) {
-          mask_out[chunk_first + lane] =
-              (static_cast<unsigned long long>(ballot_high) << 32) | ballot_low;
+        if (view.checkpoints != nullptr) {
+          float* slot =
+              view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
+          reinterpret_cast<uint16_t*>(slot + kCheckpointFloats)[lane] =
+              static_cast<uint16_t>(kept_bits);
         }
       }
     }
@@ -1202,6 +1180,8 @@ void vjp_gradients_kernel(VjpParams P) {
   uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
   uint32_t* query_rows = value_window + (SEG + kWave) * NVW; // [SEG] query words of the rows
   float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
+  uint32_t* old_key_window = reinterpret_cast<uint32_t*>(discard + kWave);  // [SEG + 64] key words
+                                                             // of the columns W + 1 to the left
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1282,6 +1262,20 @@ void vjp_gradients_kernel(VjpParams P) {
     int ring_live = 0;            // rows for which the ring still holds non-zero terms
     int ring_fresh = 0;           // ring reads that must be treated as zero
     const int last_step = view.steps - 1;
+    // the record of the chunk after this one (the walk goes upwards) is always in flight
+    float ahead_evidence = 0.0f;
+    int ahead_window = 0;
+    uint32_t ahead_kept = 0u;
+    auto fetch_record = [&](int chunk_index) {
+      const float* slot =
+          view.checkpoints + static_cast<int64_t>(chunk_index) * view.record_floats;
+      ahead_evidence = slot[lane];
+      ahead_window = __float_as_int(slot[kWave + lane]);
+      if constexpr (DROPOUT) {
+        ahead_kept = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+      }
+    };
+    if (stored) fetch_record(last_step / kChunk);
 
     for (int segment = segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * SEG;
@@ -1307,6 +1301,7 @@ void vjp_gradients_kernel(VjpParams P) {
       for (int index = lane; index < SEG + kWave; index += kWave) {
         const int a = seg_first - 63 + index;  // column; key position a - 1
         key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
+        old_key_window[index] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
       }
       if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
       wave_lds_fence();
@@ -1326,16 +1321,19 @@ void vjp_gradients_kernel(VjpParams P) {
         const int local = chunk * kChunk;               // first row of the chunk inside the segment
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
+        uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
         if (stored) {
-          const float* slot =
-              view.checkpoints + static_cast<int64_t>(first / kChunk) * kCheckpointFloats;
-          band.evidence = slot[lane];
-          band.window = __float_as_int(slot[kWave + lane]);
+          band.evidence = ahead_evidence;
+          band.window = ahead_window;
+          kept_bits = ahead_kept;
+          if (first > 0) fetch_record(first / kChunk - 1);
         } else {
           band.evidence = ck_evidence[chunk * kWave + lane];
           band.window = ck_window[chunk * kWave + lane];
         }
-        load_sliding<NVW>(band, view, first, lane, W);
+        // sliding registers of the chunk's first step: column first - lane
+        band.key_word = key_window[local + 63 - lane];
+        band.old_key_word = old_key_window[local + 63 - lane];
         const float* grad_tile = grad_rows_lds + local * GP;
         const int t_first = view.diag0 + 1 + first;
         const int a_first = first + 1;  // column of lane 0 in the chunk's first row
@@ -1349,7 +1347,7 @@ void vjp_gradients_kernel(VjpParams P) {
         }
         uint32_t route_hash = 0u;
         if constexpr (DROPOUT) {
-          if (view.masks == nullptr) route_hash = route_hash_of(first - lane);
+          if (!stored) route_hash = route_hash_of(first - lane);
         }
         if (!want_qk) {  // no utilities were written: the replay must still read finite values
 #pragma unroll
@@ -1400,8 +1398,7 @@ void vjp_gradients_kernel(VjpParams P) {
             float keep = 1.0f;
             if constexpr (DROPOUT) {
               if constexpr (CACHED) {
-                const uint32_t ballot_half = lane >= 32 ? extra.w : extra.z;
-                const int kept = __builtin_amdgcn_sbfe(static_cast<int>(ballot_half), lane & 31, 1);
+                const int kept = __builtin_amdgcn_sbfe(static_cast<int>(kept_bits), r, 1);
                 keep = __int_as_float(__float_as_int(P.inverse_keep) & kept);
               } else {
                 route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
@@ -1421,7 +1418,7 @@ void vjp_gradients_kernel(VjpParams P) {
           }
         };
         const bool steady = first >= W + kWave && rows_here == kChunk;
-        const bool cached = DROPOUT && view.masks != nullptr;
+        const bool cached = DROPOUT && stored;
         if (steady) {
           if (cached) replay(std::true_type{}, std::true_type{});
           else replay(std::true_type{}, std::false_type{});
@@ -1727,10 +1724,10 @@ int padded_value_width(int Dv) {
 
 struct VjpWorkspace {
   size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows,
-      value_bits, keep_masks, block_scratch, total;
-  int64_t mask_capacity;  // 64-lane keep ballots that fit in the workspace (0: none kept)
+      value_bits, block_scratch, total;
   size_t checkpoints;
-  int64_t checkpoint_capacity;  // checkpoint slots that fit in the workspace (0: none kept)
+  int64_t checkpoint_capacity;  // chunk records that fit in the workspace (0: none kept)
+  int record_floats;
   int resident_blocks;
   int64_t block_scratch_floats;
   int ring_rows;
@@ -1753,32 +1750,19 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.grad_rows = cursor; cursor += align_up(sizeof(float) * rows * dvp);
   w.value_bits = cursor;
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
-  // Keep decisions of the dropout hash, one 64-lane ballot per (band, row)
-  // step (1 bit per pair): written by the row-statistics pass, read back by
-  // the gradient pass.  A packed batch is sized for its worst case (a single
-  // sequence) up to a budget; the device checks whether the real batch fits
-  // and otherwise hashes again.
-  w.keep_masks = cursor;
-  w.mask_capacity = 0;
-  if (dropout) {
-    const int64_t budget = (int64_t(3) << 29) / 8;  // 1.5 GiB of ballots
-    const int64_t wanted = v.L.varlen
-        ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
-        : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
-    w.mask_capacity = v.L.varlen ? std::min(wanted, budget) : (wanted <= 2 * budget ? wanted : 0);
-    cursor += align_up(sizeof(uint64_t) * static_cast<size_t>(w.mask_capacity));
-  }
-  // (S, window) checkpoints written by the row-statistics pass for the gradient pass,
-  // which otherwise rebuilds them with forward sweeps of its own
+  // Chunk records written by the row-statistics pass for the gradient pass, which
+  // otherwise rebuilds the evidence with forward sweeps of its own and evaluates the
+  // dropout hash a second time.
   w.checkpoints = cursor;
+  w.record_floats = kCheckpointFloats + (dropout ? kKeepBitFloats : 0);
   {
-    const int64_t budget = (int64_t(1) << 32) / (sizeof(float) * kCheckpointFloats);  // 4 GiB
+    const int64_t budget = (int64_t(1) << 32) / (sizeof(float) * w.record_floats);  // 4 GiB
     const int64_t steps = v.L.varlen
         ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
         : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
     const int64_t wanted = checkpoint_slots(steps, static_cast<int64_t>(v.L.slots) * v.L.H);
     w.checkpoint_capacity = v.L.varlen ? std::min(wanted, budget) : (wanted <= budget ? wanted : 0);
-    cursor += align_up(sizeof(float) * kCheckpointFloats *
+    cursor += align_up(sizeof(float) * w.record_floats *
                        static_cast<size_t>(w.checkpoint_capacity));
   }
   const int longest = v.L.varlen ? v.L.N : v.L.T;
@@ -1814,7 +1798,7 @@ unsigned blocks_for(int64_t items, int threads) {
 int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, size_t seq_start,
                              size_t seq_len, size_t block_prefix, size_t header,
                              hipStream_t stream, int64_t* step_prefix = nullptr,
-                             int64_t mask_capacity = 0, int64_t checkpoint_capacity = 0) {
+                             int64_t checkpoint_capacity = 0) {
   if (!L.varlen) return 0;
   L.seq_start = at<int32_t>(workspace, seq_start);
   L.seq_len = at<int32_t>(workspace, seq_len);
@@ -1822,8 +1806,8 @@ int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, 
   L.step_prefix = step_prefix;
   hipLaunchKernelGGL(prepare_sequences_kernel, dim3(1), dim3(256), 0, stream, p->cu_seqlens, L.S,
                      L.N, at<int32_t>(workspace, seq_start), at<int32_t>(workspace, seq_len),
-                     at<int32_t>(workspace, block_prefix), step_prefix, L.H, mask_capacity,
-                     checkpoint_capacity, at<int32_t>(workspace, header));
+                     at<int32_t>(workspace, block_prefix), step_prefix, L.H, checkpoint_capacity,
+                     at<int32_t>(workspace, header));
   return 0;
 }
 
@@ -1902,7 +1886,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int GP = DVP;
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (1 + NVW) + SEG + kWave;
+                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
@@ -1951,8 +1935,7 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   Layout L = view.L;
   const VjpWorkspace w = carve_vjp(view, dropout_p > 0.0f);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
-                           stream, at<int64_t>(workspace, w.step_prefix), w.mask_capacity,
-                           w.checkpoint_capacity);
+                           stream, at<int64_t>(workspace, w.step_prefix), w.checkpoint_capacity);
   const int dvp = padded_value_width(L.Dv);
   const int nvw = value_words(L.Dv);
   const int64_t symbol_elements = view.symbol_rows * L.D;
@@ -2019,8 +2002,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   P.grad_value = grad_value;
   P.work_counter = counter;
   P.header = at<int32_t>(workspace, w.header);
-  P.keep_masks = w.mask_capacity > 0 ? at<unsigned long long>(workspace, w.keep_masks) : nullptr;
   P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
+  P.record_floats = w.record_floats;
   P.block_scratch = at<float>(workspace, w.block_scratch);
   P.block_scratch_floats = w.block_scratch_floats;
   P.ring_rows = w.ring_rows;
