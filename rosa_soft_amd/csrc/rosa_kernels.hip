@@ -1182,6 +1182,7 @@ void vjp_gradients_kernel(VjpParams P) {
   float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
   uint32_t* old_key_window = reinterpret_cast<uint32_t*>(discard + kWave);  // [SEG + 64] key words
                                                              // of the columns W + 1 to the left
+  uint32_t* ck_kept = old_key_window + SEG + kWave;          // [SEG_CHUNKS][64] keep decisions
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1262,20 +1263,69 @@ void vjp_gradients_kernel(VjpParams P) {
     int ring_live = 0;            // rows for which the ring still holds non-zero terms
     int ring_fresh = 0;           // ring reads that must be treated as zero
     const int last_step = view.steps - 1;
-    // the record of the chunk after this one (the walk goes upwards) is always in flight
-    float ahead_evidence = 0.0f;
-    int ahead_window = 0;
-    uint32_t ahead_kept = 0u;
-    auto fetch_record = [&](int chunk_index) {
-      const float* slot =
-          view.checkpoints + static_cast<int64_t>(chunk_index) * view.record_floats;
-      ahead_evidence = slot[lane];
-      ahead_window = __float_as_int(slot[kWave + lane]);
-      if constexpr (DROPOUT) {
-        ahead_kept = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+    // The global atomics of a chunk are issued one chunk later, right before the next
+    // chunk's replay, so that their latency is covered by arithmetic instead of being
+    // waited for at the next chunk's first register reuse.
+    v4f done_value[VT];
+    v4f done_key[DT];
+    v4f done_query[DT];
+    int done_first = -1;  // first step of the chunk whose results are pending (-1: none)
+    int done_rows = 0;
+    auto issue_pending = [&]() {
+      if (done_first < 0) return;
+      const bool full = done_rows == kChunk;  // then every row and column of the chunk exists
+      const int64_t row0 = static_cast<int64_t>(u.start) + view.diag0 + 1 + done_first + 4 * lg;
+      const int64_t column0 = static_cast<int64_t>(u.start) + done_first + 1 + 4 * lg;
+      const int64_t last_token = static_cast<int64_t>(u.start) + view.len - 1;
+      const int64_t symbol_stride = static_cast<int64_t>(P.L.H) * D;
+      const int64_t value_stride = static_cast<int64_t>(P.L.Hv) * Dv;
+      if (want_q) {
+#pragma unroll
+        for (int n = 0; n < DT; ++n) {
+          const int bit = 16 * n + li;
+          if (bit < D) {
+            float* target = P.grad_query + (row0 * P.L.H + u.head) * D + bit;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (full || 4 * lg + e < done_rows) {
+                atomicAdd(target + e * symbol_stride, symbol_scale * done_query[n][e]);
+              }
+            }
+          }
+        }
       }
+      if (want_v) {
+#pragma unroll
+        for (int n = 0; n < VT; ++n) {
+          const int d = 16 * n + li;
+          if (d < Dv) {
+            float* target = P.grad_value + (column0 * P.L.Hv + hv) * Dv + d;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (full || column0 + e <= last_token) {
+                atomicAdd(target + e * value_stride, done_value[n][e]);
+              }
+            }
+          }
+        }
+      }
+      if (want_k) {
+#pragma unroll
+        for (int n = 0; n < DT; ++n) {
+          const int bit = 16 * n + li;
+          if (bit < D) {
+            float* target = P.grad_key + ((column0 - 1) * P.L.H + u.head) * D + bit;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (full || column0 + e <= last_token) {
+                atomicAdd(target + e * symbol_stride, symbol_scale * done_key[n][e]);
+              }
+            }
+          }
+        }
+      }
+      done_first = -1;
     };
-    if (stored) fetch_record(last_step / kChunk);
 
     for (int segment = segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * SEG;
@@ -1304,8 +1354,21 @@ void vjp_gradients_kernel(VjpParams P) {
         old_key_window[index] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
       }
       if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
-      wave_lds_fence();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
+      if (stored) {
+        // the chunk records of the segment: (S, window) before each chunk, keep decisions
+        for (int chunk = 0; chunk < chunks; ++chunk) {
+          const float* slot = view.checkpoints +
+              static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
+          ck_evidence[chunk * kWave + lane] = slot[lane];
+          ck_window[chunk * kWave + lane] = __float_as_int(slot[kWave + lane]);
+          if constexpr (DROPOUT) {
+            ck_kept[chunk * kWave + lane] =
+                reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+          }
+        }
+      }
+      wave_lds_fence();
       // segment-level forward sweep: checkpoint before every chunk
       for (int chunk = 0; !stored && chunk < chunks; ++chunk) {
         ck_evidence[chunk * kWave + lane] = band.evidence;
@@ -1321,21 +1384,13 @@ void vjp_gradients_kernel(VjpParams P) {
         const int local = chunk * kChunk;               // first row of the chunk inside the segment
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
-        uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
-        if (stored) {
-          band.evidence = ahead_evidence;
-          band.window = ahead_window;
-          kept_bits = ahead_kept;
-          if (first > 0) fetch_record(first / kChunk - 1);
-        } else {
-          band.evidence = ck_evidence[chunk * kWave + lane];
-          band.window = ck_window[chunk * kWave + lane];
-        }
+        band.evidence = ck_evidence[chunk * kWave + lane];
+        band.window = ck_window[chunk * kWave + lane];
+        const uint32_t kept_bits = DROPOUT ? ck_kept[chunk * kWave + lane] : 0u;  // bit r: row r kept
         // sliding registers of the chunk's first step: column first - lane
         band.key_word = key_window[local + 63 - lane];
         band.old_key_word = old_key_window[local + 63 - lane];
         const float* grad_tile = grad_rows_lds + local * GP;
-        const int t_first = view.diag0 + 1 + first;
         const int a_first = first + 1;  // column of lane 0 in the chunk's first row
         const uint32_t* key_tile = key_window + local;  // window column c <-> a = a_first - 64 + c
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
@@ -1345,6 +1400,7 @@ void vjp_gradients_kernel(VjpParams P) {
                                  discard, lane);
           wave_lds_fence();
         }
+        issue_pending();
         uint32_t route_hash = 0u;
         if constexpr (DROPOUT) {
           if (!stored) route_hash = route_hash_of(first - lane);
@@ -1522,9 +1578,14 @@ void vjp_gradients_kernel(VjpParams P) {
           }
           // row sums: rows are complete for this band after the chunk
           if (want_q) {
-            v4f query_acc[DT];
+            // four interleaved partial sums: no product waits for the one before it
+            constexpr int kParts = 4;
+            v4f query_part[kParts][DT];
 #pragma unroll
-            for (int n = 0; n < DT; ++n) query_acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int part = 0; part < kParts; ++part) {
+#pragma unroll
+              for (int n = 0; n < DT; ++n) query_part[part][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            }
             // k slice lg of step s <-> window column 20 lg + s: every lane reads 20
             // consecutive key words
             uint32_t key_words[4 * kWindowTiles];
@@ -1543,54 +1604,28 @@ void vjp_gradients_kernel(VjpParams P) {
               const float a_value = tile[li * kTilePitch + 16 + 64 - c + li];
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
-                query_acc[n] = mfma_16x16x4(a_value, negated_symbol(key_words[step], 16 * n + li),
-                                            query_acc[n]);
+                query_part[step % kParts][n] =
+                    mfma_16x16x4(a_value, negated_symbol(key_words[step], 16 * n + li),
+                                 query_part[step % kParts][n]);
               }
             }
 #pragma unroll
             for (int n = 0; n < DT; ++n) {
-              const int bit = 16 * n + li;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int r = 4 * lg + e;
-                if (bit < D && r < rows_here) {
-                  const int64_t token = static_cast<int64_t>(u.start) + t_first + r;
-                  atomicAdd(&P.grad_query[(token * P.L.H + u.head) * D + bit],
-                            symbol_scale * query_acc[n][e]);
-                }
-              }
+              done_query[n] = (query_part[0][n] + query_part[1][n]) +
+                              (query_part[2][n] + query_part[3][n]);
             }
           }
         }
-        // the last window tile (columns a_first .. a_first + 15) is complete: flush it,
-        // then shift the window up by one tile
+        // the last window tile (columns a_first .. a_first + 15) is complete: park it with
+        // the chunk's row sums, then shift the window up by one tile
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int a = a_first + 4 * lg + e;
-          if (a <= view.len - 1) {
-            const int64_t token = static_cast<int64_t>(u.start) + a;
-            if (want_v) {
+        for (int n = 0; n < VT; ++n) done_value[n] = value_acc[kWindowTiles - 1][n];
 #pragma unroll
-              for (int n = 0; n < VT; ++n) {
-                const int d = 16 * n + li;
-                if (d < Dv) {
-                  atomicAdd(&P.grad_value[(token * P.L.Hv + hv) * Dv + d],
-                            value_acc[kWindowTiles - 1][n][e]);
-                }
-              }
-            }
-            if (want_k) {
-#pragma unroll
-              for (int n = 0; n < DT; ++n) {
-                const int bit = 16 * n + li;
-                if (bit < D) {
-                  atomicAdd(&P.grad_key[((token - 1) * P.L.H + u.head) * D + bit],
-                            symbol_scale * key_acc[kWindowTiles - 1][n][e]);
-                }
-              }
-            }
-          }
-        }
+        for (int n = 0; n < DT; ++n) done_key[n] = key_acc[kWindowTiles - 1][n];
+        done_first = first;
+        done_rows = rows_here;
+        // wide tiles have no registers to spare for carrying the results across a chunk
+        if constexpr (VT > 1 || DT > 1) issue_pending();
 #pragma unroll
         for (int m = kWindowTiles - 1; m > 0; --m) {
 #pragma unroll
@@ -1605,6 +1640,7 @@ void vjp_gradients_kernel(VjpParams P) {
         wave_lds_fence();
       }
     }
+    issue_pending();
   }
 }
 
@@ -1886,7 +1922,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int GP = DVP;
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave;
+                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave + (SEG / kChunk) * kWave;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
