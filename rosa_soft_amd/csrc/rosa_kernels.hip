@@ -772,15 +772,25 @@ __device__ __forceinline__ RowSymbols staged_symbols(const uint32_t* row) {
 // One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
 // STEADY: every lane of the wave is past its diagonal's first W + 1 rows, so no
 // lane needs masking (true for all but the first W + 64 rows of a band).
-template <int NVW, bool STEADY = false>
+// QUIET (with STEADY): the caller knows that no overflow term of these rows can move
+// a float32 result; the window is not tracked and the overflow is taken as zero.
+template <int NVW, bool STEADY = false, bool QUIET = false>
 __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbols& symbols, int i,
                                                 int lane, int W, float gate_log2) {
   const int a0 = i + 1;
   band.key_word = dpp_wave_shr1(symbols.key, band.key_word);
-  band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
   StepOut out;
   out.a = a0 - lane;
   const int mismatches = __popc(symbols.query ^ band.key_word);
+  if constexpr (STEADY && QUIET) {
+    out.active = true;
+    out.gate = fast_exp2(-gate_log2 * static_cast<float>(mismatches));
+    out.overflow = 0.0f;
+    band.evidence = fmaf(out.gate, band.evidence, out.gate);
+    out.evidence = band.evidence;
+    return out;
+  }
+  band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
   if constexpr (STEADY) {
     out.active = true;
     band.window += mismatches - __popc(symbols.old_query ^ band.old_key_word);
@@ -1017,8 +1027,9 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
         float* slot =
             view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
         slot[lane] = band.evidence;
-        slot[kWave + lane] = __int_as_float(band.window);
       }
+      const int window_before = band.window;
+      float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
         utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
@@ -1046,6 +1057,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           const int i = min(chunk_first + r, last_step);
           const int t = view.diag0 + 1 + i;
           const StepOut s = forward_step<NVW, STEADY>(band, symbols, i, lane, W, P.gate_log2);
+          peak_overflow = fmaxf(peak_overflow, s.overflow);
           const float one_plus = 1.0f + s.evidence;
           const float root = one_plus * fast_rsq(one_plus);
           const bool live = STEADY || (s.active && r < rows_here);
@@ -1083,11 +1095,15 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           if (needs_utility) atomicAdd(&row_stats->z, numerator_sum);
         }
       }
-      if constexpr (DROPOUT) {
-        // the gradient pass reads the decisions back instead of hashing again
-        if (view.checkpoints != nullptr) {
-          float* slot =
-              view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
+      if (view.checkpoints != nullptr) {
+        float* slot =
+            view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
+        // the sign bit of the window word tells the gradient pass that some overflow term
+        // of the chunk is large enough to matter
+        const bool noisy = __ballot(peak_overflow >= P.tail_threshold) != 0ull;
+        slot[kWave + lane] = __int_as_float(window_before | (noisy ? INT32_MIN : 0));
+        if constexpr (DROPOUT) {
+          // the gradient pass reads the decisions back instead of hashing again
           reinterpret_cast<uint16_t*>(slot + kCheckpointFloats)[lane] =
               static_cast<uint16_t>(kept_bits);
         }
@@ -1194,6 +1210,7 @@ void vjp_gradients_kernel(VjpParams P) {
   const bool want_k = (P.gradient_mask & ROSA_GRAD_KEY) != 0;
   const bool want_v = (P.gradient_mask & ROSA_GRAD_VALUE) != 0;
   const bool want_qk = want_q || want_k;
+  const float adjoint_gain = 0.5f * kSqrtScale * P.scale;  // scale * U'(S) * sqrt(1 + S)
   // the contractions run on negated symbols
   const float symbol_scale = -0.5f * P.mismatch_scale / static_cast<float>(D);
   float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
@@ -1385,7 +1402,10 @@ void vjp_gradients_kernel(VjpParams P) {
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
         band.evidence = ck_evidence[chunk * kWave + lane];
-        band.window = ck_window[chunk * kWave + lane];
+        const int window_word = ck_window[chunk * kWave + lane];
+        band.window = window_word & INT32_MAX;
+        // stored records say whether any overflow term of the chunk matters
+        const bool chunk_quiet = stored && __builtin_amdgcn_readfirstlane(window_word) >= 0;
         const uint32_t kept_bits = DROPOUT ? ck_kept[chunk * kWave + lane] : 0u;  // bit r: row r kept
         // sliding registers of the chunk's first step: column first - lane
         band.key_word = key_window[local + 63 - lane];
@@ -1419,9 +1439,10 @@ void vjp_gradients_kernel(VjpParams P) {
         // the general form rows past the end of the band (only in the band's last
         // chunk) repeat the last row's data and are masked, which keeps the loop
         // free of branches.
-        auto replay = [&](auto steady_tag, auto cached_tag) {
+        auto replay = [&](auto steady_tag, auto cached_tag, auto quiet_tag) {
           constexpr bool STEADY = decltype(steady_tag)::value;
           constexpr bool CACHED = decltype(cached_tag)::value;  // keep decisions are read back
+          constexpr bool QUIET = decltype(quiet_tag)::value;    // overflow terms are negligible
           const uint32_t* row = rows + local * kRowWords;
           const float* slot = tile + 16 + lane;
           uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
@@ -1445,7 +1466,8 @@ void vjp_gradients_kernel(VjpParams P) {
             const int t = view.diag0 + 1 + i;
             const float shift = __uint_as_float(extra.x);
             const float expected = __uint_as_float(extra.y);
-            const StepOut s = forward_step<NVW, STEADY>(band, symbols, i, lane, W, P.gate_log2);
+            const StepOut s =
+                forward_step<NVW, STEADY, QUIET>(band, symbols, i, lane, W, P.gate_log2);
             const float one_plus = 1.0f + s.evidence;
             const float inv_root = fast_rsq(one_plus);
             const float root = one_plus * inv_root;
@@ -1462,8 +1484,8 @@ void vjp_gradients_kernel(VjpParams P) {
                 keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
               }
             }
-            const float adjoint = P.scale * probability * (keep * utility - expected) *
-                                  (0.5f * kSqrtScale * inv_root);
+            const float adjoint =
+                (probability * adjoint_gain) * (keep * utility - expected) * inv_root;
             tile[r * kTilePitch + 16 + lane] = probability * keep;
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
@@ -1475,12 +1497,15 @@ void vjp_gradients_kernel(VjpParams P) {
         };
         const bool steady = first >= W + kWave && rows_here == kChunk;
         const bool cached = DROPOUT && stored;
-        if (steady) {
-          if (cached) replay(std::true_type{}, std::true_type{});
-          else replay(std::true_type{}, std::false_type{});
+        if (steady && chunk_quiet) {
+          if (cached) replay(std::true_type{}, std::true_type{}, std::true_type{});
+          else replay(std::true_type{}, std::false_type{}, std::true_type{});
+        } else if (steady) {
+          if (cached) replay(std::true_type{}, std::true_type{}, std::false_type{});
+          else replay(std::true_type{}, std::false_type{}, std::false_type{});
         } else {
-          if (cached) replay(std::false_type{}, std::true_type{});
-          else replay(std::false_type{}, std::false_type{});
+          if (cached) replay(std::false_type{}, std::true_type{}, std::false_type{});
+          else replay(std::false_type{}, std::false_type{}, std::false_type{});
         }
         wave_lds_fence();
 
@@ -1509,11 +1534,7 @@ void vjp_gradients_kernel(VjpParams P) {
         if (want_qk) {
           wave_lds_fence();
           // reverse walk of the chunk: gate adjoints replace the weights
-          float peak_overflow = keep_overflow[0];
-#pragma unroll
-          for (int r = 1; r < kChunk; ++r) peak_overflow = fmaxf(peak_overflow, keep_overflow[r]);
-          const bool quiet = steady && ring_live == 0 &&
-                             __ballot(peak_overflow >= P.tail_threshold) == 0ull;
+          const bool quiet = steady && chunk_quiet && ring_live == 0;
           if (quiet) {
             // no overflow term of the chunk can move a gradient and the ring is empty:
             // h = b (S + o), nothing to mask
