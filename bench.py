@@ -141,9 +141,9 @@ def run_step(rosa, config, leaves, cu_seqlens):
 def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
     """Time the CPU oracle (a port, float64, OpenMP) on a slice of the workload.
 
-    The slice is one batch element and one value-head group over a prefix of
-    the sequence chosen so that the run stays near the budget; its time is
-    scaled by the pair count to the whole workload.
+    The slice is one batch element, a prefix of the sequence and a number of
+    value-head groups chosen so that the run takes about 10 to 30 s; its time
+    is scaled by the pair count to the whole workload.
     """
 
     from oracle import c_oracle
@@ -153,14 +153,15 @@ def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
         start, end = int(cu_seqlens[0]), int(cu_seqlens[1])
         query, key, value = (t[start:end].unsqueeze(0) for t in (query, key, value))
     group = config["H"] // config["Hv"]
-    query, key, value = query[:1, :, :group], key[:1, :, :group], value[:1, :, :1]
     threads = c_oracle.num_threads()
     rows = min(query.size(1), 512)
-    grad_output = None
+    groups = 1  # value-head groups in the slice
     elapsed = 0.0
     while True:
-        q, k, v = (t[:, :rows].contiguous() for t in (query, key, value))
-        grad_output = torch.ones(1, rows, group, config["Dv"]) / (rows * group * config["Dv"])
+        heads = groups * group
+        q, k = (t[:1, :rows, :heads].contiguous() for t in (query, key))
+        v = value[:1, :rows, :groups].contiguous()
+        grad_output = torch.ones(1, rows, heads, config["Dv"]) / (rows * heads * config["Dv"])
         begin = time.perf_counter()
         out, _, _ = c_oracle.hard_forward(q, k, v, config["W"])
         forward_seconds = time.perf_counter() - begin
@@ -169,9 +170,15 @@ def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
             dropout_p=config["p"], mismatch_scale=config["ms"], seed=12345 if config["p"] > 0 else None,
         )
         elapsed = time.perf_counter() - begin
-        if rows >= query.size(1) or elapsed * 4.0 > budget_seconds:
+        if elapsed * 4.0 > budget_seconds:
             break
-        rows = min(query.size(1), rows * 2)
+        if rows < query.size(1):  # first grow the sequence prefix (work grows 4x) ...
+            rows = min(query.size(1), rows * 2)
+        elif groups < config["Hv"]:  # ... then the number of value-head groups
+            groups = min(config["Hv"], groups * 4)
+        else:
+            break
+    group = groups * group
     slice_pairs = group * rows * (rows - 1) // 2
     seconds_full = elapsed * pair_count(config) / max(slice_pairs, 1)
     return dict(
