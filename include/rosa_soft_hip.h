@@ -79,6 +79,21 @@ int rosa_hip_hard_forward(const rosa_problem* problem, const void* query,
                           size_t workspace_bytes, void* stream);
 
 /*
+ * Hard forward that also reports what it selected: `routes` as above and
+ * `lengths`, the exact matched suffix length of the selected route (0 for the
+ * null route), both optional int32 tensors in the packed-symbol layout.  This
+ * is the selected-route part of inspect_rosa_soft (rosa_soft/testing.py:28-117:
+ * selected_route_indices, and exact_suffix_lengths taken at the selected route)
+ * without its O(T^2) tensors, so route statistics such as
+ * examples/fit_soft_reference.py:419-459 can be computed at training shapes.
+ */
+int rosa_hip_hard_routes(const rosa_problem* problem, const void* query,
+                         const void* key, const void* value, void* output,
+                         int32_t* packed_query, int32_t* packed_key,
+                         int32_t* routes, int32_t* lengths, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/*
  * Dense surrogate VJP.  Replaces surrogate_vjp_cuda (rosa_soft_kernels.cu:1923-2379)
  * and surrogate_vjp_varlen_cuda (:2382-2638).  Gradients are float32 in the
  * layout of the corresponding input and are fully overwritten; pass NULL for

@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_forward_workspace_bytes",
     "rosa_hip_vjp_workspace_bytes",
     "rosa_hip_hard_forward",
+    "rosa_hip_hard_routes",
     "rosa_hip_surrogate_vjp",
     "rosa_hip_read_offset_error",
     "rosa_hip_stage_timing",
@@ -84,6 +85,10 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_hard_forward.restype = ctypes.c_int
     library.rosa_hip_hard_forward.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_hard_routes.restype = ctypes.c_int
+    library.rosa_hip_hard_routes.argtypes = [
+        problem_p, vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
     ]
     library.rosa_hip_surrogate_vjp.restype = ctypes.c_int
     library.rosa_hip_surrogate_vjp.argtypes = [
@@ -181,6 +186,49 @@ def hard_forward(
         )
     _check(status, "rosa_hip_hard_forward")
     return output, packed_q, packed_k, routes
+
+
+def hard_routes(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    max_suffix_length: int,
+    cu_seqlens: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Hard forward with its selection: ``(output, routes, lengths)``.
+
+    ``routes`` and ``lengths`` are int32 in the layout of the inputs without the
+    feature axis (``[B, T, H]`` dense, ``[N, H]`` packed): the selected route
+    index local to its sequence (0 = null route) and the exact matched suffix
+    length of that route (0 for the null route).
+    """
+
+    library = load()
+    assert query.is_cuda and query.is_contiguous() and key.is_contiguous() and value.is_contiguous()
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    if cu_seqlens is None:
+        word_shape = (problem.B, problem.H, problem.T)
+        out_shape = (problem.B, problem.T, problem.H, problem.Dv)
+    else:
+        word_shape = (problem.H, problem.N)
+        out_shape = (problem.N, problem.H, problem.Dv)
+    with torch.cuda.device(query.device):
+        output = torch.empty(out_shape, dtype=query.dtype, device=query.device)
+        words = [torch.empty(word_shape, dtype=torch.int32, device=query.device) for _ in range(4)]
+        size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
+        workspace = torch.empty(max(size, 256), dtype=torch.uint8, device=query.device)
+        status = library.rosa_hip_hard_routes(
+            ctypes.byref(problem), _ptr(query), _ptr(key), _ptr(value), _ptr(output),
+            _ptr(words[0]), _ptr(words[1]), _ptr(words[2]), _ptr(words[3]), _ptr(workspace),
+            workspace.numel(), _stream(query),
+        )
+    _check(status, "rosa_hip_hard_routes")
+    # head-major words -> the layout of the inputs
+    if cu_seqlens is None:
+        routes, lengths = (w.permute(0, 2, 1).contiguous() for w in words[2:])
+    else:
+        routes, lengths = (w.t().contiguous() for w in words[2:])
+    return output, routes, lengths
 
 
 def surrogate_vjp(

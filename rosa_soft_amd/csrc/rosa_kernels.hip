@@ -438,7 +438,7 @@ template <bool VARLEN, bool WIDE>
 __global__ __launch_bounds__(kWave) void hard_route_kernel(
     Layout L, const uint32_t* __restrict__ packed_query,
     const uint32_t* __restrict__ packed_key, int32_t* __restrict__ routes,
-    int32_t* __restrict__ source_token, int shift) {
+    int32_t* __restrict__ lengths, int32_t* __restrict__ source_token, int shift) {
   const Unit u = decode_unit<VARLEN>(L, blockIdx.x);
   if (!u.valid) return;
   const int blocks = (u.len + 63) >> 6;
@@ -492,6 +492,7 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
   }
   const int route = best_run > 0 ? best_route : 0;
   if (routes != nullptr) routes[u.word_base + t] = route;
+  if (lengths != nullptr) lengths[u.word_base + t] = best_run;
   source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
 }
 
@@ -1871,7 +1872,8 @@ int launch_prepare_sequences(const rosa_problem* p, Layout& L, void* workspace, 
 template <int DTYPE>
 int run_forward(const rosa_problem* p, const ProblemView& view, const void* query,
                 const void* key, const void* value, void* output, int32_t* packed_query,
-                int32_t* packed_key, int32_t* routes, void* workspace, hipStream_t stream) {
+                int32_t* packed_key, int32_t* routes, int32_t* lengths, void* workspace,
+                hipStream_t stream) {
   Layout L = view.L;
   const ForwardWorkspace w = carve_forward(view);
   stage_begin(kStageForward, stream);
@@ -1898,18 +1900,18 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   if (L.varlen) {
     if (wide) {
       hipLaunchKernelGGL((hard_route_kernel<true, true>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift);
     } else {
       hipLaunchKernelGGL((hard_route_kernel<true, false>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift);
     }
   } else {
     if (wide) {
       hipLaunchKernelGGL((hard_route_kernel<false, true>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift);
     } else {
       hipLaunchKernelGGL((hard_route_kernel<false, false>), dim3(units), dim3(kWave), 0, stream,
-                         L, pq, pk, routes, source_token, shift);
+                         L, pq, pk, routes, lengths, source_token, shift);
     }
   }
   const int64_t out_elements = view.symbol_rows * L.Dv;
@@ -2116,10 +2118,10 @@ size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_ma
   return carve_vjp(view, dropout != 0).total;
 }
 
-int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const void* key,
-                          const void* value, void* output, int32_t* packed_query,
-                          int32_t* packed_key, int32_t* routes, void* workspace,
-                          size_t workspace_bytes, void* stream) {
+int rosa_hip_hard_routes(const rosa_problem* problem, const void* query, const void* key,
+                         const void* value, void* output, int32_t* packed_query,
+                         int32_t* packed_key, int32_t* routes, int32_t* lengths,
+                         void* workspace, size_t workspace_bytes, void* stream) {
   ProblemView view;
   const int bad = check_problem(problem, &view);
   if (bad != 0) return bad;
@@ -2130,14 +2132,22 @@ int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const 
   switch (problem->dtype) {
     case ROSA_DTYPE_F32:
       return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
-                                         packed_key, routes, workspace, s);
+                                         packed_key, routes, lengths, workspace, s);
     case ROSA_DTYPE_F16:
       return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
-                                         packed_key, routes, workspace, s);
+                                         packed_key, routes, lengths, workspace, s);
     default:
       return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
-                                          packed_key, routes, workspace, s);
+                                          packed_key, routes, lengths, workspace, s);
   }
+}
+
+int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const void* key,
+                          const void* value, void* output, int32_t* packed_query,
+                          int32_t* packed_key, int32_t* routes, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  return rosa_hip_hard_routes(problem, query, key, value, output, packed_query, packed_key,
+                              routes, nullptr, workspace, workspace_bytes, stream);
 }
 
 int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const void* key,

@@ -325,3 +325,58 @@ def test_device_matches_reference_golden_vectors(cabi):
         rtol, atol = bars[dtype]
         for label, got in zip(("gq", "gk", "gv"), grads):
             torch.testing.assert_close(got.cpu(), torch.from_numpy(vectors[name + "/" + label]), rtol=rtol, atol=atol)
+
+
+# --------------------------------------------------------------------------- selection side channel
+
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,pattern", [
+    (2, 130, 2, 4, 1, 5, 16, "random"),
+    (1, 300, 2, 3, 2, 4, 40, "shifted"),
+    (1, 193, 1, 8, 1, 8, 128, "all_match"),
+    (1, 150, 2, 2, 1, 7, 9, "periodic"),
+])
+def test_selected_routes_and_suffix_lengths_match_oracle(cabi, c_oracle, B, T, H, D, Hv, Dv, W,
+                                                         pattern):
+    # selected_route_indices and the exact suffix length at the selected route, the part of
+    # the reference's inspection (rosa_soft/testing.py:28-117) the device can report
+    from rosa_soft_amd.diagnostics import inspect_hard_routes
+
+    query, key, value, _ = make_case(B, T, H, D, Hv, Dv, seed=T + 3, pattern=pattern)
+    output, inspection = inspect_hard_routes(
+        query.to(DEVICE), key.to(DEVICE), value.to(DEVICE), max_suffix_length=W
+    )
+    want_out, want_routes, want_lengths = c_oracle.hard_forward(query, key, value, W)
+    assert torch.equal(output.cpu(), want_out)
+    assert inspection.selected_route_indices.shape == (B, T, H)
+    assert torch.equal(inspection.selected_route_indices.cpu(), want_routes.permute(0, 2, 1))
+    assert torch.equal(inspection.selected_suffix_lengths.cpu(), want_lengths.permute(0, 2, 1))
+    assert inspection.effective_max_suffix_length == min(W, T)
+    stats = inspection.route_stats()
+    assert 0.0 <= stats["null_rate"] <= 1.0 and stats["max_match_length"] <= min(W, T)
+    # the null route has length 0 and only the null route has
+    assert torch.equal(inspection.null_route_mask, inspection.selected_suffix_lengths == 0)
+
+
+def test_selected_routes_of_a_packed_batch(cabi, c_oracle):
+    from rosa_soft_amd.diagnostics import inspect_hard_routes
+
+    lengths = [5, 0, 70, 1, 129]
+    total = sum(lengths)
+    query = nonzero_randn((total, 2, 3), seed=21)
+    key = nonzero_randn((total, 2, 3), seed=22)
+    value = nonzero_randn((total, 1, 4), seed=23)
+    offsets = torch.tensor([0] + list(np.cumsum(lengths)), dtype=torch.int32)
+    output, inspection = inspect_hard_routes(
+        query.to(DEVICE), key.to(DEVICE), value.to(DEVICE), offsets.to(DEVICE), max_suffix_length=12
+    )
+    assert inspection.selected_route_indices.shape == (total, 2)
+    for start, length in zip(offsets[:-1].tolist(), lengths):
+        if length == 0:
+            continue
+        piece = slice(start, start + length)
+        want_out, want_routes, want_lengths = c_oracle.hard_forward(
+            query[piece].unsqueeze(0), key[piece].unsqueeze(0), value[piece].unsqueeze(0), 12
+        )
+        assert torch.equal(output[piece].cpu(), want_out[0])
+        assert torch.equal(inspection.selected_route_indices[piece].cpu(), want_routes[0].t())
+        assert torch.equal(inspection.selected_suffix_lengths[piece].cpu(), want_lengths[0].t())
