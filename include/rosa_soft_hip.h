@@ -111,6 +111,41 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
                            void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Streaming hard router: the device-resident counterpart of RosaRuntime::update_packed
+ * (rosa_soft/csrc/rosa_runtime.cpp:333-487), whose per-(slot, head) suffix automaton
+ * (:34-227) answers, for every new token, "which earlier key position ends the longest
+ * (at most W) match of the query suffix, latest on ties".  Here every (slot, head) keeps
+ * its masked query, key and payload symbols as bytes in caller-owned device memory
+ * (`capacity` bytes per run, layouts [S][H][capacity] and [S][Hp][capacity]) and an
+ * update appends the chunk and routes its rows against all earlier keys with the kernel
+ * of the hard forward.  Outputs follow the reference: `matched_key_end` int64 [tokens][H],
+ * the global key end position in the slot's history or -1; `output` uint8 [tokens][H], the
+ * payload symbol after the matched key, 0 for the null route.  `chunk_offsets` [S+1] and
+ * `history_lengths` [S] are device int32; the caller checks that
+ * history_lengths[s] + chunk length <= capacity and advances the lengths afterwards.
+ * `longest_chunk` is the largest number of new tokens of any slot.
+ */
+typedef struct rosa_router_update {
+  int32_t S, H, Hp, W;
+  int32_t qk_bits, payload_bits;
+  int32_t capacity;
+  int32_t tokens;
+  int32_t longest_chunk;
+  const int32_t* chunk_offsets;
+  const int32_t* history_lengths;
+  uint8_t* query_history;
+  uint8_t* key_history;
+  uint8_t* payload_history;
+  const uint8_t* query;
+  const uint8_t* key;
+  const uint8_t* payload;
+  uint8_t* output;
+  int64_t* matched_key_end;
+} rosa_router_update;
+
+int rosa_hip_router_update(const rosa_router_update* update, void* stream);
+
+/*
  * Asynchronous device-side diagnostics.  Invalid cu_seqlens values (not
  * starting at 0, decreasing, or not ending at N) cannot be seen by the host
  * without a synchronisation, so the kernels clamp them to a safe range, and

@@ -83,7 +83,7 @@ class BuildCapabilities:
 BUILD_CAPABILITIES = BuildCapabilities(
     variant="rocm" if _has_device_operators else "reference",
     compiled_extension=_has_compiled_extension,
-    rosa_runtime=False,
+    rosa_runtime=_has_device_operators,
     rosa_soft_cuda=_has_device_operators,
 )
 
@@ -114,14 +114,15 @@ else:
         _raise_unavailable("rosa_soft_varlen training operator", _BUILD_HINT)
 
 
-class RosaRuntime:
-    """The CPU hard-inference runtime is not part of this build."""
+if _has_device_operators:
+    from .runtime import RosaRuntime
+else:
 
-    def __init__(self, *args, **kwargs):
-        _raise_unavailable(
-            "RosaRuntime",
-            "This package covers the training operators only.",
-        )
+    class RosaRuntime:
+        """The device-resident hard router needs the HIP library."""
+
+        def __init__(self, *args, **kwargs):
+            _raise_unavailable("RosaRuntime", _BUILD_HINT)
 
 
 def rosa_soft_reference(*args, **kwargs):

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_surrogate_vjp",
+    "rosa_hip_router_update",
     "rosa_hip_read_offset_error",
     "rosa_hip_stage_timing",
     "rosa_hip_stage_count",
@@ -53,6 +54,32 @@ class RosaProblem(ctypes.Structure):
         ("Dv", ctypes.c_int),
         ("W", ctypes.c_int),
         ("cu_seqlens", ctypes.c_void_p),
+    ]
+
+
+class RosaRouterUpdate(ctypes.Structure):
+    """``rosa_router_update`` of ``include/rosa_soft_hip.h``."""
+
+    _fields_ = [
+        ("S", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Hp", ctypes.c_int32),
+        ("W", ctypes.c_int32),
+        ("qk_bits", ctypes.c_int32),
+        ("payload_bits", ctypes.c_int32),
+        ("capacity", ctypes.c_int32),
+        ("tokens", ctypes.c_int32),
+        ("longest_chunk", ctypes.c_int32),
+        ("chunk_offsets", ctypes.c_void_p),
+        ("history_lengths", ctypes.c_void_p),
+        ("query_history", ctypes.c_void_p),
+        ("key_history", ctypes.c_void_p),
+        ("payload_history", ctypes.c_void_p),
+        ("query", ctypes.c_void_p),
+        ("key", ctypes.c_void_p),
+        ("payload", ctypes.c_void_p),
+        ("output", ctypes.c_void_p),
+        ("matched_key_end", ctypes.c_void_p),
     ]
 
 
@@ -90,6 +117,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_hard_routes.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
     ]
+    library.rosa_hip_router_update.restype = ctypes.c_int
+    library.rosa_hip_router_update.argtypes = [ctypes.POINTER(RosaRouterUpdate), vp]
     library.rosa_hip_surrogate_vjp.restype = ctypes.c_int
     library.rosa_hip_surrogate_vjp.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp,
@@ -281,6 +310,16 @@ def vjp_workspace_bytes(query: Tensor, value: Tensor, max_suffix_length: int,
                         cu_seqlens: Optional[Tensor] = None) -> int:
     problem = make_problem(query, value, max_suffix_length, cu_seqlens)
     return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0))
+
+
+def router_update(update: RosaRouterUpdate, device: torch.device) -> None:
+    """Enqueue one streaming-router update on the current stream of ``device``."""
+
+    with torch.cuda.device(device):
+        status = load().rosa_hip_router_update(
+            ctypes.byref(update), torch.cuda.current_stream(device).cuda_stream
+        )
+    _check(status, "rosa_hip_router_update")
 
 
 def stage_timing(enable: bool) -> None:

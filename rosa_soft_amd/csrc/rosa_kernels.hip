@@ -2089,6 +2089,108 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   return 0;
 }
 
+
+// ---------------------------------------------------------------------------
+// streaming hard router (inference): the hard forward over a growing history
+// ---------------------------------------------------------------------------
+//
+// Every (slot, head) keeps its query, key and payload symbols (one byte each) in
+// device memory, `capacity` bytes per run.  An update appends a chunk of tokens to
+// every slot and routes exactly the new rows against all keys before them; the
+// answer per row is the end position of the matched key (route - 1, or -1 for the
+// null route) and the payload symbol that follows it.
+
+struct RouterUpdate {
+  int S, H, Hp, W;
+  int capacity;
+  int qk_mask, payload_mask;
+  const int32_t* chunk_offsets;  // [S + 1] token offsets of the chunk, per slot
+  const int32_t* history_lengths;  // [S] tokens a slot held before this chunk
+  uint8_t* query_history;        // [S][H][capacity]
+  uint8_t* key_history;          // [S][H][capacity]
+  uint8_t* payload_history;      // [S][Hp][capacity]
+  const uint8_t* query;          // [tokens][H]
+  const uint8_t* key;            // [tokens][H]
+  const uint8_t* payload;        // [tokens][Hp]
+  uint8_t* output;               // [tokens][H]
+  int64_t* matched_key_end;      // [tokens][H]
+  int tokens;
+};
+
+__global__ __launch_bounds__(256) void router_append_kernel(RouterUpdate U) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= static_cast<int64_t>(U.tokens) * U.H) return;
+  const int token = static_cast<int>(index / U.H);
+  const int head = static_cast<int>(index - static_cast<int64_t>(token) * U.H);
+  int low = 0, high = U.S;  // slot with offsets[slot] <= token < offsets[slot + 1]
+  while (low + 1 < high) {
+    const int mid = (low + high) >> 1;
+    if (U.chunk_offsets[mid] <= token) low = mid; else high = mid;
+  }
+  // empty slots share their offset with a neighbour: take the last one that starts here
+  while (low + 1 < U.S && U.chunk_offsets[low + 1] <= token) ++low;
+  const int slot = low;
+  const int position = U.history_lengths[slot] + (token - U.chunk_offsets[slot]);
+  const int64_t run = (static_cast<int64_t>(slot) * U.H + head) * U.capacity + position;
+  U.query_history[run] = U.query[index] & U.qk_mask;
+  U.key_history[run] = U.key[index] & U.qk_mask;
+  if (head < U.Hp) {
+    U.payload_history[(static_cast<int64_t>(slot) * U.Hp + head) * U.capacity + position] =
+        U.payload[static_cast<int64_t>(token) * U.Hp + head] & U.payload_mask;
+  }
+}
+
+// One wave owns 64 consecutive new rows of one (slot, head) (lane = row) and walks over
+// the routes exactly like hard_route_kernel; the first row block starts at the slot's old
+// length, so its predecessor row lies in the history.
+__global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
+  const int slot = blockIdx.y / U.H;
+  const int head = blockIdx.y - slot * U.H;
+  const int old_length = U.history_lengths[slot];
+  const int chunk_begin = U.chunk_offsets[slot];
+  const int new_length = old_length + (U.chunk_offsets[slot + 1] - chunk_begin);
+  const int t0 = old_length + static_cast<int>(blockIdx.x) * kWave;
+  if (t0 >= new_length) return;
+  const int lane = threadIdx.x;
+  const int64_t run_base = (static_cast<int64_t>(slot) * U.H + head) * U.capacity;
+  const uint8_t* q = U.query_history + run_base;
+  const uint8_t* k = U.key_history + run_base;
+  const int t = t0 + lane;
+  const bool row_ok = t < new_length;
+  const uint32_t q_symbol = row_ok ? q[t] : 0u;
+  const int W = U.W;
+  uint64_t best = 0;
+  int run = 0;
+  const int a_last = min(t0 + kWave - 1, new_length - 1);
+  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+    const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
+    int halo = 0;
+    if (column >= 1 && column <= t0 - 1) {
+      const int limit = min(W, column);
+      while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+    }
+    const uint32_t key_chunk = column < new_length ? k[column] : 0u;  // key of route a0 + lane
+    const int count = min(kWave, a_last - a0 + 1);
+    for (int j = 0; j < count; ++j) {
+      const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+      const int halo_j = __builtin_amdgcn_readlane(halo, j);
+      const int above = dpp_wave_shr1(halo_j, run);
+      const int a = a0 + j;
+      const bool match = (q_symbol == k_symbol) && (a <= t);
+      run = match ? min(above + 1, W) : 0;
+      best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
+    }
+  }
+  if (!row_ok) return;
+  const int route = (best >> 32) > 0 ? static_cast<int>(best & 0xffffffffu) : 0;
+  const int64_t token = chunk_begin + (t - old_length);
+  const int payload_head = head / (U.H / U.Hp);
+  U.matched_key_end[token * U.H + head] = route > 0 ? route - 1 : -1;
+  U.output[token * U.H + head] = route > 0
+      ? U.payload_history[(static_cast<int64_t>(slot) * U.Hp + payload_head) * U.capacity + route]
+      : uint8_t(0);
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -2197,6 +2299,49 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const
                                       mismatch_scale, gradient_mask, grad_query, grad_key,
                                       grad_value, workspace, s);
   }
+}
+
+int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
+  if (update == nullptr) return fail(1, "router update is NULL");
+  const rosa_router_update& u = *update;
+  if (u.S < 1 || u.H < 1 || u.Hp < 1 || u.H % u.Hp != 0)
+    return fail(1, "router: heads must be a positive multiple of payload heads");
+  if (u.qk_bits < 1 || u.qk_bits > 8 || u.payload_bits < 1 || u.payload_bits > 8)
+    return fail(1, "router: symbol widths must be in [1, 8]");
+  if (u.W < 1) return fail(1, "router: max_suffix_length must be >= 1");
+  if (u.tokens < 0 || u.longest_chunk < 0 || u.capacity < 1)
+    return fail(1, "router: negative size");
+  if (u.tokens == 0) return 0;
+  if (!u.chunk_offsets || !u.history_lengths || !u.query_history || !u.key_history ||
+      !u.payload_history || !u.query || !u.key || !u.payload || !u.output || !u.matched_key_end)
+    return fail(2, "router: NULL pointer");
+  if (static_cast<int64_t>(u.S) * u.H > 65535)
+    return fail(1, "router: slots * heads must not exceed 65535");
+  RouterUpdate U;
+  U.S = u.S; U.H = u.H; U.Hp = u.Hp; U.W = u.W;
+  U.capacity = u.capacity;
+  U.qk_mask = (1 << u.qk_bits) - 1;
+  U.payload_mask = (1 << u.payload_bits) - 1;
+  U.chunk_offsets = u.chunk_offsets;
+  U.history_lengths = u.history_lengths;
+  U.query_history = u.query_history;
+  U.key_history = u.key_history;
+  U.payload_history = u.payload_history;
+  U.query = u.query; U.key = u.key; U.payload = u.payload;
+  U.output = u.output;
+  U.matched_key_end = u.matched_key_end;
+  U.tokens = u.tokens;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t symbols = static_cast<int64_t>(u.tokens) * u.H;
+  hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
+  const unsigned row_blocks = static_cast<unsigned>((u.longest_chunk + kWave - 1) / kWave);
+  if (row_blocks > 0) {
+    hipLaunchKernelGGL(router_route_kernel, dim3(row_blocks, static_cast<unsigned>(u.S * u.H)),
+                       dim3(kWave), 0, s, U);
+  }
+  const hipError_t status = hipGetLastError();
+  if (status != hipSuccess) return fail_hip(status, "router launch");
+  return 0;
 }
 
 int rosa_hip_stage_timing(int enable) {

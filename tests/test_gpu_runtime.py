@@ -1,0 +1,208 @@
+"""Device-resident ``RosaRuntime`` against the CPU oracle (needs a real MI355X).
+
+Mirrors the reference's ``tests/test_runtime.py:96-420``: same shapes, seeds and properties,
+with the brute-force definition (``oracle/router_oracle.py``) as the expected side.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import router_oracle
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def rosa():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import rosa_soft_amd
+
+    assert rosa_soft_amd.BUILD_CAPABILITIES.rosa_runtime
+    return rosa_soft_amd
+
+
+def random_packed(shape, bits, seed):
+    return torch.randint(0, 1 << bits, shape, dtype=torch.uint8,
+                         generator=torch.Generator().manual_seed(seed))
+
+
+def expect_dense(query, key, payload, qk_bits, payload_bits, horizon):
+    output, ends = router_oracle.route_dense(query.numpy(), key.numpy(), payload.numpy(), qk_bits,
+                                             payload_bits, horizon)
+    return torch.from_numpy(output), torch.from_numpy(ends)
+
+
+@pytest.mark.parametrize("horizon", [1, 2, 5, 64])
+def test_packed_dense_matches_oracle(rosa, horizon):
+    batch, tokens, heads, payload_heads, bits = 2, 19, 4, 2, 4
+    query = random_packed((batch, tokens, heads), bits, 1)
+    key = random_packed((batch, tokens, heads), bits, 2)
+    payload = random_packed((batch, tokens, payload_heads), bits, 3)
+    want = expect_dense(query, key, payload, bits, bits, horizon)
+    with rosa.RosaRuntime(heads, payload_heads, bits, bits, horizon) as runtime:
+        got = runtime.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
+        stats = runtime.stats
+    assert got[0].dtype == torch.uint8 and got[1].dtype == torch.int64
+    assert got[0].device.type == "cuda"
+    assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[1].cpu(), want[1])
+    assert stats[2] == batch * payload_heads * tokens
+
+
+@pytest.mark.parametrize("horizon", [1, 2, 4])
+def test_binary_length_four_state_space(rosa, horizon):
+    patterns = torch.tensor([[(code >> shift) & 1 for shift in range(4)] for code in range(16)],
+                            dtype=torch.uint8).unsqueeze(-1)
+    query = patterns.repeat_interleave(16, dim=0)
+    key = patterns.repeat(16, 1, 1)
+    payload = torch.arange(4, dtype=torch.uint8).view(1, 4, 1).expand(256, -1, -1).contiguous()
+    want = expect_dense(query, key, payload, 1, 2, horizon)
+    with rosa.RosaRuntime(1, 1, 1, 2, horizon) as runtime:
+        got = runtime.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
+    assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[1].cpu(), want[1])
+
+
+def test_finite_horizon_changes_route_and_host_inputs_come_back_on_the_host(rosa):
+    query = torch.zeros(1, 6, 1, dtype=torch.uint8)
+    key = torch.tensor([[[0], [0], [0], [1], [0], [0]]], dtype=torch.uint8)
+    payload = torch.tensor([[[1], [2], [3], [4], [5], [6]]], dtype=torch.uint8)
+    answers = {1: ([0, 2, 3, 4, 4, 6], [-1, 0, 1, 2, 2, 4]), 4: ([0, 2, 3, 4, 4, 4], [-1, 0, 1, 2, 2, 2])}
+    for horizon, (want_output, want_ends) in answers.items():
+        with rosa.RosaRuntime(1, 1, 1, 3, horizon) as runtime:
+            output, ends = runtime.update_packed(query, key, payload)
+        assert output.device.type == "cpu" and ends.device.type == "cpu"
+        assert output.reshape(-1).tolist() == want_output
+        assert ends.reshape(-1).tolist() == want_ends
+
+
+def test_varlen_and_grouped_payload_heads(rosa):
+    lengths = [4, 9, 0, 6]
+    offsets = torch.tensor([0, 4, 13, 13, 19], dtype=torch.int32)
+    heads, payload_heads, bits, horizon = 6, 3, 3, 4
+    total = sum(lengths)
+    query = random_packed((total, heads), bits, 4)
+    key = random_packed((total, heads), bits, 5)
+    payload = random_packed((total, payload_heads), bits, 6)
+    router = router_oracle.StreamingRouter(heads, payload_heads, bits, bits, horizon)
+    want = router.update_packed(query.numpy(), key.numpy(), payload.numpy(), offsets.tolist())
+    with rosa.RosaRuntime(heads, payload_heads, bits, bits, horizon) as runtime:
+        got = runtime.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE),
+                                    cu_seqlens=offsets)
+    assert torch.equal(got[0].cpu(), torch.from_numpy(want[0]))
+    assert torch.equal(got[1].cpu(), torch.from_numpy(want[1]))
+
+
+def test_chunked_updates_equal_one_shot_and_histories_grow(rosa):
+    # 700 tokens per slot: several 64-row blocks per chunk, unaligned chunk starts, and the
+    # history outgrows its first allocation twice
+    batch, tokens, heads, payload_heads, bits, horizon = 2, 700, 3, 1, 2, 9
+    query = random_packed((batch, tokens, heads), bits, 7)
+    key = random_packed((batch, tokens, heads), bits, 8)
+    payload = random_packed((batch, tokens, payload_heads), 5, 9)
+    want = expect_dense(query, key, payload, bits, 5, horizon)
+    with rosa.RosaRuntime(heads, payload_heads, bits, 5, horizon) as one_shot:
+        whole = one_shot.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
+    assert torch.equal(whole[0].cpu(), want[0]) and torch.equal(whole[1].cpu(), want[1])
+    chunks = [0, 3, 11, 200, 201, 457, 640, tokens]
+    outputs, positions = [], []
+    with rosa.RosaRuntime(heads, payload_heads, bits, 5, horizon) as chunked:
+        for begin, end in zip(chunks[:-1], chunks[1:]):
+            output, ends = chunked.update_packed(
+                query[:, begin:end].to(DEVICE), key[:, begin:end].to(DEVICE),
+                payload[:, begin:end].to(DEVICE),
+            )
+            outputs.append(output)
+            positions.append(ends)
+        assert chunked.memory_stats()["payload_symbols"] == batch * payload_heads * tokens
+    assert torch.equal(torch.cat(outputs, dim=1).cpu(), want[0])
+    assert torch.equal(torch.cat(positions, dim=1).cpu(), want[1])
+
+
+def test_single_token_decode_steps(rosa):
+    heads, bits, horizon, tokens = 2, 1, 6, 90
+    query = random_packed((1, tokens, heads), bits, 17)
+    key = random_packed((1, tokens, heads), bits, 18)
+    payload = random_packed((1, tokens, heads), 8, 19)
+    want = expect_dense(query, key, payload, bits, 8, horizon)
+    ends = []
+    with rosa.RosaRuntime(heads, heads, bits, 8, horizon) as runtime:
+        for t in range(tokens):
+            step = runtime.update_packed(query[:, t:t + 1].to(DEVICE), key[:, t:t + 1].to(DEVICE),
+                                         payload[:, t:t + 1].to(DEVICE))
+            ends.append(step[1])
+    assert torch.equal(torch.cat(ends, dim=1).cpu(), want[1])
+
+
+def test_unpacked_null_route_is_exact_zero_and_logit_interface(rosa):
+    # reference tests/test_runtime.py:318-345
+    query = torch.ones(1, 5, 1, 2, device=DEVICE)
+    key = -torch.ones_like(query)
+    payload = torch.ones(1, 5, 1, 3, device=DEVICE)
+    with rosa.RosaRuntime(1, 1, 2, 3, 3) as runtime:
+        output, ends = runtime.update(query, key, payload)
+    assert output.shape == (1, 5, 1, 3) and output.dtype == torch.float32
+    assert torch.count_nonzero(output) == 0 and torch.all(ends == -1)
+    with rosa.RosaRuntime(1, 1, 2, 3, 3) as runtime:
+        output, ends = runtime.update(query, query, payload)
+    assert torch.equal(output[0, 1:], torch.ones(4, 1, 3, device=DEVICE))
+    assert ends.reshape(-1).tolist() == [-1, 0, 1, 2, 3]
+
+
+def test_lifecycle_slot_and_sequence_id_checks(rosa):
+    symbols = torch.zeros(2, 3, 1, dtype=torch.uint8, device=DEVICE)
+    runtime = rosa.RosaRuntime(1, 1, 1, 1, 2)
+    assert runtime.state == "OPEN"
+    runtime.update_packed(symbols, symbols, symbols, sequence_ids=[7, 9])
+    with pytest.raises(RuntimeError, match="sequence_ids changed"):  # checked before the slots
+        runtime.update_packed(symbols[:1], symbols[:1], symbols[:1], sequence_ids=[7])
+    with pytest.raises(RuntimeError, match="sequence_ids are required"):
+        runtime.update_packed(symbols, symbols, symbols)
+    with pytest.raises(RuntimeError, match="sequence_ids changed"):
+        runtime.update_packed(symbols, symbols, symbols, sequence_ids=[9, 7])
+    with pytest.raises(ValueError, match="must be unique"):
+        runtime.update_packed(symbols, symbols, symbols, sequence_ids=[7, 7])
+    runtime.reset()
+    assert runtime.stats == (0, 0, 0)
+    runtime.update_packed(symbols[:1], symbols[:1], symbols[:1])
+    with pytest.raises(RuntimeError, match="slot count is fixed"):
+        runtime.update_packed(symbols, symbols, symbols)
+    with pytest.raises(RuntimeError, match="first update"):
+        runtime.update_packed(symbols[:1], symbols[:1], symbols[:1], sequence_ids=[1])
+    with pytest.raises(TypeError, match="torch.uint8"):
+        runtime.update_packed(symbols.int(), symbols.int(), symbols.int())
+    with pytest.raises(ValueError, match="head count must equal num_heads"):
+        wide = torch.zeros(1, 3, 2, dtype=torch.uint8, device=DEVICE)
+        runtime.update_packed(wide, wide, wide)
+    runtime.close()
+    assert runtime.state == "CLOSED"
+    with pytest.raises(RuntimeError, match="closed"):
+        runtime.update_packed(symbols[:1], symbols[:1], symbols[:1])
+    runtime.close()  # idempotent
+    with pytest.raises(ValueError, match=r"qk_bits must be in \[1, 8\]"):
+        rosa.RosaRuntime(1, 1, 9, 1, 1)
+    with pytest.raises(RuntimeError, match="divisible"):
+        rosa.RosaRuntime(3, 2, 1, 1, 1)
+
+
+def test_state_dict_round_trip_and_async_handle(rosa):
+    heads, bits, horizon = 2, 3, 5
+    query = random_packed((1, 60, heads), bits, 31)
+    key = random_packed((1, 60, heads), bits, 32)
+    payload = random_packed((1, 60, 1), bits, 33)
+    want = expect_dense(query, key, payload, bits, bits, horizon)
+    first = rosa.RosaRuntime(heads, 1, bits, bits, horizon)
+    first.update_packed(query[:, :25].to(DEVICE), key[:, :25].to(DEVICE), payload[:, :25].to(DEVICE))
+    saved = first.state_dict()
+    first.close()
+    second = rosa.RosaRuntime(heads, 1, bits, bits, horizon)
+    second.load_state_dict(saved)
+    side = torch.cuda.Stream(device=DEVICE)
+    work = second.update_packed(query[:, 25:].to(DEVICE), key[:, 25:].to(DEVICE),
+                                payload[:, 25:].to(DEVICE), stream=side, async_op=True)
+    output, ends = work.wait()
+    torch.cuda.synchronize()
+    assert torch.equal(ends.cpu(), want[1][:, 25:]) and torch.equal(output.cpu(), want[0][:, 25:])
+    second.close()
