@@ -194,12 +194,116 @@ def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
     )
 
 
+RUNTIME_WORKLOADS = {
+    # the metric shape served by the device-resident hard router: one prefill update
+    "runtime_prefill": dict(S=2, T=4096, H=64, Hp=16, qk_bits=8, payload_bits=8, W=128),
+    # 8 slots with 4096 tokens of history each, then single-token updates
+    "runtime_decode": dict(S=8, T=4096, H=64, Hp=16, qk_bits=8, payload_bits=8, W=128, decode=64),
+}
+
+
+def runtime_symbols(config, tokens, seed):
+    generator = torch.Generator().manual_seed(seed)
+    draw = lambda heads, bits: torch.randint(
+        0, 1 << bits, (config["S"], tokens, heads), dtype=torch.uint8, generator=generator)
+    return (draw(config["H"], config["qk_bits"]), draw(config["H"], config["qk_bits"]),
+            draw(config["Hp"], config["payload_bits"]))
+
+
+def runtime_cpu_baseline(config, query, key, payload) -> dict:
+    """The reference's own CPU runtime (built from its source under oracle/_ref) on the same
+    prefill, repeated until about ten seconds have passed."""
+
+    from oracle import router_oracle
+
+    native = router_oracle.reference_runtime()
+    if native is None:
+        return dict(value=None, unit="tokens/s", cores=0, kind="reference",
+                    sample="oracle/_ref is not built")
+    slots, tokens, heads = query.shape
+    offsets = torch.arange(0, (slots + 1) * tokens, tokens, dtype=torch.int64)
+    flat = lambda x: x.reshape(slots * tokens, x.size(2)).contiguous()
+    repeats, elapsed = 0, 0.0
+    while elapsed < 10.0 and repeats < 200:
+        runtime = native(heads, payload.size(2), config["qk_bits"], config["payload_bits"],
+                         config["W"])
+        begin = time.perf_counter()
+        runtime.update_packed(offsets, flat(query), flat(key), flat(payload))
+        elapsed += time.perf_counter() - begin
+        repeats += 1
+    return dict(
+        value=repeats * slots * tokens / elapsed, unit="tokens/s",
+        cores=torch.get_num_threads(), kind="reference",
+        sample=(f"rosa_runtime.cpp update_packed, {slots} slots x {tokens} tokens x {heads} heads, "
+                f"{repeats} repeats in {elapsed:.2f} s (OpenMP over slots x heads)"),
+    )
+
+
+def run_runtime_workload(args) -> None:
+    """Streaming hard router: prefill or decode throughput of the device-resident runtime."""
+
+    import rosa_soft_amd
+
+    config = RUNTIME_WORKLOADS[args.workload]
+    device = torch.device("cuda:0")
+    query, key, payload = (t.to(device) for t in runtime_symbols(config, config["T"], 7))
+    decode = config.get("decode", 0)
+    make = lambda: rosa_soft_amd.RosaRuntime(config["H"], config["Hp"], config["qk_bits"],
+                                             config["payload_bits"], config["W"])
+    begin_event = torch.cuda.Event(enable_timing=True)
+    end_event = torch.cuda.Event(enable_timing=True)
+    timed_ms = 0.0
+    if decode:
+        step_q, step_k, step_p = (t.to(device) for t in runtime_symbols(config, decode, 8))
+        for step in range(args.warmup + args.steps):
+            runtime = make()
+            runtime.update_packed(query, key, payload)
+            torch.cuda.synchronize()
+            begin_event.record()
+            for t in range(decode):
+                runtime.update_packed(step_q[:, t:t + 1], step_k[:, t:t + 1], step_p[:, t:t + 1])
+            end_event.record()
+            torch.cuda.synchronize()
+            if step >= args.warmup:
+                timed_ms += begin_event.elapsed_time(end_event)
+            runtime.close()
+        tokens = config["S"] * decode
+    else:
+        for step in range(args.warmup + args.steps):
+            runtime = make()
+            torch.cuda.synchronize()
+            begin_event.record()
+            runtime.update_packed(query, key, payload)
+            end_event.record()
+            torch.cuda.synchronize()
+            if step >= args.warmup:
+                timed_ms += begin_event.elapsed_time(end_event)
+            runtime.close()
+        tokens = config["S"] * config["T"]
+    ms_per_step = timed_ms / args.steps
+    pairs = config["S"] * config["H"] * (
+        decode * config["T"] if decode else config["T"] * (config["T"] - 1) // 2)
+    record = {
+        "metric": "router tokens/sec", "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: " + ", ".join(f"{k}={v}" for k, v in config.items()),
+                   "tokens_per_step": tokens, "pairs_per_step": pairs},
+        "gpairs_per_s": pairs / (ms_per_step * 1e-3) / 1e9,
+    }
+    if not args.no_cpu_baseline and not decode:
+        record["cpu_baseline"] = runtime_cpu_baseline(config, query.cpu(), key.cpu(), payload.cpu())
+    print(json.dumps(record))
+
+
 def main() -> None:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=10)
     parser.add_argument("--warmup", type=int, default=3)
-    parser.add_argument("--workload", default="metric", choices=sorted(WORKLOADS))
+    parser.add_argument("--workload", default="metric",
+                        choices=sorted(WORKLOADS) + sorted(RUNTIME_WORKLOADS))
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument(
         "--copy-calibration", type=int, default=0, metavar="MIB",
@@ -223,6 +327,10 @@ def main() -> None:
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": source.numel() * 4, "copy_bytes_written": source.numel() * 4,
                           "launches": 3}))
+        return
+
+    if args.workload in RUNTIME_WORKLOADS:
+        run_runtime_workload(args)
         return
 
     import rosa_soft_amd

@@ -120,10 +120,12 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
  * update appends the chunk and routes its rows against all earlier keys with the kernel
  * of the hard forward.  Outputs follow the reference: `matched_key_end` int64 [tokens][H],
  * the global key end position in the slot's history or -1; `output` uint8 [tokens][H], the
- * payload symbol after the matched key, 0 for the null route.  `chunk_offsets` [S+1] and
- * `history_lengths` [S] are device int32; the caller checks that
- * history_lengths[s] + chunk length <= capacity and advances the lengths afterwards.
- * `longest_chunk` is the largest number of new tokens of any slot.
+ * payload symbol after the matched key, 0 for the null route.  `chunk_offsets` [S+1]
+ * (device int32) may be NULL when every slot brings `uniform_chunk` tokens.
+ * `history_lengths` [S] (device int32) is read and then advanced by the chunk lengths, so
+ * consecutive updates need no host traffic; the caller keeps
+ * history length + chunk length <= capacity.  `longest_chunk` is the largest number of new
+ * tokens of any slot (small chunks are routed by a per-row kernel).
  */
 typedef struct rosa_router_update {
   int32_t S, H, Hp, W;
@@ -131,8 +133,9 @@ typedef struct rosa_router_update {
   int32_t capacity;
   int32_t tokens;
   int32_t longest_chunk;
+  int32_t uniform_chunk;
   const int32_t* chunk_offsets;
-  const int32_t* history_lengths;
+  int32_t* history_lengths;
   uint8_t* query_history;
   uint8_t* key_history;
   uint8_t* payload_history;

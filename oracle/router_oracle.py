@@ -13,7 +13,9 @@ length is the null route.  The answer is ``e`` (``-1`` for null) and the payload
 ``tests/test_runtime.py:19-77``; this file is that definition restated with numpy, plus a
 streaming wrapper that feeds chunks to it the way ``update_packed`` is called.
 
-Pinned by ``tests/test_router_oracle.py``: the hand-derived answers of the reference's
+Pinned by ``tests/test_router_oracle.py``: the reference's own runtime built from its source
+(``oracle/_ref/librosa_runtime_ref.so``, see ``reference_runtime``) on seeded batches, chunked
+and packed; the hand-derived answers of the reference's
 finite-horizon example (``tests/test_runtime.py:166-217``), exhaustive agreement with an
 independent formulation (run lengths by dynamic programming along diagonals) on all binary
 strings of length four, and the relation to the training hard forward.
@@ -104,3 +106,22 @@ def route_dense(query: np.ndarray, key: np.ndarray, payload: np.ndarray, qk_bits
         payload.reshape(batch * tokens, -1), offsets,
     )
     return output.reshape(batch, tokens, heads), ends.reshape(batch, tokens, heads)
+
+
+def reference_runtime():
+    """``torch.classes.rosa_soft.RosaRuntime`` of the reference, if ``make -C oracle ref`` built it.
+
+    The class is compiled from ``/root/reference/rosa_soft/csrc/rosa_runtime.cpp`` where it
+    lies; returns ``None`` when the library is absent.
+    """
+
+    import os
+
+    import torch
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_ref",
+                        "librosa_runtime_ref.so")
+    if not os.path.exists(path):
+        return None
+    torch.ops.load_library(path)
+    return torch.classes.rosa_soft.RosaRuntime

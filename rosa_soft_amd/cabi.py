@@ -70,6 +70,7 @@ class RosaRouterUpdate(ctypes.Structure):
         ("capacity", ctypes.c_int32),
         ("tokens", ctypes.c_int32),
         ("longest_chunk", ctypes.c_int32),
+        ("uniform_chunk", ctypes.c_int32),
         ("chunk_offsets", ctypes.c_void_p),
         ("history_lengths", ctypes.c_void_p),
         ("query_history", ctypes.c_void_p),

@@ -2100,12 +2100,15 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
 // answer per row is the end position of the matched key (route - 1, or -1 for the
 // null route) and the payload symbol that follows it.
 
+constexpr int kRouterDecodeRows = 8;  // chunks up to this many rows use the per-row kernel
+
 struct RouterUpdate {
   int S, H, Hp, W;
   int capacity;
   int qk_mask, payload_mask;
-  const int32_t* chunk_offsets;  // [S + 1] token offsets of the chunk, per slot
-  const int32_t* history_lengths;  // [S] tokens a slot held before this chunk
+  const int32_t* chunk_offsets;  // [S + 1] token offsets of the chunk per slot, or NULL:
+  int uniform_chunk;             //   then every slot brings this many tokens
+  int32_t* history_lengths;      // [S] tokens a slot held before this chunk (advanced at the end)
   uint8_t* query_history;        // [S][H][capacity]
   uint8_t* key_history;          // [S][H][capacity]
   uint8_t* payload_history;      // [S][Hp][capacity]
@@ -2117,20 +2120,27 @@ struct RouterUpdate {
   int tokens;
 };
 
+__device__ __forceinline__ int router_chunk_begin(const RouterUpdate& U, int slot) {
+  return U.chunk_offsets != nullptr ? U.chunk_offsets[slot] : slot * U.uniform_chunk;
+}
+
 __global__ __launch_bounds__(256) void router_append_kernel(RouterUpdate U) {
   const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (index >= static_cast<int64_t>(U.tokens) * U.H) return;
   const int token = static_cast<int>(index / U.H);
   const int head = static_cast<int>(index - static_cast<int64_t>(token) * U.H);
-  int low = 0, high = U.S;  // slot with offsets[slot] <= token < offsets[slot + 1]
-  while (low + 1 < high) {
-    const int mid = (low + high) >> 1;
-    if (U.chunk_offsets[mid] <= token) low = mid; else high = mid;
+  int slot;
+  if (U.chunk_offsets == nullptr) {
+    slot = token / U.uniform_chunk;
+  } else {
+    int low = 0, high = U.S;  // last slot with offsets[slot] <= token (empty slots share offsets)
+    while (low + 1 < high) {
+      const int mid = (low + high) >> 1;
+      if (U.chunk_offsets[mid] <= token) low = mid; else high = mid;
+    }
+    slot = low;
   }
-  // empty slots share their offset with a neighbour: take the last one that starts here
-  while (low + 1 < U.S && U.chunk_offsets[low + 1] <= token) ++low;
-  const int slot = low;
-  const int position = U.history_lengths[slot] + (token - U.chunk_offsets[slot]);
+  const int position = U.history_lengths[slot] + (token - router_chunk_begin(U, slot));
   const int64_t run = (static_cast<int64_t>(slot) * U.H + head) * U.capacity + position;
   U.query_history[run] = U.query[index] & U.qk_mask;
   U.key_history[run] = U.key[index] & U.qk_mask;
@@ -2147,8 +2157,8 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
   const int slot = blockIdx.y / U.H;
   const int head = blockIdx.y - slot * U.H;
   const int old_length = U.history_lengths[slot];
-  const int chunk_begin = U.chunk_offsets[slot];
-  const int new_length = old_length + (U.chunk_offsets[slot + 1] - chunk_begin);
+  const int chunk_begin = router_chunk_begin(U, slot);
+  const int new_length = old_length + (router_chunk_begin(U, slot + 1) - chunk_begin);
   const int t0 = old_length + static_cast<int>(blockIdx.x) * kWave;
   if (t0 >= new_length) return;
   const int lane = threadIdx.x;
@@ -2189,6 +2199,52 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
   U.output[token * U.H + head] = route > 0
       ? U.payload_history[(static_cast<int64_t>(slot) * U.Hp + payload_head) * U.capacity + route]
       : uint8_t(0);
+}
+
+
+// Few new rows per slot (decoding): one wave per (slot, head, new row); the lanes share the
+// routes of the row, each comparing its suffixes directly, and the wave keeps the maximum of
+// the packed key (length, route): longest first, latest on ties.
+__global__ __launch_bounds__(kWave) void router_decode_kernel(RouterUpdate U) {
+  const int slot = blockIdx.y / U.H;
+  const int head = blockIdx.y - slot * U.H;
+  const int old_length = U.history_lengths[slot];
+  const int chunk_begin = router_chunk_begin(U, slot);
+  const int rows = router_chunk_begin(U, slot + 1) - chunk_begin;
+  const int row = blockIdx.x;
+  if (row >= rows) return;
+  const int lane = threadIdx.x;
+  const int t = old_length + row;
+  const int64_t run_base = (static_cast<int64_t>(slot) * U.H + head) * U.capacity;
+  const uint8_t* q = U.query_history + run_base;
+  const uint8_t* k = U.key_history + run_base;
+  unsigned long long best = 0ull;
+  for (int a = 1 + lane; a <= t; a += kWave) {
+    const int limit = min(U.W, a);
+    int length = 0;
+    while (length < limit && q[t - length] == k[a - 1 - length]) ++length;
+    const unsigned long long packed =
+        (static_cast<unsigned long long>(length) << 32) | static_cast<uint32_t>(a);
+    best = max(best, packed);
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    best = max(best, static_cast<unsigned long long>(__shfl_xor(best, offset, kWave)));
+  }
+  if (lane != 0) return;
+  const int route = (best >> 32) > 0 ? static_cast<int>(best & 0xffffffffull) : 0;
+  const int64_t token = chunk_begin + row;
+  const int payload_head = head / (U.H / U.Hp);
+  U.matched_key_end[token * U.H + head] = route > 0 ? route - 1 : -1;
+  U.output[token * U.H + head] = route > 0
+      ? U.payload_history[(static_cast<int64_t>(slot) * U.Hp + payload_head) * U.capacity + route]
+      : uint8_t(0);
+}
+
+__global__ __launch_bounds__(256) void router_advance_kernel(RouterUpdate U) {
+  const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= U.S) return;
+  U.history_lengths[slot] += router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot);
 }
 
 }  // namespace
@@ -2312,7 +2368,9 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   if (u.tokens < 0 || u.longest_chunk < 0 || u.capacity < 1)
     return fail(1, "router: negative size");
   if (u.tokens == 0) return 0;
-  if (!u.chunk_offsets || !u.history_lengths || !u.query_history || !u.key_history ||
+  if (!u.chunk_offsets && static_cast<int64_t>(u.uniform_chunk) * u.S != u.tokens)
+    return fail(1, "router: without chunk_offsets every slot brings uniform_chunk tokens");
+  if (!u.history_lengths || !u.query_history || !u.key_history ||
       !u.payload_history || !u.query || !u.key || !u.payload || !u.output || !u.matched_key_end)
     return fail(2, "router: NULL pointer");
   if (static_cast<int64_t>(u.S) * u.H > 65535)
@@ -2323,6 +2381,7 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   U.qk_mask = (1 << u.qk_bits) - 1;
   U.payload_mask = (1 << u.payload_bits) - 1;
   U.chunk_offsets = u.chunk_offsets;
+  U.uniform_chunk = u.uniform_chunk;
   U.history_lengths = u.history_lengths;
   U.query_history = u.query_history;
   U.key_history = u.key_history;
@@ -2334,11 +2393,15 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t symbols = static_cast<int64_t>(u.tokens) * u.H;
   hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
-  const unsigned row_blocks = static_cast<unsigned>((u.longest_chunk + kWave - 1) / kWave);
-  if (row_blocks > 0) {
-    hipLaunchKernelGGL(router_route_kernel, dim3(row_blocks, static_cast<unsigned>(u.S * u.H)),
+  const unsigned runs = static_cast<unsigned>(u.S * u.H);
+  if (u.longest_chunk > 0 && u.longest_chunk <= kRouterDecodeRows) {
+    hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(u.longest_chunk), runs),
                        dim3(kWave), 0, s, U);
+  } else if (u.longest_chunk > 0) {
+    const unsigned row_blocks = static_cast<unsigned>((u.longest_chunk + kWave - 1) / kWave);
+    hipLaunchKernelGGL(router_route_kernel, dim3(row_blocks, runs), dim3(kWave), 0, s, U);
   }
+  hipLaunchKernelGGL(router_advance_kernel, dim3(blocks_for(u.S, 256)), dim3(256), 0, s, U);
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "router launch");
   return 0;

@@ -232,7 +232,8 @@ class RosaRuntime:
         self._slot_count = -1
         self._sequence_ids: Optional[Tuple[int, ...]] = None
         self._slots_initialized = False
-        self._lengths: list = []            # host copy of the per-slot history lengths
+        self._lengths: list = []            # host mirror of the per-slot history lengths
+        self._device_lengths: Optional[Tensor] = None   # [S] int32, advanced by the library
         self._capacity = 0
         self._query_history: Optional[Tensor] = None    # [S, H, capacity] uint8
         self._key_history: Optional[Tensor] = None      # [S, H, capacity] uint8
@@ -448,7 +449,10 @@ class RosaRuntime:
             return output, ends
         chunk_lengths = [after - before for before, after in zip(offsets[:-1], offsets[1:])]
         self._grow(max(old + new for old, new in zip(self._lengths, chunk_lengths)))
-        tables = torch.tensor([offsets, self._lengths + [0]], dtype=torch.int32).to(self._device)
+        if self._device_lengths is None:
+            self._device_lengths = torch.tensor(self._lengths, dtype=torch.int32).to(self._device)
+        uniform = all(length == chunk_lengths[0] for length in chunk_lengths)
+        tables = None if uniform else torch.tensor(offsets, dtype=torch.int32).to(self._device)
         update = cabi.RosaRouterUpdate()
         update.S, update.H, update.Hp = self._slot_count, self._num_heads, self._num_payload_heads
         update.W = min(self._max_suffix_length, 2**31 - 1)
@@ -456,8 +460,9 @@ class RosaRuntime:
         update.capacity = self._capacity
         update.tokens = tokens
         update.longest_chunk = max(chunk_lengths)
-        update.chunk_offsets = tables[0].data_ptr()
-        update.history_lengths = tables[1].data_ptr()
+        update.uniform_chunk = chunk_lengths[0] if uniform else 0
+        update.chunk_offsets = None if uniform else tables.data_ptr()
+        update.history_lengths = self._device_lengths.data_ptr()
         update.query_history = self._query_history.data_ptr()
         update.key_history = self._key_history.data_ptr()
         update.payload_history = self._payload_history.data_ptr()
@@ -465,8 +470,8 @@ class RosaRuntime:
             query.data_ptr(), key.data_ptr(), payload.data_ptr()
         update.output, update.matched_key_end = output.data_ptr(), ends.data_ptr()
         cabi.router_update(update, self._device)
-        # the launch is stream-ordered; keep the small tables alive until it has run
-        tables.record_stream(torch.cuda.current_stream(self._device))
+        if tables is not None:  # stream-ordered launch: keep the table alive until it has run
+            tables.record_stream(torch.cuda.current_stream(self._device))
         self._lengths = [old + new for old, new in zip(self._lengths, chunk_lengths)]
         return output, ends
 

@@ -94,3 +94,35 @@ def test_router_equals_the_training_hard_forward(c_oracle):
     unpacked = logits(output, value_bits)
     unpacked[torch.from_numpy(ends < 0)] = 0.0
     assert torch.equal(unpacked, hard)
+
+
+def test_oracle_equals_the_reference_runtime_built_from_source():
+    # oracle/_ref/librosa_runtime_ref.so is the reference's rosa_runtime.cpp compiled as is
+    import pytest
+
+    native = router_oracle.reference_runtime()
+    if native is None:
+        pytest.skip("oracle/_ref is not built (make -C oracle ref)")
+    rng = np.random.default_rng(3)
+    for heads, payload_heads, qk_bits, payload_bits, horizon, lengths in (
+        (4, 2, 4, 4, 5, [19, 19]),
+        (6, 3, 3, 3, 4, [4, 9, 0, 6]),
+        (2, 1, 1, 8, 64, [130]),
+        (1, 1, 8, 1, 1, [40, 1]),
+    ):
+        total = sum(lengths)
+        offsets = [0] + list(np.cumsum(lengths))
+        query = rng.integers(0, 256, (total, heads), dtype=np.uint8)
+        key = rng.integers(0, 256, (total, heads), dtype=np.uint8)
+        payload = rng.integers(0, 256, (total, payload_heads), dtype=np.uint8)
+        mine = router_oracle.StreamingRouter(heads, payload_heads, qk_bits, payload_bits, horizon)
+        theirs = native(heads, payload_heads, qk_bits, payload_bits, horizon)
+        # two updates: the second continues every slot's history
+        for part in range(2):
+            want = theirs.update_packed(torch.tensor(offsets, dtype=torch.int64),
+                                        torch.from_numpy(query), torch.from_numpy(key),
+                                        torch.from_numpy(payload))
+            got = mine.update_packed(query, key, payload, offsets)
+            assert np.array_equal(got[0], want[0].numpy()), (heads, horizon, part)
+            assert np.array_equal(got[1], want[1].numpy()), (heads, horizon, part)
+            query, key, payload = key.copy(), query.copy(), payload[::-1].copy()
