@@ -552,6 +552,8 @@ struct VjpParams {
   const int32_t* header;        // [0] offsets flag, [1] work counter, [3] chunk records fit
   float* checkpoints;           // one record per (band, 16-row chunk), or NULL
   int record_floats;            // kCheckpointFloats (+ kKeepBitFloats with dropout)
+  int value_stride;             // value width of the tensors (L.Dv is the slice being processed)
+  int value_offset;             // first value dimension of the slice
   float* block_scratch;         // per resident block: ring + segment checkpoints
   int64_t block_scratch_floats;
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
@@ -562,7 +564,7 @@ struct VjpParams {
 template <int DTYPE>
 __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
     const void* __restrict__ grad_output, float* __restrict__ grad_rows, int64_t rows, int H,
-    int Dv, int dvp, int T, int N, int varlen) {
+    int Dv, int dvp, int T, int N, int varlen, int value_stride, int value_offset) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (row >= rows) return;  // row = token * H + h (token-major)
   const int64_t token = row / H;
@@ -575,7 +577,8 @@ __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
     dst = (b * H + h) * T + (token - b * T);
   }
   for (int d = 0; d < dvp; ++d) {
-    grad_rows[dst * dvp + d] = d < Dv ? load_as_float<DTYPE>(grad_output, row * Dv + d) : 0.0f;
+    grad_rows[dst * dvp + d] =
+        d < Dv ? load_as_float<DTYPE>(grad_output, row * value_stride + value_offset + d) : 0.0f;
   }
 }
 
@@ -583,7 +586,7 @@ __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
 template <int DTYPE>
 __global__ __launch_bounds__(256) void pack_value_bits_kernel(
     const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
-    int Dv, int nvw, int T, int N, int varlen) {
+    int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (row >= rows) return;  // row = token * Hv + hv
   const int64_t token = row / Hv;
@@ -599,7 +602,9 @@ __global__ __launch_bounds__(256) void pack_value_bits_kernel(
     uint32_t word = 0u;
     for (int bit = 0; bit < 32; ++bit) {
       const int d = w * 32 + bit;
-      if (d < Dv && load_as_float<DTYPE>(value, row * Dv + d) > 0.0f) word |= 1u << bit;
+      if (d < Dv && load_as_float<DTYPE>(value, row * value_stride + value_offset + d) > 0.0f) {
+        word |= 1u << bit;
+      }
     }
     value_bits[dst * nvw + w] = word;
   }
@@ -1296,7 +1301,7 @@ void vjp_gradients_kernel(VjpParams P) {
       const int64_t column0 = static_cast<int64_t>(u.start) + done_first + 1 + 4 * lg;
       const int64_t last_token = static_cast<int64_t>(u.start) + view.len - 1;
       const int64_t symbol_stride = static_cast<int64_t>(P.L.H) * D;
-      const int64_t value_stride = static_cast<int64_t>(P.L.Hv) * Dv;
+      const int64_t value_stride = static_cast<int64_t>(P.L.Hv) * P.value_stride;
       if (want_q) {
 #pragma unroll
         for (int n = 0; n < DT; ++n) {
@@ -1317,7 +1322,8 @@ void vjp_gradients_kernel(VjpParams P) {
         for (int n = 0; n < VT; ++n) {
           const int d = 16 * n + li;
           if (d < Dv) {
-            float* target = P.grad_value + (column0 * P.L.Hv + hv) * Dv + d;
+            float* target =
+                P.grad_value + (column0 * P.L.Hv + hv) * P.value_stride + P.value_offset + d;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               if (full || column0 + e <= last_token) {
@@ -1771,6 +1777,8 @@ ForwardWorkspace carve_forward(const ProblemView& v) {
   return w;
 }
 
+constexpr int kValueSlice = 64;  // value dimensions one backward pass covers
+
 int value_words(int Dv) { return (Dv + 31) / 32; }
 
 int padded_value_width(int Dv) {
@@ -1803,11 +1811,12 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.block_prefix = cursor; cursor += align_up(sizeof(int32_t) * (s + 1));
   w.step_prefix = cursor; cursor += align_up(sizeof(int64_t) * (s + 1));
   const size_t rows = static_cast<size_t>(v.symbol_rows);
-  const int dvp = padded_value_width(v.L.Dv);
+  const int slice_width = std::min(v.L.Dv, kValueSlice);
+  const int dvp = padded_value_width(slice_width);
   w.stats = cursor; cursor += align_up(sizeof(float) * 4 * rows);
   w.grad_rows = cursor; cursor += align_up(sizeof(float) * rows * dvp);
   w.value_bits = cursor;
-  cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(v.L.Dv));
+  cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(slice_width));
   // Chunk records written by the row-statistics pass for the gradient pass, which
   // otherwise rebuilds the evidence with forward sweeps of its own and evaluates the
   // dropout hash a second time.
@@ -1995,10 +2004,12 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   const VjpWorkspace w = carve_vjp(view, dropout_p > 0.0f);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
                            stream, at<int64_t>(workspace, w.step_prefix), w.checkpoint_capacity);
-  const int dvp = padded_value_width(L.Dv);
-  const int nvw = value_words(L.Dv);
+  // Value widths above 64 are processed in slices of 64 dimensions, one full backward per
+  // slice: the route weights do not depend on the values, dV of a slice needs only that
+  // slice, and dQ / dK are linear in the utilities, i.e. they are the sum over the slices.
+  const int full_width = L.Dv;
   const int64_t symbol_elements = view.symbol_rows * L.D;
-  const int64_t value_elements = view.value_rows * L.Dv;
+  const int64_t value_elements = view.value_rows * full_width;
   stage_begin(kStagePrepare, stream);
   {
     const int64_t largest = std::max(symbol_elements, value_elements);
@@ -2007,6 +2018,11 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
                        grad_query ? symbol_elements : 0, grad_key, grad_key ? symbol_elements : 0,
                        grad_value, grad_value ? value_elements : 0);
   }
+  for (int value_offset = 0; value_offset < full_width; value_offset += kValueSlice) {
+  L.Dv = std::min(kValueSlice, full_width - value_offset);
+  const int dvp = padded_value_width(L.Dv);
+  const int nvw = value_words(L.Dv);
+  if (value_offset > 0) stage_begin(kStagePrepare, stream);
 
   float4* stats = at<float4>(workspace, w.stats);
   float* grad_rows = at<float>(workspace, w.grad_rows);
@@ -2016,10 +2032,10 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
 
   hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>, dim3(blocks_for(view.symbol_rows, 256)),
                      dim3(256), 0, stream, grad_output, grad_rows, view.symbol_rows,
-                     L.H, L.Dv, dvp, L.T, L.N, L.varlen);
+                     L.H, L.Dv, dvp, L.T, L.N, L.varlen, full_width, value_offset);
   hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
                      dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
-                     L.T, L.N, L.varlen);
+                     L.T, L.N, L.varlen, full_width, value_offset);
   if (L.varlen) {
     hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
                        dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
@@ -2063,6 +2079,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   P.header = at<int32_t>(workspace, w.header);
   P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
   P.record_floats = w.record_floats;
+  P.value_stride = full_width;
+  P.value_offset = value_offset;
   P.block_scratch = at<float>(workspace, w.block_scratch);
   P.block_scratch_floats = w.block_scratch_floats;
   P.ring_rows = w.ring_rows;
@@ -2078,6 +2096,7 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     status = dispatch_vjp<2, 64>(P, w, analytic, dropout, stream);
   }
   if (status != 0) return status;
+  }  // value slices
   const int64_t finalize_items = std::max(symbol_elements, value_elements);
   stage_begin(kStageFinalize, stream);
   hipLaunchKernelGGL(finalize_gradients_kernel<DTYPE>, dim3(blocks_for(finalize_items, 256)),
@@ -2330,8 +2349,6 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const
     return fail(1, "surrogate_vjp: scale, mismatch_scale > 0 and 0 <= dropout_p < 1 required");
   if (dropout_p > 0.0f && dropout_seed == nullptr)
     return fail(2, "surrogate_vjp: dropout_seed must be given exactly when dropout_p > 0");
-  if (problem->Dv > 64)
-    return fail(4, "surrogate_vjp: value dimension above 64 is not supported by this build");
   if (workspace_bytes < carve_vjp(view, dropout_p > 0.0f).total)
     return fail(3, "surrogate_vjp: workspace too small");
   if (!(gradient_mask & ROSA_GRAD_QUERY)) grad_query = nullptr;

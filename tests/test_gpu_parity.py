@@ -143,6 +143,8 @@ VJP_CASES = [
     (1, 1200, 2, 8, 1, 8, 128, 1.0, 0.1, 3.0, torch.float32, "random"),
     (1, 180, 2, 8, 2, 8, 32, 10.0, 0.0, 3.0, torch.float32, "shifted"),   # row-maximum pass
     (1, 120, 1, 4, 1, 4, 8, 30.0, 0.2, 0.5, torch.float32, "periodic"),  # row-maximum pass
+    (1, 90, 2, 4, 1, 70, 12, 1.0, 0.1, 3.0, torch.float32, "random"),    # two value slices
+    (1, 70, 2, 3, 2, 130, 8, 1.0, 0.0, 3.0, torch.bfloat16, "shifted"),  # three value slices
 ]
 
 
