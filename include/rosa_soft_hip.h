@@ -62,6 +62,17 @@ size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_ma
                                     float scale, int dropout);
 
 /*
+ * Upper bound in bytes on the chunk records (evidence checkpoints and dropout keep
+ * decisions) that the backward workspace holds between its two passes; the default is
+ * 4 GiB, (size_t)-1 restores it, 0 forbids the records.  A backward whose records do not
+ * fit recomputes instead (forward sweeps and a second hash evaluation in the gradient
+ * pass): same results, less memory, more time.  Process-wide; call it before sizing the
+ * workspace.  The reference has no counterpart (its backward keeps no state between
+ * kernels); the knob exists for callers that must bound the workspace.
+ */
+void rosa_hip_set_record_budget(size_t bytes);
+
+/*
  * Exact hard forward.  Replaces hard_forward_cuda (rosa_soft_kernels.cu:1766-1834)
  * and hard_forward_varlen_cuda (:1837-1920): sign-packs query and key into
  * head-major int32 words (dense [B,H,T], packed [H,N]), finds the

@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_last_error",
     "rosa_hip_forward_workspace_bytes",
     "rosa_hip_vjp_workspace_bytes",
+    "rosa_hip_set_record_budget",
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_surrogate_vjp",
@@ -110,6 +111,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_vjp_workspace_bytes.argtypes = [
         problem_p, ctypes.c_int, ctypes.c_float, ctypes.c_int,
     ]
+    library.rosa_hip_set_record_budget.restype = None
+    library.rosa_hip_set_record_budget.argtypes = [ctypes.c_size_t]
     library.rosa_hip_hard_forward.restype = ctypes.c_int
     library.rosa_hip_hard_forward.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
@@ -321,6 +324,13 @@ def router_update(update: RosaRouterUpdate, device: torch.device) -> None:
             ctypes.byref(update), torch.cuda.current_stream(device).cuda_stream
         )
     _check(status, "rosa_hip_router_update")
+
+
+def set_record_budget(limit_bytes: Optional[int]) -> None:
+    """Bound the chunk records of the backward workspace (``None`` restores the default)."""
+
+    load().rosa_hip_set_record_budget(ctypes.c_size_t(-1).value if limit_bytes is None
+                                      else int(limit_bytes))
 
 
 def stage_timing(enable: bool) -> None:

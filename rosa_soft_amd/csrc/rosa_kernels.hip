@@ -1779,6 +1779,10 @@ ForwardWorkspace carve_forward(const ProblemView& v) {
 
 constexpr int kValueSlice = 64;  // value dimensions one backward pass covers
 
+// bytes of chunk records the backward workspace may hold (4 GiB unless the caller lowers it)
+constexpr size_t kDefaultRecordBudget = size_t(1) << 32;
+size_t g_record_budget_bytes = kDefaultRecordBudget;
+
 int value_words(int Dv) { return (Dv + 31) / 32; }
 
 int padded_value_width(int Dv) {
@@ -1823,7 +1827,8 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.checkpoints = cursor;
   w.record_floats = kCheckpointFloats + (dropout ? kKeepBitFloats : 0);
   {
-    const int64_t budget = (int64_t(1) << 32) / (sizeof(float) * w.record_floats);  // 4 GiB
+    const int64_t budget =
+        static_cast<int64_t>(g_record_budget_bytes / (sizeof(float) * w.record_floats));
     const int64_t steps = v.L.varlen
         ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
         : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
@@ -2422,6 +2427,10 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "router launch");
   return 0;
+}
+
+void rosa_hip_set_record_budget(size_t bytes) {
+  g_record_budget_bytes = bytes == static_cast<size_t>(-1) ? kDefaultRecordBudget : bytes;
 }
 
 int rosa_hip_stage_timing(int enable) {

@@ -382,3 +382,47 @@ def test_selected_routes_of_a_packed_batch(cabi, c_oracle):
         assert torch.equal(output[piece].cpu(), want_out[0])
         assert torch.equal(inspection.selected_route_indices[piece].cpu(), want_routes[0].t())
         assert torch.equal(inspection.selected_suffix_lengths[piece].cpu(), want_lengths[0].t())
+
+
+# --------------------------------------------------------------------------- bounded workspace
+
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,p,pattern,lengths", [
+    (2, 330, 2, 4, 1, 6, 24, 0.2, "random", None),
+    (1, 400, 1, 8, 1, 8, 128, 0.0, "all_match", None),
+    (1, 0, 2, 3, 2, 5, 16, 0.1, "random", [70, 0, 1, 300, 129]),
+])
+def test_backward_without_chunk_records_recomputes_to_the_same_gradients(
+        cabi, c_oracle, B, T, H, D, Hv, Dv, W, p, pattern, lengths):
+    # with the records forbidden the gradient pass sweeps forward again and hashes again
+    seed = 99 if p > 0 else None
+    if lengths is None:
+        query, key, value, grad_output = make_case(B, T, H, D, Hv, Dv, seed=T, pattern=pattern)
+        offsets = None
+    else:
+        total = sum(lengths)
+        query, key, value, grad_output = (t[0] for t in make_case(1, total, H, D, Hv, Dv, seed=5))
+        offsets = [0] + list(np.cumsum(lengths))
+    cabi.set_record_budget(None)
+    _, _, _, _, with_records = run_device(cabi, query, key, value, grad_output, W, 1.0, p, 3.0, seed,
+                                          cu_seqlens=offsets)
+    full = cabi.vjp_workspace_bytes(query.to(DEVICE), value.to(DEVICE), W,
+                                    None if offsets is None else
+                                    torch.tensor(offsets, dtype=torch.int32, device=DEVICE))
+    cabi.set_record_budget(0)
+    try:
+        small = cabi.vjp_workspace_bytes(query.to(DEVICE), value.to(DEVICE), W,
+                                         None if offsets is None else
+                                         torch.tensor(offsets, dtype=torch.int32, device=DEVICE))
+        _, _, _, _, without = run_device(cabi, query, key, value, grad_output, W, 1.0, p, 3.0, seed,
+                                         cu_seqlens=offsets)
+    finally:
+        cabi.set_record_budget(None)
+    assert small < full
+    if lengths is None:
+        want = c_oracle.surrogate_vjp(query, key, value, grad_output, max_suffix_length=W,
+                                      dropout_p=p, seed=seed)
+        for name, got, expected in zip(("grad_query", "grad_key", "grad_value"), without, want):
+            assert_gradients_close(got, expected, name)
+    # both ways of getting the state give the same gradients up to summation order
+    for got, expected in zip(without, with_records):
+        assert_gradients_close(got, expected.cpu())
