@@ -166,43 +166,65 @@ __device__ __forceinline__ void store_sign(void* base, int64_t index, int sign) 
   }
 }
 
-// One round of the counter hash.  (The two 32-bit multiplies run at quarter rate; building
-// them from 16-bit dot products, v_dot2_u32_u16, was measured slower on gfx950.)
-__device__ __forceinline__ uint32_t mix32(uint32_t s) {
-  s ^= s >> 16;
-  s *= 0x7feb352du;
+// The counter hash (reference rosa_soft_kernels.cu:549-586) is six rounds of
+//   h(x): x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16
+// chained as s = h(s ^ key).  fold16(x) = x ^ (x >> 16) is linear over xor and its own
+// inverse, so the closing fold of one round, the key and the opening fold of the next
+// round collapse into one xor:  fold16(fold16(x) ^ key) = x ^ fold16(key).  The rounds
+// below therefore carry the state *before* its closing fold and take keys that are
+// already folded; only the last round is closed.  Same bits, two instructions fewer per
+// round.  (The two 32-bit multiplies are slow instructions; building them from 16-bit
+// dot products, v_dot2_u32_u16, was measured slower on gfx950.)
+__device__ __forceinline__ uint32_t fold16(uint32_t x) { return x ^ (x >> 16); }
+
+__device__ __forceinline__ uint32_t open_round(uint32_t folded_input) {
+  uint32_t s = folded_input * 0x7feb352du;
   s ^= s >> 15;
-  s *= 0x846ca68bu;
-  s ^= s >> 16;
-  return s;
+  return s * 0x846ca68bu;
 }
 
-// Dropout multiplier of one (row, route); head/batch/seed salts are folded by
-// the caller into wave-uniform constants.
+// Wave-uniform part of the dropout decision of one (row, route): the folded keys of
+// rounds two to six and the integer form of the keep test.
 struct DropoutKey {
-  uint32_t row_salt;    // row ^ 0xb5297a4d
-  uint32_t head_salt;   // head ^ 0x63d83595
-  uint32_t batch_salt;  // batch ^ 0xa511e9b3
-  uint32_t seed_low;
-  uint32_t seed_high_salt;  // seed_high ^ 0x9e3779b9
+  uint32_t row_key;    // fold16(row ^ 0xb5297a4d)
+  uint32_t head_key;   // fold16(head ^ 0x63d83595)
+  uint32_t batch_key;  // fold16(batch ^ 0xa511e9b3)
+  uint32_t seed_low_key;
+  uint32_t seed_high_key;  // fold16(seed_high ^ 0x9e3779b9)
+  uint32_t keep_from;      // keep iff the hash is at least this
 };
 
-// first hash round: depends on the route only, so a band computes it once per
-// column (for the column entering at lane 0) and slides it with the columns
-__device__ __forceinline__ uint32_t route_hash_of(int route) {
-  return mix32(static_cast<uint32_t>(route) ^ 0x68e31da4u);
+// The uniform of a pair is (hash >> 8) * 2^-24 and the pair is kept iff uniform >= p.
+// Both sides are exact in float32, so this is hash >= ceil(p * 2^24) * 256.
+__device__ __forceinline__ DropoutKey make_dropout_key(uint64_t seed, int head, int batch,
+                                                       float dropout_p) {
+  DropoutKey key;
+  key.row_key = 0;
+  key.head_key = fold16(static_cast<uint32_t>(head) ^ 0x63d83595u);
+  key.batch_key = fold16(static_cast<uint32_t>(batch) ^ 0xa511e9b3u);
+  key.seed_low_key = fold16(static_cast<uint32_t>(seed));
+  key.seed_high_key = fold16(static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u);
+  key.keep_from = static_cast<uint32_t>(ceilf(dropout_p * 16777216.0f)) << 8;
+  return key;
 }
 
-__device__ __forceinline__ float dropout_multiplier(const DropoutKey& key, uint32_t route_hash,
-                                                    float dropout_p, float inverse_keep) {
-  uint32_t s = route_hash;
-  s = mix32(s ^ key.row_salt);
-  s = mix32(s ^ key.head_salt);
-  s = mix32(s ^ key.batch_salt);
-  s = mix32(s ^ key.seed_low);
-  s = mix32(s ^ key.seed_high_salt);
-  const float uniform = static_cast<float>(s >> 8) * 0x1.0p-24f;
-  return uniform >= dropout_p ? inverse_keep : 0.0f;
+__device__ __forceinline__ void set_row(DropoutKey& key, int row) {
+  key.row_key = fold16(static_cast<uint32_t>(row) ^ 0xb5297a4du);
+}
+
+// first hash round (open): depends on the route only, so a band computes it once per
+// column (for the column entering at lane 0) and slides it with the columns
+__device__ __forceinline__ uint32_t route_hash_of(int route) {
+  return open_round(fold16(static_cast<uint32_t>(route) ^ 0x68e31da4u));
+}
+
+__device__ __forceinline__ bool dropout_keeps(const DropoutKey& key, uint32_t route_hash) {
+  uint32_t s = open_round(route_hash ^ key.row_key);
+  s = open_round(s ^ key.head_key);
+  s = open_round(s ^ key.batch_key);
+  s = open_round(s ^ key.seed_low_key);
+  s = open_round(s ^ key.seed_high_key);
+  return fold16(s) >= key.keep_from;
 }
 
 // ---------------------------------------------------------------------------
@@ -1003,11 +1025,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   const int W = P.L.W;
   DropoutKey key;
   if constexpr (DROPOUT) {
-    const uint64_t seed = static_cast<uint64_t>(*P.dropout_seed);
-    key.head_salt = static_cast<uint32_t>(u.head) ^ 0x63d83595u;
-    key.batch_salt = static_cast<uint32_t>(u.seq) ^ 0xa511e9b3u;
-    key.seed_low = static_cast<uint32_t>(seed);
-    key.seed_high_salt = static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u;
+    key = make_dropout_key(static_cast<uint64_t>(*P.dropout_seed), u.head, u.seq, P.dropout_p);
   }
   Band<NVW> band;
   band.evidence = 0.0f;
@@ -1071,9 +1089,10 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           float keep = 1.0f;
           if constexpr (DROPOUT) {
             route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-            key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-            keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
-            kept_bits |= keep != 0.0f ? (1u << r) : 0u;
+            set_row(key, t);
+            const bool kept = dropout_keeps(key, route_hash);
+            keep = kept ? P.inverse_keep : 0.0f;
+            kept_bits |= kept ? (1u << r) : 0u;
           }
           weights[r * kWeightPitch + lane] = weight;
           utilities[r * kUtilityPitch + lane] = weight * keep * utility;
@@ -1238,11 +1257,7 @@ void vjp_gradients_kernel(VjpParams P) {
     if (!make_view<NVW, VARLEN>(P, u, view, hv)) continue;
     DropoutKey key;
     if constexpr (DROPOUT) {
-      const uint64_t seed = static_cast<uint64_t>(*P.dropout_seed);
-      key.head_salt = static_cast<uint32_t>(u.head) ^ 0x63d83595u;
-      key.batch_salt = static_cast<uint32_t>(u.seq) ^ 0xa511e9b3u;
-      key.seed_low = static_cast<uint32_t>(seed);
-      key.seed_high_salt = static_cast<uint32_t>(seed >> 32) ^ 0x9e3779b9u;
+      key = make_dropout_key(static_cast<uint64_t>(*P.dropout_seed), u.head, u.seq, P.dropout_p);
     }
 
     // column accumulators of the 80-column window, one MFMA tile per 16 columns
@@ -1487,8 +1502,8 @@ void vjp_gradients_kernel(VjpParams P) {
                 keep = __int_as_float(__float_as_int(P.inverse_keep) & kept);
               } else {
                 route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
-                key.row_salt = static_cast<uint32_t>(t) ^ 0xb5297a4du;
-                keep = dropout_multiplier(key, route_hash, P.dropout_p, P.inverse_keep);
+                set_row(key, t);
+                keep = dropout_keeps(key, route_hash) ? P.inverse_keep : 0.0f;
               }
             }
             const float adjoint =
