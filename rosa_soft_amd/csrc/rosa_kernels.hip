@@ -582,44 +582,69 @@ struct VjpParams {
   int total_units;
 };
 
-// grad_output -> float32 head-major rows padded to DVP
+// grad_output -> float32 head-major rows padded to DVP.  One thread per float of the
+// destination: stores are contiguous, loads are runs of Dv elements.
 template <int DTYPE>
 __global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
     const void* __restrict__ grad_output, float* __restrict__ grad_rows, int64_t rows, int H,
     int Dv, int dvp, int T, int N, int varlen, int value_stride, int value_offset) {
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (row >= rows) return;  // row = token * H + h (token-major)
-  const int64_t token = row / H;
-  const int h = static_cast<int>(row - token * H);
-  int64_t dst;
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= rows * dvp) return;
+  const int64_t dst = index / dvp;  // head-major row
+  const int d = static_cast<int>(index - dst * dvp);
+  int64_t source_row;  // token * H + h
   if (varlen) {
-    dst = static_cast<int64_t>(h) * N + token;
+    const int64_t h = dst / N;
+    source_row = (dst - h * N) * H + h;
   } else {
-    const int64_t b = token / T;
-    dst = (b * H + h) * T + (token - b * T);
+    const int64_t bh = dst / T;
+    const int64_t b = bh / H;
+    source_row = (b * T + (dst - bh * T)) * H + (bh - b * H);
   }
-  for (int d = 0; d < dvp; ++d) {
-    grad_rows[dst * dvp + d] =
-        d < Dv ? load_as_float<DTYPE>(grad_output, row * value_stride + value_offset + d) : 0.0f;
+  grad_rows[index] =
+      d < Dv ? load_as_float<DTYPE>(grad_output, source_row * value_stride + value_offset + d)
+             : 0.0f;
+}
+
+__device__ __forceinline__ int64_t value_word_row(int64_t row, int Hv, int T, int N, int varlen) {
+  const int64_t token = row / Hv;  // row = token * Hv + hv
+  const int64_t hv = row - token * Hv;
+  if (varlen) return hv * N + token;
+  const int64_t b = token / T;
+  return (b * Hv + hv) * T + (token - b * T);
+}
+
+// Value sign bits for widths 8, 16, 32 and 64: one lane per element in the order of the
+// tensor, one wave ballot per 64 elements; the lane at the start of a 32-bit group (or of
+// a narrower row) stores that group's word.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void pack_value_bits_ballot_kernel(
+    const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
+    int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool inside = index < rows * Dv;
+  const int64_t row = index / Dv;
+  const int d = static_cast<int>(index - row * Dv);
+  const bool positive =
+      inside && load_as_float<DTYPE>(value, row * value_stride + value_offset + d) > 0.0f;
+  const uint64_t ballot = __ballot(positive);
+  if (inside && (d & 31) == 0) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t word = static_cast<uint32_t>(ballot >> lane);
+    if (Dv < 32) word &= (1u << Dv) - 1u;
+    value_bits[value_word_row(row, Hv, T, N, varlen) * nvw + (d >> 5)] = word;
   }
 }
 
 // value sign bits, head-major over value heads: word index (seq, hv, t) like the symbol words
+// (any width: one thread per row)
 template <int DTYPE>
 __global__ __launch_bounds__(256) void pack_value_bits_kernel(
     const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
     int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (row >= rows) return;  // row = token * Hv + hv
-  const int64_t token = row / Hv;
-  const int hv = static_cast<int>(row - token * Hv);
-  int64_t dst;
-  if (varlen) {
-    dst = static_cast<int64_t>(hv) * N + token;
-  } else {
-    const int64_t b = token / T;
-    dst = (b * Hv + hv) * T + (token - b * T);
-  }
+  const int64_t dst = value_word_row(row, Hv, T, N, varlen);
   for (int w = 0; w < nvw; ++w) {
     uint32_t word = 0u;
     for (int bit = 0; bit < 32; ++bit) {
@@ -2050,12 +2075,20 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   int32_t* counter = at<int32_t>(workspace, w.header) + 1;
   const bool analytic = analytic_reference_is_safe(L, scale);
 
-  hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>, dim3(blocks_for(view.symbol_rows, 256)),
-                     dim3(256), 0, stream, grad_output, grad_rows, view.symbol_rows,
-                     L.H, L.Dv, dvp, L.T, L.N, L.varlen, full_width, value_offset);
-  hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
-                     dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
-                     L.T, L.N, L.varlen, full_width, value_offset);
+  hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>,
+                     dim3(blocks_for(view.symbol_rows * dvp, 256)), dim3(256), 0, stream,
+                     grad_output, grad_rows, view.symbol_rows, L.H, L.Dv, dvp, L.T, L.N, L.varlen,
+                     full_width, value_offset);
+  if (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) {
+    hipLaunchKernelGGL(pack_value_bits_ballot_kernel<DTYPE>,
+                       dim3(blocks_for(view.value_rows * L.Dv, 256)), dim3(256), 0, stream, value,
+                       value_bits, view.value_rows, L.Hv, L.Dv, nvw, L.T, L.N, L.varlen,
+                       full_width, value_offset);
+  } else {
+    hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
+                       dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
+                       L.T, L.N, L.varlen, full_width, value_offset);
+  }
   if (L.varlen) {
     hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
                        dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
