@@ -474,44 +474,77 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
   const bool row_ok = t < u.len;
   const uint32_t q_word = row_ok ? q[t] : 0u;
   const int W = L.W;
-  using Best = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
-  Best best = 0;
-  int run = 0;
   const int a_last = min(t0 + kWave - 1, u.len - 1);
-  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
-    const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
-    int halo = 0;
-    if (column >= 1 && column <= t0 - 1) {
-      const int limit = min(W, column);
-      while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
-    }
-    const uint32_t key_chunk = column < u.len ? k[column] : 0u;  // key word of route a0 + lane
-    const int count = min(kWave, a_last - a0 + 1);
-#pragma unroll
-    for (int j = 0; j < kWave; ++j) {
-      if (j >= count) break;
-      const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
-      const int halo_j = __builtin_amdgcn_readlane(halo, j);
-      const int above = dpp_wave_shr1(halo_j, run);
-      const int a = a0 + j;
-      const bool match = (q_word == k_word) && (a <= t);
-      run = match ? min(above + 1, W) : 0;
-      if constexpr (WIDE) {
-        best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
-      } else {
-        best = max(best, (static_cast<uint32_t>(run) << shift) | static_cast<uint32_t>(a));
-      }
-    }
-  }
-  if (!row_ok) return;
   int best_run, best_route;
   if constexpr (WIDE) {
+    uint64_t best = 0;
+    int run = 0;
+    for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+      const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
+      int halo = 0;
+      if (column >= 1 && column <= t0 - 1) {
+        const int limit = min(W, column);
+        while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+      }
+      const uint32_t key_chunk = column < u.len ? k[column] : 0u;  // key word of route a0 + lane
+      const int count = min(kWave, a_last - a0 + 1);
+      for (int j = 0; j < count; ++j) {
+        const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
+        const int halo_j = __builtin_amdgcn_readlane(halo, j);
+        const int above = dpp_wave_shr1(halo_j, run);
+        const int a = a0 + j;
+        const bool match = (q_word == k_word) && (a <= t);
+        run = match ? min(above + 1, W) : 0;
+        best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
+      }
+    }
     best_run = static_cast<int>(best >> 32);
     best_route = static_cast<int>(best & 0xffffffffu);
   } else {
-    best_run = static_cast<int>(best >> shift);
-    best_route = static_cast<int>(best & ((1u << shift) - 1u));
+    // The same recurrence on `missing` = (W - run) << shift, so that the step is one
+    // saturating subtraction and the key needs no shift: the winner is the *minimum* of
+    // missing | (low - a), i.e. longest run first, latest route on ties.
+    const uint32_t one = 1u << shift;
+    const uint32_t low = one - 1u;
+    const uint32_t cap = static_cast<uint32_t>(W) << shift;
+    uint32_t best = cap | low;  // run 0
+    uint32_t missing = cap;
+    for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+      const int column = a0 - 1 + lane;
+      int halo = 0;
+      if (column >= 1 && column <= t0 - 1) {
+        const int limit = min(W, column);
+        while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+      }
+      const uint32_t halo_missing = cap - (static_cast<uint32_t>(halo) << shift);
+      const uint32_t key_chunk = column < u.len ? k[column] : 0u;
+      const uint32_t route_low = low - static_cast<uint32_t>(a0);
+      if (a0 + kWave - 1 <= t0) {
+        // every route of the chunk precedes every row of the block: nothing to mask
+#pragma unroll
+        for (int j = 0; j < kWave; ++j) {
+          const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
+          const uint32_t above =
+              dpp_wave_shr1(static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+          missing = q_word == k_word ? __builtin_elementwise_sub_sat(above, one) : cap;
+          best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+        }
+      } else {
+        const int count = min(kWave, a_last - a0 + 1);
+        for (int j = 0; j < count; ++j) {
+          const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
+          const uint32_t above =
+              dpp_wave_shr1(static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+          const bool match = (q_word == k_word) && (a0 + j <= t);
+          missing = match ? __builtin_elementwise_sub_sat(above, one) : cap;
+          best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+        }
+      }
+    }
+    best_run = W - static_cast<int>(best >> shift);
+    best_route = static_cast<int>(low - (best & low));
   }
+  if (!row_ok) return;
   const int route = best_run > 0 ? best_route : 0;
   if (routes != nullptr) routes[u.word_base + t] = route;
   if (lengths != nullptr) lengths[u.word_base + t] = best_run;
