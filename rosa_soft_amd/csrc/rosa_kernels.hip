@@ -454,8 +454,98 @@ __global__ __launch_bounds__(256) void pack_symbols_rows_kernel(
 // run(t-1, a-1) is the previous step's value of the lane above, fetched with
 // one DPP shift.  Lane 0 has no lane above: its predecessor row t0-1 is
 // evaluated directly, 64 routes at a time, by an early-exit compare loop.
-// The winner is the maximum of the packed key (run << shift) | a, which is
-// "longest first, latest on ties"; a zero run never produces a route.
+// The winner is "longest first, latest on ties"; a zero run never produces a route.
+// Both scans serve the training forward (32-bit symbol words) and the streaming router
+// (byte symbols): `q` and `k` are the symbols of one (sequence, head), `length` rows long.
+struct RouteWinner {
+  int run;    // matched suffix length, 0 if no route matched
+  int route;  // a, meaningful when run > 0
+};
+
+// run length of route `column` on row t0 - 1 (the row above the block), for lane 0
+template <typename Symbol>
+__device__ __forceinline__ int halo_run(const Symbol* q, const Symbol* k, int t0, int column,
+                                        int W) {
+  int halo = 0;
+  if (column >= 1 && column <= t0 - 1) {
+    const int limit = min(W, column);
+    while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+  }
+  return halo;
+}
+
+// Any length: the winner is the maximum of the 64-bit key (run << 32) | a.
+template <typename Symbol>
+__device__ __forceinline__ RouteWinner scan_routes_wide(const Symbol* q, const Symbol* k, int t0,
+                                                        int length, int W, int lane,
+                                                        uint32_t q_symbol) {
+  const int t = t0 + lane;
+  const int a_last = min(t0 + kWave - 1, length - 1);
+  uint64_t best = 0;
+  int run = 0;
+  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+    const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
+    const int halo = halo_run(q, k, t0, column, W);
+    const uint32_t key_chunk = column < length ? k[column] : 0u;  // key symbol of route a0 + lane
+    const int count = min(kWave, a_last - a0 + 1);
+    for (int j = 0; j < count; ++j) {
+      const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+      const int halo_j = __builtin_amdgcn_readlane(halo, j);
+      const int above = dpp_wave_shr1(halo_j, run);
+      const int a = a0 + j;
+      const bool match = (q_symbol == k_symbol) && (a <= t);
+      run = match ? min(above + 1, W) : 0;
+      best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
+    }
+  }
+  return RouteWinner{static_cast<int>(best >> 32), static_cast<int>(best & 0xffffffffu)};
+}
+
+// length < 2^shift and W < 2^(32 - shift).  The same recurrence on
+// `missing` = (W - run) << shift, so that the step is one saturating subtraction and the
+// key needs no shift: the winner is the *minimum* of missing | (low - a).  Chunks of 64
+// routes that lie entirely below the row block need no causal mask and are unrolled.
+template <typename Symbol>
+__device__ __forceinline__ RouteWinner scan_routes_narrow(const Symbol* q, const Symbol* k,
+                                                          int t0, int length, int W, int shift,
+                                                          int lane, uint32_t q_symbol) {
+  const int t = t0 + lane;
+  const int a_last = min(t0 + kWave - 1, length - 1);
+  const uint32_t one = 1u << shift;
+  const uint32_t low = one - 1u;
+  const uint32_t cap = static_cast<uint32_t>(W) << shift;
+  uint32_t best = cap | low;  // run 0
+  uint32_t missing = cap;
+  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
+    const int column = a0 - 1 + lane;
+    const int halo = halo_run(q, k, t0, column, W);
+    const uint32_t halo_missing = cap - (static_cast<uint32_t>(halo) << shift);
+    const uint32_t key_chunk = column < length ? k[column] : 0u;
+    const uint32_t route_low = low - static_cast<uint32_t>(a0);
+    if (a0 + kWave - 1 <= t0) {
+#pragma unroll
+      for (int j = 0; j < kWave; ++j) {
+        const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+        const uint32_t above = dpp_wave_shr1(
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+        missing = q_symbol == k_symbol ? __builtin_elementwise_sub_sat(above, one) : cap;
+        best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+      }
+    } else {
+      const int count = min(kWave, a_last - a0 + 1);
+      for (int j = 0; j < count; ++j) {
+        const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+        const uint32_t above = dpp_wave_shr1(
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+        const bool match = (q_symbol == k_symbol) && (a0 + j <= t);
+        missing = match ? __builtin_elementwise_sub_sat(above, one) : cap;
+        best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+      }
+    }
+  }
+  return RouteWinner{W - static_cast<int>(best >> shift), static_cast<int>(low - (best & low))};
+}
+
 template <bool VARLEN, bool WIDE>
 __global__ __launch_bounds__(kWave) void hard_route_kernel(
     Layout L, const uint32_t* __restrict__ packed_query,
@@ -473,81 +563,12 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
   const int t = t0 + lane;
   const bool row_ok = t < u.len;
   const uint32_t q_word = row_ok ? q[t] : 0u;
-  const int W = L.W;
-  const int a_last = min(t0 + kWave - 1, u.len - 1);
-  int best_run, best_route;
-  if constexpr (WIDE) {
-    uint64_t best = 0;
-    int run = 0;
-    for (int a0 = 1; a0 <= a_last; a0 += kWave) {
-      const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
-      int halo = 0;
-      if (column >= 1 && column <= t0 - 1) {
-        const int limit = min(W, column);
-        while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
-      }
-      const uint32_t key_chunk = column < u.len ? k[column] : 0u;  // key word of route a0 + lane
-      const int count = min(kWave, a_last - a0 + 1);
-      for (int j = 0; j < count; ++j) {
-        const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
-        const int halo_j = __builtin_amdgcn_readlane(halo, j);
-        const int above = dpp_wave_shr1(halo_j, run);
-        const int a = a0 + j;
-        const bool match = (q_word == k_word) && (a <= t);
-        run = match ? min(above + 1, W) : 0;
-        best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
-      }
-    }
-    best_run = static_cast<int>(best >> 32);
-    best_route = static_cast<int>(best & 0xffffffffu);
-  } else {
-    // The same recurrence on `missing` = (W - run) << shift, so that the step is one
-    // saturating subtraction and the key needs no shift: the winner is the *minimum* of
-    // missing | (low - a), i.e. longest run first, latest route on ties.
-    const uint32_t one = 1u << shift;
-    const uint32_t low = one - 1u;
-    const uint32_t cap = static_cast<uint32_t>(W) << shift;
-    uint32_t best = cap | low;  // run 0
-    uint32_t missing = cap;
-    for (int a0 = 1; a0 <= a_last; a0 += kWave) {
-      const int column = a0 - 1 + lane;
-      int halo = 0;
-      if (column >= 1 && column <= t0 - 1) {
-        const int limit = min(W, column);
-        while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
-      }
-      const uint32_t halo_missing = cap - (static_cast<uint32_t>(halo) << shift);
-      const uint32_t key_chunk = column < u.len ? k[column] : 0u;
-      const uint32_t route_low = low - static_cast<uint32_t>(a0);
-      if (a0 + kWave - 1 <= t0) {
-        // every route of the chunk precedes every row of the block: nothing to mask
-#pragma unroll
-        for (int j = 0; j < kWave; ++j) {
-          const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
-          const uint32_t above =
-              dpp_wave_shr1(static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
-          missing = q_word == k_word ? __builtin_elementwise_sub_sat(above, one) : cap;
-          best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
-        }
-      } else {
-        const int count = min(kWave, a_last - a0 + 1);
-        for (int j = 0; j < count; ++j) {
-          const uint32_t k_word = __builtin_amdgcn_readlane(key_chunk, j);
-          const uint32_t above =
-              dpp_wave_shr1(static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
-          const bool match = (q_word == k_word) && (a0 + j <= t);
-          missing = match ? __builtin_elementwise_sub_sat(above, one) : cap;
-          best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
-        }
-      }
-    }
-    best_run = W - static_cast<int>(best >> shift);
-    best_route = static_cast<int>(low - (best & low));
-  }
+  const RouteWinner winner = WIDE ? scan_routes_wide(q, k, t0, u.len, L.W, lane, q_word)
+                                  : scan_routes_narrow(q, k, t0, u.len, L.W, shift, lane, q_word);
   if (!row_ok) return;
-  const int route = best_run > 0 ? best_route : 0;
+  const int route = winner.run > 0 ? winner.route : 0;
   if (routes != nullptr) routes[u.word_base + t] = route;
-  if (lengths != nullptr) lengths[u.word_base + t] = best_run;
+  if (lengths != nullptr) lengths[u.word_base + t] = winner.run;
   source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
 }
 
@@ -2273,31 +2294,13 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
   const int t = t0 + lane;
   const bool row_ok = t < new_length;
   const uint32_t q_symbol = row_ok ? q[t] : 0u;
-  const int W = U.W;
-  uint64_t best = 0;
-  int run = 0;
-  const int a_last = min(t0 + kWave - 1, new_length - 1);
-  for (int a0 = 1; a0 <= a_last; a0 += kWave) {
-    const int column = a0 - 1 + lane;  // route index on the predecessor row t0 - 1
-    int halo = 0;
-    if (column >= 1 && column <= t0 - 1) {
-      const int limit = min(W, column);
-      while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
-    }
-    const uint32_t key_chunk = column < new_length ? k[column] : 0u;  // key of route a0 + lane
-    const int count = min(kWave, a_last - a0 + 1);
-    for (int j = 0; j < count; ++j) {
-      const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
-      const int halo_j = __builtin_amdgcn_readlane(halo, j);
-      const int above = dpp_wave_shr1(halo_j, run);
-      const int a = a0 + j;
-      const bool match = (q_symbol == k_symbol) && (a <= t);
-      run = match ? min(above + 1, W) : 0;
-      best = max(best, (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a));
-    }
-  }
+  const int shift = 32 - __clz(new_length);  // new_length < 2^shift
+  const bool narrow = shift <= 16 && U.W < 65536;
+  const RouteWinner winner =
+      narrow ? scan_routes_narrow(q, k, t0, new_length, U.W, shift, lane, q_symbol)
+             : scan_routes_wide(q, k, t0, new_length, U.W, lane, q_symbol);
   if (!row_ok) return;
-  const int route = (best >> 32) > 0 ? static_cast<int>(best & 0xffffffffu) : 0;
+  const int route = winner.run > 0 ? winner.route : 0;
   const int64_t token = chunk_begin + (t - old_length);
   const int payload_head = head / (U.H / U.Hp);
   U.matched_key_end[token * U.H + head] = route > 0 ? route - 1 : -1;
