@@ -1287,6 +1287,7 @@ __global__ __launch_bounds__(kWave)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
+  constexpr bool kFetchAhead = VT == 1 && DT == 1;  // registers to spare for operands in flight
   constexpr int GP = DVP;               // pitch of the staged grad_output rows
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
@@ -1613,22 +1614,49 @@ void vjp_gradients_kernel(VjpParams P) {
         // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
         // element (column c, row r) of the skewed matrix is tile[r][64 - c + r].
         if (want_v) {
-#pragma unroll
-          for (int step = 0; step < kChunk / 4; ++step) {
+          // narrow tiles: operands of every product are fetched one k step ahead, without
+          // branches, so that the loads of a step fly while the products of the step before
+          // it run (wide tiles have no registers to spare for that)
+          float a_next[kWindowTiles];
+          float grad_next[VT];
+          const auto fetch = [&](int step) {
             const int r = step + 4 * lg;
-            float grad_b[VT];
 #pragma unroll
             for (int n = 0; n < VT; ++n) {
-              grad_b[n] = (16 * n + li < DVP) ? grad_tile[r * GP + 16 * n + li] : 0.0f;
+              grad_next[n] = grad_tile[r * GP + min(16 * n + li, DVP - 1)];
             }
 #pragma unroll
             for (int m = 0; m < kWindowTiles; ++m) {
-              const float a_value = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+              a_next[m] = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+            }
+          };
+          if constexpr (kFetchAhead) fetch(0);
+#pragma unroll
+          for (int step = 0; step < kChunk / 4; ++step) {
+            if constexpr (!kFetchAhead) fetch(step);
+            float a_now[kWindowTiles];
+            float grad_now[VT];
+#pragma unroll
+            for (int m = 0; m < kWindowTiles; ++m) a_now[m] = a_next[m];
+#pragma unroll
+            for (int n = 0; n < VT; ++n) grad_now[n] = grad_next[n];
+            if constexpr (kFetchAhead) {
+              if (step + 1 < kChunk / 4) fetch(step + 1);
+              // keep the loads above the products (the scheduler would sink each load to its use)
+              __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int n = 0; n < VT; ++n) {  // columns past the value width are padding
+              if (16 * n + li >= DVP) grad_now[n] = 0.0f;
+            }
+#pragma unroll
+            for (int m = 0; m < kWindowTiles; ++m) {
 #pragma unroll
               for (int n = 0; n < VT; ++n) {
-                value_acc[m][n] = mfma_16x16x4(a_value, grad_b[n], value_acc[m][n]);
+                value_acc[m][n] = mfma_16x16x4(a_now[m], grad_now[n], value_acc[m][n]);
               }
             }
+            if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
           }
         }
 
@@ -1681,21 +1709,39 @@ void vjp_gradients_kernel(VjpParams P) {
           wave_lds_fence();
 
           if (want_k) {
-#pragma unroll
-            for (int step = 0; step < kChunk / 4; ++step) {
+            float a_next[kWindowTiles];
+            uint32_t q_next = 0u;
+            const auto fetch = [&](int step) {
               const int r = step + 4 * lg;
-              float query_b[DT];
-              const uint32_t q_word = query_rows[local + r];
-#pragma unroll
-              for (int n = 0; n < DT; ++n) query_b[n] = negated_symbol(q_word, 16 * n + li);
+              q_next = query_rows[local + r];
 #pragma unroll
               for (int m = 0; m < kWindowTiles; ++m) {
-                const float a_value = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+                a_next[m] = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+              }
+            };
+            if constexpr (kFetchAhead) fetch(0);
+#pragma unroll
+            for (int step = 0; step < kChunk / 4; ++step) {
+              if constexpr (!kFetchAhead) fetch(step);
+              float a_now[kWindowTiles];
+#pragma unroll
+              for (int m = 0; m < kWindowTiles; ++m) a_now[m] = a_next[m];
+              const uint32_t q_word = q_next;
+              if constexpr (kFetchAhead) {
+                if (step + 1 < kChunk / 4) fetch(step + 1);
+              }
+              float query_b[DT];
+#pragma unroll
+              for (int n = 0; n < DT; ++n) query_b[n] = negated_symbol(q_word, 16 * n + li);
+              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int m = 0; m < kWindowTiles; ++m) {
 #pragma unroll
                 for (int n = 0; n < DT; ++n) {
-                  key_acc[m][n] = mfma_16x16x4(a_value, query_b[n], key_acc[m][n]);
+                  key_acc[m][n] = mfma_16x16x4(a_now[m], query_b[n], key_acc[m][n]);
                 }
               }
+              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
             }
           }
           // row sums: rows are complete for this band after the chunk
@@ -1720,16 +1766,27 @@ void vjp_gradients_kernel(VjpParams P) {
               key_words[4 * quad + 2] = four.z;
               key_words[4 * quad + 3] = four.w;
             }
+            // the tile column of step s, fetched kAhead steps before its product
+            constexpr int kAhead = kFetchAhead ? 8 : 1;
+            float a_ahead[kAhead];
+            const auto tile_value = [&](int step) {
+              const int c = 4 * kWindowTiles * lg + step;
+              return tile[li * kTilePitch + 16 + 64 - c + li];
+            };
+#pragma unroll
+            for (int step = 0; step < kAhead; ++step) a_ahead[step] = tile_value(step);
 #pragma unroll
             for (int step = 0; step < 4 * kWindowTiles; ++step) {
-              const int c = 4 * kWindowTiles * lg + step;
-              const float a_value = tile[li * kTilePitch + 16 + 64 - c + li];
+              const float a_value = a_ahead[step % kAhead];
+              if (step + kAhead < 4 * kWindowTiles) a_ahead[step % kAhead] = tile_value(step + kAhead);
+              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
                 query_part[step % kParts][n] =
                     mfma_16x16x4(a_value, negated_symbol(key_words[step], 16 * n + li),
                                  query_part[step % kParts][n]);
               }
+              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int n = 0; n < DT; ++n) {
