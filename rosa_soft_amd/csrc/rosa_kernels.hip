@@ -1461,29 +1461,120 @@ void vjp_gradients_kernel(VjpParams P) {
       }
       // one round trip brings in everything the segment needs
       wave_lds_fence();
-      stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W);
-      if (lane < SEG) {
-        const int i = seg_first + lane;
-        query_rows[lane] = i < view.steps ? view.q[view.diag0 + 1 + i] : 0u;
-      }
-      stage_grad_rows<DVP>(view, seg_first, SEG, lane, grad_rows_lds, GP);
-      for (int index = lane; index < SEG + kWave; index += kWave) {
-        const int a = seg_first - 63 + index;  // column; key position a - 1
-        key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
-        old_key_window[index] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
-      }
-      if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
-      if (stored) {
-        // the chunk records of the segment: (S, window) before each chunk, keep decisions
-        for (int chunk = 0; chunk < chunks; ++chunk) {
-          const float* slot = view.checkpoints +
-              static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
-          ck_evidence[chunk * kWave + lane] = slot[lane];
-          ck_window[chunk * kWave + lane] = __float_as_int(slot[kWave + lane]);
-          if constexpr (DROPOUT) {
-            ck_kept[chunk * kWave + lane] =
-                reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+      if constexpr (kFetchAhead) {
+        // Narrow tiles have the registers to issue every global load of the segment before
+        // the first of them is used, so the segment costs one memory latency, not one per
+        // staged array.
+        static_assert(SEG == kWave, "one row per lane");
+        const int i = min(seg_first + lane, view.steps - 1);  // rows past the end repeat the last
+        const int t = view.diag0 + 1 + i;
+        uint4 symbols;
+        symbols.x = view.q[t];
+        symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+        symbols.z = view.k[i];
+        symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
+        const uint4 record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
+        uint32_t key_in[2], old_key_in[2], value_in[2 * NVW];
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+          const int a = seg_first - 63 + part * kWave + lane;  // column; key position a - 1
+          key_in[part] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
+          old_key_in[part] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
+        }
+#pragma unroll
+        for (int part = 0; part < 2 * NVW; ++part) {
+          const int index = part * kWave + lane;
+          const int column = index / NVW;
+          const int a = seg_first - 63 + column;
+          value_in[part] = (want_qk && a >= 1 && a <= view.len - 1)
+              ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
+        }
+        constexpr int kQuads = DVP / 4;
+        float4 grad_in[kQuads];
+#pragma unroll
+        for (int part = 0; part < kQuads; ++part) {
+          const int index = part * kWave + lane;
+          const int r = index / kQuads;
+          grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (seg_first + r < view.steps) {
+            grad_in[part] = *reinterpret_cast<const float4*>(
+                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * DVP +
+                4 * (index - r * kQuads));
+          }
+        }
+        float record_evidence[SEG_CHUNKS];
+        int record_window[SEG_CHUNKS];
+        uint32_t record_kept[SEG_CHUNKS];
+#pragma unroll
+        for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
+          record_evidence[chunk] = 0.0f;
+          record_window[chunk] = 0;
+          record_kept[chunk] = 0u;
+          if (stored && chunk < chunks) {
+            // (S, window) before the chunk and, with dropout, its keep decisions
+            const float* slot = view.checkpoints +
+                static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
+            record_evidence[chunk] = slot[lane];
+            record_window[chunk] = __float_as_int(slot[kWave + lane]);
+            if constexpr (DROPOUT) {
+              record_kept[chunk] = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
+        row_words[0] = symbols;
+        row_words[1] = make_uint4(record.y, record.z, 0u, 0u);
+        query_rows[lane] = seg_first + lane < view.steps ? symbols.x : 0u;
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+          key_window[part * kWave + lane] = key_in[part];
+          old_key_window[part * kWave + lane] = old_key_in[part];
+        }
+        if (want_qk) {
+#pragma unroll
+          for (int part = 0; part < 2 * NVW; ++part) value_window[part * kWave + lane] = value_in[part];
+        }
+#pragma unroll
+        for (int part = 0; part < kQuads; ++part) {
+          const int index = part * kWave + lane;
+          const int r = index / kQuads;
+          *reinterpret_cast<float4*>(grad_rows_lds + r * GP + 4 * (index - r * kQuads)) =
+              grad_in[part];
+        }
+        if (stored) {
+#pragma unroll
+          for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
+            ck_evidence[chunk * kWave + lane] = record_evidence[chunk];
+            ck_window[chunk * kWave + lane] = record_window[chunk];
+            if constexpr (DROPOUT) ck_kept[chunk * kWave + lane] = record_kept[chunk];
+          }
+        }
+      } else {
+        stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W);
+        if (lane < SEG) {
+          const int i = seg_first + lane;
+          query_rows[lane] = i < view.steps ? view.q[view.diag0 + 1 + i] : 0u;
+        }
+        stage_grad_rows<DVP>(view, seg_first, SEG, lane, grad_rows_lds, GP);
+        for (int index = lane; index < SEG + kWave; index += kWave) {
+          const int a = seg_first - 63 + index;  // column; key position a - 1
+          key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
+          old_key_window[index] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
+        }
+        if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
+        if (stored) {
+          // the chunk records of the segment: (S, window) before each chunk, keep decisions
+          for (int chunk = 0; chunk < chunks; ++chunk) {
+            const float* slot = view.checkpoints +
+                static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
+            ck_evidence[chunk * kWave + lane] = slot[lane];
+            ck_window[chunk * kWave + lane] = __float_as_int(slot[kWave + lane]);
+            if constexpr (DROPOUT) {
+              ck_kept[chunk * kWave + lane] =
+                  reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+            }
           }
         }
       }
@@ -1547,22 +1638,35 @@ void vjp_gradients_kernel(VjpParams P) {
           constexpr bool QUIET = decltype(quiet_tag)::value;    // overflow terms are negligible
           const uint32_t* row = rows + local * kRowWords;
           const float* slot = tile + 16 + lane;
-          uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
-          uint4 next_extra = *reinterpret_cast<const uint4*>(row + 4);
-          float next_utility = *slot;
+          // row words and utilities are fetched kRowsAhead rows before their use
+          constexpr int kRowsAhead = kFetchAhead ? 2 : 1;
+          uint4 ahead_symbols[kRowsAhead];
+          uint4 ahead_extra[kRowsAhead];
+          float ahead_utility[kRowsAhead];
+#pragma unroll
+          for (int r = 0; r < kRowsAhead; ++r) {
+            ahead_symbols[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords);
+            ahead_extra[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords + 4);
+            ahead_utility[r] = slot[r * kTilePitch];
+          }
 #pragma unroll
           for (int r = 0; r < kChunk; ++r) {
-            const RowSymbols symbols{next_symbols.x, next_symbols.y, next_symbols.z,
-                                     next_symbols.w};
-            const uint4 extra = next_extra;
+            const uint4 words = ahead_symbols[r % kRowsAhead];
+            const RowSymbols symbols{words.x, words.y, words.z, words.w};
+            const uint4 extra = ahead_extra[r % kRowsAhead];
             // the slot holds the pair's utility (anything finite when no symbol
             // gradient is wanted, in which case the adjoint is never used)
-            const float utility = next_utility;
-            if (r + 1 < kChunk) {  // the next row's words are on their way while this one runs
-              next_symbols = *reinterpret_cast<const uint4*>(row + (r + 1) * kRowWords);
-              next_extra = *reinterpret_cast<const uint4*>(row + (r + 1) * kRowWords + 4);
-              next_utility = slot[(r + 1) * kTilePitch];
+            const float utility = ahead_utility[r % kRowsAhead];
+            if (r + kRowsAhead < kChunk) {
+              const int ahead = r + kRowsAhead;
+              ahead_symbols[r % kRowsAhead] =
+                  *reinterpret_cast<const uint4*>(row + ahead * kRowWords);
+              ahead_extra[r % kRowsAhead] =
+                  *reinterpret_cast<const uint4*>(row + ahead * kRowWords + 4);
+              ahead_utility[r % kRowsAhead] = slot[ahead * kTilePitch];
             }
+            // the loads stay here, ahead of their use (the scheduler would sink them)
+            if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
             const bool row_ok = r < rows_here;
             const int i = min(first + r, last_step);
             const int t = view.diag0 + 1 + i;
