@@ -1462,46 +1462,57 @@ void vjp_gradients_kernel(VjpParams P) {
       // one round trip brings in everything the segment needs
       wave_lds_fence();
       const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
-      if constexpr (kFetchAhead) {
-        // Narrow tiles have the registers to issue every global load of the segment before
-        // the first of them is used, so the segment costs one memory latency, not one per
-        // staged array.
-        static_assert(SEG == kWave, "one row per lane");
+      constexpr bool kHeavy = VT > 2 || DT > 1;
+      if constexpr (!kHeavy) {
+        // Every global load of the segment is issued before the first of them is used, so
+        // the segment costs one memory latency (two when the grad_output rows need the
+        // registers of the other arrays), not one per staged array.  The widest tiles have
+        // no registers to spare at this point and stage array by array.
+        const bool row_lane = lane < SEG;
         const int i = min(seg_first + lane, view.steps - 1);  // rows past the end repeat the last
         const int t = view.diag0 + 1 + i;
-        uint4 symbols;
-        symbols.x = view.q[t];
-        symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
-        symbols.z = view.k[i];
-        symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
-        const uint4 record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
-        uint32_t key_in[2], old_key_in[2], value_in[2 * NVW];
-#pragma unroll
-        for (int part = 0; part < 2; ++part) {
-          const int a = seg_first - 63 + part * kWave + lane;  // column; key position a - 1
-          key_in[part] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
-          old_key_in[part] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
+        uint4 symbols = make_uint4(0u, 0u, 0u, 0u);
+        uint4 record = make_uint4(0u, 0u, 0u, 0u);
+        if (row_lane) {
+          symbols.x = view.q[t];
+          symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+          symbols.z = view.k[i];
+          symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
+          record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
         }
+        constexpr int kKeyParts = (SEG + 2 * kWave - 1) / kWave;
+        uint32_t key_in[kKeyParts], old_key_in[kKeyParts];
 #pragma unroll
-        for (int part = 0; part < 2 * NVW; ++part) {
+        for (int part = 0; part < kKeyParts; ++part) {
+          const int a = seg_first - 63 + part * kWave + lane;  // column; key position a - 1
+          const bool inside = part * kWave + lane < SEG + kWave && a <= view.len - 1;
+          key_in[part] = (inside && a >= 1) ? view.k[a - 1] : 0u;
+          old_key_in[part] = (inside && a - W - 2 >= 0) ? view.k[a - W - 2] : 0u;
+        }
+        const auto store_rows_and_keys = [&]() {
+          if (row_lane) {
+            uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
+            row_words[0] = symbols;
+            row_words[1] = make_uint4(record.y, record.z, 0u, 0u);
+            query_rows[lane] = seg_first + lane < view.steps ? symbols.x : 0u;
+          }
+#pragma unroll
+          for (int part = 0; part < kKeyParts; ++part) {
+            if (part * kWave + lane < SEG + kWave) {
+              key_window[part * kWave + lane] = key_in[part];
+              old_key_window[part * kWave + lane] = old_key_in[part];
+            }
+          }
+        };
+        constexpr int kValueParts = ((SEG + kWave) * NVW + kWave - 1) / kWave;
+        uint32_t value_in[kValueParts];
+#pragma unroll
+        for (int part = 0; part < kValueParts; ++part) {
           const int index = part * kWave + lane;
           const int column = index / NVW;
           const int a = seg_first - 63 + column;
-          value_in[part] = (want_qk && a >= 1 && a <= view.len - 1)
+          value_in[part] = (want_qk && column < SEG + kWave && a >= 1 && a <= view.len - 1)
               ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
-        }
-        constexpr int kQuads = DVP / 4;
-        float4 grad_in[kQuads];
-#pragma unroll
-        for (int part = 0; part < kQuads; ++part) {
-          const int index = part * kWave + lane;
-          const int r = index / kQuads;
-          grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          if (seg_first + r < view.steps) {
-            grad_in[part] = *reinterpret_cast<const float4*>(
-                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * DVP +
-                4 * (index - r * kQuads));
-          }
         }
         float record_evidence[SEG_CHUNKS];
         int record_window[SEG_CHUNKS];
@@ -1522,34 +1533,64 @@ void vjp_gradients_kernel(VjpParams P) {
             }
           }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
-        row_words[0] = symbols;
-        row_words[1] = make_uint4(record.y, record.z, 0u, 0u);
-        query_rows[lane] = seg_first + lane < view.steps ? symbols.x : 0u;
+        const auto store_values_and_records = [&]() {
+          if (want_qk) {
 #pragma unroll
-        for (int part = 0; part < 2; ++part) {
-          key_window[part * kWave + lane] = key_in[part];
-          old_key_window[part * kWave + lane] = old_key_in[part];
-        }
-        if (want_qk) {
-#pragma unroll
-          for (int part = 0; part < 2 * NVW; ++part) value_window[part * kWave + lane] = value_in[part];
-        }
-#pragma unroll
-        for (int part = 0; part < kQuads; ++part) {
-          const int index = part * kWave + lane;
-          const int r = index / kQuads;
-          *reinterpret_cast<float4*>(grad_rows_lds + r * GP + 4 * (index - r * kQuads)) =
-              grad_in[part];
-        }
-        if (stored) {
-#pragma unroll
-          for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
-            ck_evidence[chunk * kWave + lane] = record_evidence[chunk];
-            ck_window[chunk * kWave + lane] = record_window[chunk];
-            if constexpr (DROPOUT) ck_kept[chunk * kWave + lane] = record_kept[chunk];
+            for (int part = 0; part < kValueParts; ++part) {
+              if (part * kWave + lane < (SEG + kWave) * NVW) {
+                value_window[part * kWave + lane] = value_in[part];
+              }
+            }
           }
+          if (stored) {
+#pragma unroll
+            for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
+              ck_evidence[chunk * kWave + lane] = record_evidence[chunk];
+              ck_window[chunk * kWave + lane] = record_window[chunk];
+              if constexpr (DROPOUT) ck_kept[chunk * kWave + lane] = record_kept[chunk];
+            }
+          }
+        };
+        const auto store_rows_and_columns = [&]() {
+          store_rows_and_keys();
+          store_values_and_records();
+        };
+        if constexpr (!kFetchAhead) {
+          __builtin_amdgcn_sched_barrier(0);
+          store_rows_and_columns();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        constexpr int kQuads = DVP / 4;
+        constexpr int kGradParts = SEG * kQuads / kWave;
+        static_assert(kGradParts * kWave == SEG * kQuads, "whole float4s per lane");
+        // the grad_output rows come in groups that fit the registers free at this point
+        constexpr int kGradGroup = kGradParts;
+#pragma unroll
+        for (int group = 0; group < kGradParts; group += kGradGroup) {
+          float4 grad_in[kGradGroup];
+#pragma unroll
+          for (int part = 0; part < kGradGroup; ++part) {
+            const int index = (group + part) * kWave + lane;
+            const int r = index / kQuads;
+            grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (seg_first + r < view.steps) {
+              grad_in[part] = *reinterpret_cast<const float4*>(
+                  view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * DVP +
+                  4 * (index - r * kQuads));
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (kFetchAhead) {
+            if (group == 0) store_rows_and_columns();
+          }
+#pragma unroll
+          for (int part = 0; part < kGradGroup; ++part) {
+            const int index = (group + part) * kWave + lane;
+            const int r = index / kQuads;
+            *reinterpret_cast<float4*>(grad_rows_lds + r * GP + 4 * (index - r * kQuads)) =
+                grad_in[part];
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       } else {
         stage_rows<NVW, kRowFull>(view, seg_first, SEG, lane, rows, W);
