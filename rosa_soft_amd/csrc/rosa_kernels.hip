@@ -92,6 +92,12 @@ __device__ __forceinline__ uint32_t dpp_wave_shr1(uint32_t fill_lane0, uint32_t 
       dpp_wave_shr1(static_cast<int>(fill_lane0), static_cast<int>(src)));
 }
 
+// lanes 8..15 of every 16 receive src of the lane eight below; lanes 0..7 keep `keep`
+__device__ __forceinline__ float dpp_row_shr8(float keep, float src) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(keep), __float_as_int(src),
+                                                    0x118, 0xf, 0xf, false));
+}
+
 template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ float dpp_add(float acc, float src) {
   const int moved =
@@ -1389,58 +1395,57 @@ void vjp_gradients_kernel(VjpParams P) {
     v4f done_query[DT];
     int done_first = -1;  // first step of the chunk whose results are pending (-1: none)
     int done_rows = 0;
+    // One completed 16 x 16 tile: lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li.
+    // With at most 8 live columns the upper half of every 16 lanes takes rows e + 2 from the
+    // lower half, so that two instructions carry what would otherwise take four.
+    auto add_tile = [&](float* base, int64_t row_stride, int columns, v4f values, float scale,
+                        int rows_left) {
+      // base: element (row 4 lg, column 0); rows_left: valid rows counted from row 4 lg
+      if (columns <= 8) {
+        const int half = li >> 3;
+        const float first = dpp_row_shr8(values[0], values[2]);
+        const float second = dpp_row_shr8(values[1], values[3]);
+        if ((li & 7) < columns) {
+          float* target = base + (li & 7) + 2 * half * row_stride;
+          if (2 * half < rows_left) atomicAdd(target, scale * first);
+          if (2 * half + 1 < rows_left) atomicAdd(target + row_stride, scale * second);
+        }
+      } else if (li < columns) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (e < rows_left) atomicAdd(base + li + e * row_stride, scale * values[e]);
+        }
+      }
+    };
     auto issue_pending = [&]() {
       if (done_first < 0) return;
-      const bool full = done_rows == kChunk;  // then every row and column of the chunk exists
       const int64_t row0 = static_cast<int64_t>(u.start) + view.diag0 + 1 + done_first + 4 * lg;
       const int64_t column0 = static_cast<int64_t>(u.start) + done_first + 1 + 4 * lg;
       const int64_t last_token = static_cast<int64_t>(u.start) + view.len - 1;
       const int64_t symbol_stride = static_cast<int64_t>(P.L.H) * D;
       const int64_t value_stride = static_cast<int64_t>(P.L.Hv) * P.value_stride;
+      const int rows_left = done_rows - 4 * lg;
+      const int columns_left =
+          static_cast<int>(min(static_cast<int64_t>(kChunk), last_token - column0 + 1));
       if (want_q) {
 #pragma unroll
         for (int n = 0; n < DT; ++n) {
-          const int bit = 16 * n + li;
-          if (bit < D) {
-            float* target = P.grad_query + (row0 * P.L.H + u.head) * D + bit;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (full || 4 * lg + e < done_rows) {
-                atomicAdd(target + e * symbol_stride, symbol_scale * done_query[n][e]);
-              }
-            }
-          }
+          add_tile(P.grad_query + (row0 * P.L.H + u.head) * D + 16 * n, symbol_stride, D - 16 * n,
+                   done_query[n], symbol_scale, rows_left);
         }
       }
       if (want_v) {
 #pragma unroll
         for (int n = 0; n < VT; ++n) {
-          const int d = 16 * n + li;
-          if (d < Dv) {
-            float* target =
-                P.grad_value + (column0 * P.L.Hv + hv) * P.value_stride + P.value_offset + d;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (full || column0 + e <= last_token) {
-                atomicAdd(target + e * value_stride, done_value[n][e]);
-              }
-            }
-          }
+          add_tile(P.grad_value + (column0 * P.L.Hv + hv) * P.value_stride + P.value_offset + 16 * n,
+                   value_stride, Dv - 16 * n, done_value[n], 1.0f, columns_left);
         }
       }
       if (want_k) {
 #pragma unroll
         for (int n = 0; n < DT; ++n) {
-          const int bit = 16 * n + li;
-          if (bit < D) {
-            float* target = P.grad_key + ((column0 - 1) * P.L.H + u.head) * D + bit;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (full || column0 + e <= last_token) {
-                atomicAdd(target + e * symbol_stride, symbol_scale * done_key[n][e]);
-              }
-            }
-          }
+          add_tile(P.grad_key + ((column0 - 1) * P.L.H + u.head) * D + 16 * n, symbol_stride,
+                   D - 16 * n, done_key[n], symbol_scale, columns_left);
         }
       }
       done_first = -1;
