@@ -1398,55 +1398,73 @@ void vjp_gradients_kernel(VjpParams P) {
     // One completed 16 x 16 tile: lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li.
     // With at most 8 live columns the upper half of every 16 lanes takes rows e + 2 from the
     // lower half, so that two instructions carry what would otherwise take four.
-    auto add_tile = [&](float* base, int64_t row_stride, int columns, v4f values, float scale,
-                        int rows_left) {
-      // base: element (row 4 lg, column 0); rows_left: valid rows counted from row 4 lg
+    // `base` (element (row 0, column 0) of the tile) and `row_stride` are wave-uniform, so
+    // the address of a lane is a scalar pointer plus a 32-bit lane offset; FULL tiles (every
+    // row exists) need no row test.
+    auto add_tile = [&](auto full_tag, float* base, uint32_t row_stride, int columns, v4f values,
+                        float scale, int rows_left) {
+      constexpr bool FULL = decltype(full_tag)::value;
+      // rows_left: valid rows counted from row 4 lg
       if (columns <= 8) {
         const int half = li >> 3;
         const float first = dpp_row_shr8(values[0], values[2]);
         const float second = dpp_row_shr8(values[1], values[3]);
         if ((li & 7) < columns) {
-          float* target = base + (li & 7) + 2 * half * row_stride;
-          if (2 * half < rows_left) atomicAdd(target, scale * first);
-          if (2 * half + 1 < rows_left) atomicAdd(target + row_stride, scale * second);
+          const uint32_t offset = static_cast<uint32_t>(4 * lg + 2 * half) * row_stride + (li & 7);
+          if (FULL || 2 * half < rows_left) atomicAdd(base + offset, scale * first);
+          if (FULL || 2 * half + 1 < rows_left) {
+            atomicAdd(base + row_stride + offset, scale * second);
+          }
         }
       } else if (li < columns) {
+        const uint32_t offset = static_cast<uint32_t>(4 * lg) * row_stride + li;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if (e < rows_left) atomicAdd(base + li + e * row_stride, scale * values[e]);
+          if (FULL || e < rows_left) atomicAdd(base + e * row_stride + offset, scale * values[e]);
         }
       }
     };
     auto issue_pending = [&]() {
       if (done_first < 0) return;
-      const int64_t row0 = static_cast<int64_t>(u.start) + view.diag0 + 1 + done_first + 4 * lg;
-      const int64_t column0 = static_cast<int64_t>(u.start) + done_first + 1 + 4 * lg;
+      // wave-uniform tokens of the tile's row 0 and column 0
+      const int64_t row_token = static_cast<int64_t>(u.start) + view.diag0 + 1 + done_first;
+      const int64_t column_token = static_cast<int64_t>(u.start) + done_first + 1;
       const int64_t last_token = static_cast<int64_t>(u.start) + view.len - 1;
-      const int64_t symbol_stride = static_cast<int64_t>(P.L.H) * D;
-      const int64_t value_stride = static_cast<int64_t>(P.L.Hv) * P.value_stride;
-      const int rows_left = done_rows - 4 * lg;
-      const int columns_left =
-          static_cast<int>(min(static_cast<int64_t>(kChunk), last_token - column0 + 1));
-      if (want_q) {
+      const uint32_t symbol_stride = static_cast<uint32_t>(P.L.H) * D;
+      const uint32_t value_stride = static_cast<uint32_t>(P.L.Hv) * P.value_stride;
+      float* query_base = P.grad_query + (row_token * P.L.H + u.head) * D;
+      float* key_base = P.grad_key + ((column_token - 1) * P.L.H + u.head) * D;
+      float* value_base =
+          P.grad_value + (column_token * P.L.Hv + hv) * P.value_stride + P.value_offset;
+      const auto add_all = [&](auto full_tag, int rows_left, int columns_left) {
+        if (want_q) {
 #pragma unroll
-        for (int n = 0; n < DT; ++n) {
-          add_tile(P.grad_query + (row0 * P.L.H + u.head) * D + 16 * n, symbol_stride, D - 16 * n,
-                   done_query[n], symbol_scale, rows_left);
+          for (int n = 0; n < DT; ++n) {
+            add_tile(full_tag, query_base + 16 * n, symbol_stride, D - 16 * n, done_query[n],
+                     symbol_scale, rows_left);
+          }
         }
-      }
-      if (want_v) {
+        if (want_v) {
 #pragma unroll
-        for (int n = 0; n < VT; ++n) {
-          add_tile(P.grad_value + (column0 * P.L.Hv + hv) * P.value_stride + P.value_offset + 16 * n,
-                   value_stride, Dv - 16 * n, done_value[n], 1.0f, columns_left);
+          for (int n = 0; n < VT; ++n) {
+            add_tile(full_tag, value_base + 16 * n, value_stride, Dv - 16 * n, done_value[n], 1.0f,
+                     columns_left);
+          }
         }
-      }
-      if (want_k) {
+        if (want_k) {
 #pragma unroll
-        for (int n = 0; n < DT; ++n) {
-          add_tile(P.grad_key + ((column0 - 1) * P.L.H + u.head) * D + 16 * n, symbol_stride,
-                   D - 16 * n, done_key[n], symbol_scale, columns_left);
+          for (int n = 0; n < DT; ++n) {
+            add_tile(full_tag, key_base + 16 * n, symbol_stride, D - 16 * n, done_key[n],
+                     symbol_scale, columns_left);
+          }
         }
+      };
+      if (done_rows == kChunk) {  // then every row and column of the chunk exists
+        add_all(std::true_type{}, kChunk, kChunk);
+      } else {
+        const int columns = static_cast<int>(
+            min(static_cast<int64_t>(kChunk), last_token - column_token + 1));
+        add_all(std::false_type{}, done_rows - 4 * lg, columns - 4 * lg);
       }
       done_first = -1;
     };
