@@ -1395,6 +1395,15 @@ void vjp_gradients_kernel(VjpParams P) {
     v4f done_query[DT];
     int done_first = -1;  // first step of the chunk whose results are pending (-1: none)
     int done_rows = 0;
+    // step 0 of the band: row diag0 + 1 (query gradients), column 1 (value gradients, key
+    // position 0)
+    const uint32_t symbol_stride = static_cast<uint32_t>(P.L.H) * D;
+    const uint32_t value_stride = static_cast<uint32_t>(P.L.Hv) * P.value_stride;
+    float* band_query_base = P.grad_query +
+        ((static_cast<int64_t>(u.start) + view.diag0 + 1) * P.L.H + u.head) * D;
+    float* band_key_base = P.grad_key + (static_cast<int64_t>(u.start) * P.L.H + u.head) * D;
+    float* band_value_base = P.grad_value +
+        ((static_cast<int64_t>(u.start) + 1) * P.L.Hv + hv) * P.value_stride + P.value_offset;
     // One completed 16 x 16 tile: lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li.
     // With at most 8 live columns the upper half of every 16 lanes takes rows e + 2 from the
     // lower half, so that two instructions carry what would otherwise take four.
@@ -1426,16 +1435,13 @@ void vjp_gradients_kernel(VjpParams P) {
     };
     auto issue_pending = [&]() {
       if (done_first < 0) return;
-      // wave-uniform tokens of the tile's row 0 and column 0
-      const int64_t row_token = static_cast<int64_t>(u.start) + view.diag0 + 1 + done_first;
-      const int64_t column_token = static_cast<int64_t>(u.start) + done_first + 1;
-      const int64_t last_token = static_cast<int64_t>(u.start) + view.len - 1;
-      const uint32_t symbol_stride = static_cast<uint32_t>(P.L.H) * D;
-      const uint32_t value_stride = static_cast<uint32_t>(P.L.Hv) * P.value_stride;
-      float* query_base = P.grad_query + (row_token * P.L.H + u.head) * D;
-      float* key_base = P.grad_key + ((column_token - 1) * P.L.H + u.head) * D;
+      // wave-uniform element (row 0, column 0) of the three tiles: the band's bases moved
+      // by the chunk's first step
+      const uint64_t symbol_step = static_cast<uint64_t>(static_cast<uint32_t>(done_first)) * symbol_stride;
+      float* query_base = band_query_base + symbol_step;
+      float* key_base = band_key_base + symbol_step;
       float* value_base =
-          P.grad_value + (column_token * P.L.Hv + hv) * P.value_stride + P.value_offset;
+          band_value_base + static_cast<uint64_t>(static_cast<uint32_t>(done_first)) * value_stride;
       const auto add_all = [&](auto full_tag, int rows_left, int columns_left) {
         if (want_q) {
 #pragma unroll
@@ -1462,8 +1468,7 @@ void vjp_gradients_kernel(VjpParams P) {
       if (done_rows == kChunk) {  // then every row and column of the chunk exists
         add_all(std::true_type{}, kChunk, kChunk);
       } else {
-        const int columns = static_cast<int>(
-            min(static_cast<int64_t>(kChunk), last_token - column_token + 1));
+        const int columns = min(kChunk, view.len - 1 - done_first);  // columns a <= len - 1
         add_all(std::false_type{}, done_rows - 4 * lg, columns - 4 * lg);
       }
       done_first = -1;
