@@ -1474,6 +1474,22 @@ void vjp_gradients_kernel(VjpParams P) {
       done_first = -1;
     };
 
+    // Chunk records written by the row-statistics pass, (S, window) before the chunk and
+    // with dropout its keep decisions: each is fetched one chunk ahead of its use.
+    float record_evidence = 0.0f;
+    int record_window = 0;
+    uint32_t record_kept = 0u;
+    const auto fetch_record = [&](int chunk_index) {
+      const float* slot =
+          view.checkpoints + static_cast<int64_t>(chunk_index) * view.record_floats;
+      record_evidence = slot[lane];
+      record_window = __float_as_int(slot[kWave + lane]);
+      if constexpr (DROPOUT) {
+        record_kept = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
+      }
+    };
+    if (stored) fetch_record((view.steps - 1) / kChunk);
+
     for (int segment = segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * SEG;
       const int seg_last = min(view.steps, seg_first + SEG);
@@ -1542,26 +1558,7 @@ void vjp_gradients_kernel(VjpParams P) {
           value_in[part] = (want_qk && column < SEG + kWave && a >= 1 && a <= view.len - 1)
               ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
         }
-        float record_evidence[SEG_CHUNKS];
-        int record_window[SEG_CHUNKS];
-        uint32_t record_kept[SEG_CHUNKS];
-#pragma unroll
-        for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
-          record_evidence[chunk] = 0.0f;
-          record_window[chunk] = 0;
-          record_kept[chunk] = 0u;
-          if (stored && chunk < chunks) {
-            // (S, window) before the chunk and, with dropout, its keep decisions
-            const float* slot = view.checkpoints +
-                static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
-            record_evidence[chunk] = slot[lane];
-            record_window[chunk] = __float_as_int(slot[kWave + lane]);
-            if constexpr (DROPOUT) {
-              record_kept[chunk] = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
-            }
-          }
-        }
-        const auto store_values_and_records = [&]() {
+        const auto store_values = [&]() {
           if (want_qk) {
 #pragma unroll
             for (int part = 0; part < kValueParts; ++part) {
@@ -1570,18 +1567,10 @@ void vjp_gradients_kernel(VjpParams P) {
               }
             }
           }
-          if (stored) {
-#pragma unroll
-            for (int chunk = 0; chunk < SEG_CHUNKS; ++chunk) {
-              ck_evidence[chunk * kWave + lane] = record_evidence[chunk];
-              ck_window[chunk * kWave + lane] = record_window[chunk];
-              if constexpr (DROPOUT) ck_kept[chunk * kWave + lane] = record_kept[chunk];
-            }
-          }
         };
         const auto store_rows_and_columns = [&]() {
           store_rows_and_keys();
-          store_values_and_records();
+          store_values();
         };
         if constexpr (!kFetchAhead) {
           __builtin_amdgcn_sched_barrier(0);
@@ -1633,19 +1622,6 @@ void vjp_gradients_kernel(VjpParams P) {
           old_key_window[index] = (a - W - 2 >= 0 && a <= view.len - 1) ? view.k[a - W - 2] : 0u;
         }
         if (want_qk) stage_value_columns<NVW>(view, seg_first, SEG + kWave, lane, value_window);
-        if (stored) {
-          // the chunk records of the segment: (S, window) before each chunk, keep decisions
-          for (int chunk = 0; chunk < chunks; ++chunk) {
-            const float* slot = view.checkpoints +
-                static_cast<int64_t>(seg_first / kChunk + chunk) * view.record_floats;
-            ck_evidence[chunk * kWave + lane] = slot[lane];
-            ck_window[chunk * kWave + lane] = __float_as_int(slot[kWave + lane]);
-            if constexpr (DROPOUT) {
-              ck_kept[chunk * kWave + lane] =
-                  reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
-            }
-          }
-        }
       }
       wave_lds_fence();
       // segment-level forward sweep: checkpoint before every chunk
@@ -1663,12 +1639,23 @@ void vjp_gradients_kernel(VjpParams P) {
         const int local = chunk * kChunk;               // first row of the chunk inside the segment
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
-        band.evidence = ck_evidence[chunk * kWave + lane];
-        const int window_word = ck_window[chunk * kWave + lane];
+        int window_word;
+        uint32_t kept_bits = 0u;  // bit r: row r kept
+        if (stored) {
+          // this chunk's record arrived while the chunk after it ran; the record of the
+          // chunk before it sets out now
+          band.evidence = record_evidence;
+          window_word = record_window;
+          kept_bits = record_kept;
+          if (first >= kChunk) fetch_record(first / kChunk - 1);
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          band.evidence = ck_evidence[chunk * kWave + lane];
+          window_word = ck_window[chunk * kWave + lane];
+        }
         band.window = window_word & INT32_MAX;
         // stored records say whether any overflow term of the chunk matters
         const bool chunk_quiet = stored && __builtin_amdgcn_readfirstlane(window_word) >= 0;
-        const uint32_t kept_bits = DROPOUT ? ck_kept[chunk * kWave + lane] : 0u;  // bit r: row r kept
         // sliding registers of the chunk's first step: column first - lane
         band.key_word = key_window[local + 63 - lane];
         band.old_key_word = old_key_window[local + 63 - lane];
