@@ -1298,7 +1298,8 @@ void vjp_gradients_kernel(VjpParams P) {
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds[];
-  float* ck_evidence = lds;                                  // [SEG_CHUNKS][64]
+  float* ck_evidence = lds;       // [SEG_CHUNKS][64] (S, window) before each chunk when the
+                                  // row-statistics pass left no records
   int* ck_window = reinterpret_cast<int*>(lds + SEG_CHUNKS * kWave);
   float* tile = lds + 2 * SEG_CHUNKS * kWave;                // [kChunk][kTilePitch]
   float* grad_rows_lds = tile + kChunk * kTilePitch;         // [SEG][GP]
@@ -1309,7 +1310,6 @@ void vjp_gradients_kernel(VjpParams P) {
   float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
   uint32_t* old_key_window = reinterpret_cast<uint32_t*>(discard + kWave);  // [SEG + 64] key words
                                                              // of the columns W + 1 to the left
-  uint32_t* ck_kept = old_key_window + SEG + kWave;          // [SEG_CHUNKS][64] keep decisions
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1437,7 +1437,8 @@ void vjp_gradients_kernel(VjpParams P) {
       if (done_first < 0) return;
       // wave-uniform element (row 0, column 0) of the three tiles: the band's bases moved
       // by the chunk's first step
-      const uint64_t symbol_step = static_cast<uint64_t>(static_cast<uint32_t>(done_first)) * symbol_stride;
+      const uint64_t symbol_step =
+          static_cast<uint64_t>(static_cast<uint32_t>(done_first)) * symbol_stride;
       float* query_base = band_query_base + symbol_step;
       float* key_base = band_key_base + symbol_step;
       float* value_base =
@@ -1938,7 +1939,9 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
             for (int step = 0; step < 4 * kWindowTiles; ++step) {
               const float a_value = a_ahead[step % kAhead];
-              if (step + kAhead < 4 * kWindowTiles) a_ahead[step % kAhead] = tile_value(step + kAhead);
+              if (step + kAhead < 4 * kWindowTiles) {
+                a_ahead[step % kAhead] = tile_value(step + kAhead);
+              }
               if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
@@ -2270,7 +2273,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int GP = DVP;
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave + (SEG / kChunk) * kWave;
+                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave;
   const hipError_t attribute = hipFuncSetAttribute(
       reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
@@ -2335,91 +2338,92 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
                        grad_value, grad_value ? value_elements : 0);
   }
   for (int value_offset = 0; value_offset < full_width; value_offset += kValueSlice) {
-  L.Dv = std::min(kValueSlice, full_width - value_offset);
-  const int dvp = padded_value_width(L.Dv);
-  const int nvw = value_words(L.Dv);
-  if (value_offset > 0) stage_begin(kStagePrepare, stream);
+    L.Dv = std::min(kValueSlice, full_width - value_offset);
+    const int dvp = padded_value_width(L.Dv);
+    const int nvw = value_words(L.Dv);
+    if (value_offset > 0) stage_begin(kStagePrepare, stream);
 
-  float4* stats = at<float4>(workspace, w.stats);
-  float* grad_rows = at<float>(workspace, w.grad_rows);
-  uint32_t* value_bits = at<uint32_t>(workspace, w.value_bits);
-  int32_t* counter = at<int32_t>(workspace, w.header) + 1;
-  const bool analytic = analytic_reference_is_safe(L, scale);
+    float4* stats = at<float4>(workspace, w.stats);
+    float* grad_rows = at<float>(workspace, w.grad_rows);
+    uint32_t* value_bits = at<uint32_t>(workspace, w.value_bits);
+    int32_t* counter = at<int32_t>(workspace, w.header) + 1;
+    const bool analytic = analytic_reference_is_safe(L, scale);
 
-  hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>,
-                     dim3(blocks_for(view.symbol_rows * dvp, 256)), dim3(256), 0, stream,
-                     grad_output, grad_rows, view.symbol_rows, L.H, L.Dv, dvp, L.T, L.N, L.varlen,
-                     full_width, value_offset);
-  if (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) {
-    hipLaunchKernelGGL(pack_value_bits_ballot_kernel<DTYPE>,
-                       dim3(blocks_for(view.value_rows * L.Dv, 256)), dim3(256), 0, stream, value,
-                       value_bits, view.value_rows, L.Hv, L.Dv, nvw, L.T, L.N, L.varlen,
+    hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>,
+                       dim3(blocks_for(view.symbol_rows * dvp, 256)), dim3(256), 0, stream,
+                       grad_output, grad_rows, view.symbol_rows, L.H, L.Dv, dvp, L.T, L.N, L.varlen,
                        full_width, value_offset);
-  } else {
-    hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
-                       dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
-                       L.T, L.N, L.varlen, full_width, value_offset);
-  }
-  if (L.varlen) {
-    hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
-                       dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
-  } else {
-    hipLaunchKernelGGL(init_row_stats_kernel<false>, dim3(blocks_for(view.symbol_rows, 256)),
-                       dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
-  }
+    if (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) {
+      hipLaunchKernelGGL(pack_value_bits_ballot_kernel<DTYPE>,
+                         dim3(blocks_for(view.value_rows * L.Dv, 256)), dim3(256), 0, stream, value,
+                         value_bits, view.value_rows, L.Hv, L.Dv, nvw, L.T, L.N, L.varlen,
+                         full_width, value_offset);
+    } else {
+      hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
+                         dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
+                         L.T, L.N, L.varlen, full_width, value_offset);
+    }
+    if (L.varlen) {
+      hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
+                         dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
+    } else {
+      hipLaunchKernelGGL(init_row_stats_kernel<false>, dim3(blocks_for(view.symbol_rows, 256)),
+                         dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
+    }
 
-  stage_end(kStagePrepare, stream);
+    stage_end(kStagePrepare, stream);
 
-  VjpParams P;
-  memset(&P, 0, sizeof(P));
-  P.L = L;
-  P.packed_query = reinterpret_cast<const uint32_t*>(packed_query);
-  P.packed_key = reinterpret_cast<const uint32_t*>(packed_key);
-  P.value_bits = value_bits;
-  P.grad_rows = grad_rows;
-  P.stats = stats;
-  P.dropout_seed = dropout_seed;
-  P.scale = scale;
-  P.dropout_p = dropout_p;
-  P.inverse_keep = inverse_keep;
-  P.mismatch_scale = mismatch_scale;
-  P.gate_log2 = mismatch_scale * kLog2e / static_cast<float>(L.D);
-  P.logit_gain = scale * kSqrtScale * kLog2e;
-  P.null_logit = kNullScore * scale;
-  {
-    // window products this far below one cannot move a float32 gradient:
-    // 2^-34 / (W^2 * longest)
-    const int longest = L.varlen ? L.N : L.T;
-    const float exponent =
-        -34.0f - 2.0f * std::log2(static_cast<float>(L.W)) - std::log2(static_cast<float>(longest));
-    P.tail_threshold = std::exp2(std::max(exponent, -120.0f));
-  }
-  P.gradient_mask = gradient_mask;
-  P.dvp = dvp;
-  P.grad_query = grad_query;
-  P.grad_key = grad_key;
-  P.grad_value = grad_value;
-  P.work_counter = counter;
-  P.header = at<int32_t>(workspace, w.header);
-  P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
-  P.record_floats = w.record_floats;
-  P.value_stride = full_width;
-  P.value_offset = value_offset;
-  P.block_scratch = at<float>(workspace, w.block_scratch);
-  P.block_scratch_floats = w.block_scratch_floats;
-  P.ring_rows = w.ring_rows;
-  P.total_units = L.slots * L.H;
-  const bool dropout = dropout_p > 0.0f;
+    VjpParams P;
+    memset(&P, 0, sizeof(P));
+    P.L = L;
+    P.packed_query = reinterpret_cast<const uint32_t*>(packed_query);
+    P.packed_key = reinterpret_cast<const uint32_t*>(packed_key);
+    P.value_bits = value_bits;
+    P.grad_rows = grad_rows;
+    P.stats = stats;
+    P.dropout_seed = dropout_seed;
+    P.scale = scale;
+    P.dropout_p = dropout_p;
+    P.inverse_keep = inverse_keep;
+    P.mismatch_scale = mismatch_scale;
+    P.gate_log2 = mismatch_scale * kLog2e / static_cast<float>(L.D);
+    P.logit_gain = scale * kSqrtScale * kLog2e;
+    P.null_logit = kNullScore * scale;
+    {
+      // window products this far below one cannot move a float32 gradient:
+      // 2^-34 / (W^2 * longest)
+      const int longest = L.varlen ? L.N : L.T;
+      const float exponent =
+          -34.0f - 2.0f * std::log2(static_cast<float>(L.W)) -
+          std::log2(static_cast<float>(longest));
+      P.tail_threshold = std::exp2(std::max(exponent, -120.0f));
+    }
+    P.gradient_mask = gradient_mask;
+    P.dvp = dvp;
+    P.grad_query = grad_query;
+    P.grad_key = grad_key;
+    P.grad_value = grad_value;
+    P.work_counter = counter;
+    P.header = at<int32_t>(workspace, w.header);
+    P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
+    P.record_floats = w.record_floats;
+    P.value_stride = full_width;
+    P.value_offset = value_offset;
+    P.block_scratch = at<float>(workspace, w.block_scratch);
+    P.block_scratch_floats = w.block_scratch_floats;
+    P.ring_rows = w.ring_rows;
+    P.total_units = L.slots * L.H;
+    const bool dropout = dropout_p > 0.0f;
 
-  int status = 0;
-  if (nvw == 1) {
-    if (dvp == 8) status = dispatch_vjp<1, 8>(P, w, analytic, dropout, stream);
-    else if (dvp == 16) status = dispatch_vjp<1, 16>(P, w, analytic, dropout, stream);
-    else status = dispatch_vjp<1, 32>(P, w, analytic, dropout, stream);
-  } else {
-    status = dispatch_vjp<2, 64>(P, w, analytic, dropout, stream);
-  }
-  if (status != 0) return status;
+    int status = 0;
+    if (nvw == 1) {
+      if (dvp == 8) status = dispatch_vjp<1, 8>(P, w, analytic, dropout, stream);
+      else if (dvp == 16) status = dispatch_vjp<1, 16>(P, w, analytic, dropout, stream);
+      else status = dispatch_vjp<1, 32>(P, w, analytic, dropout, stream);
+    } else {
+      status = dispatch_vjp<2, 64>(P, w, analytic, dropout, stream);
+    }
+    if (status != 0) return status;
   }  // value slices
   const int64_t finalize_items = std::max(symbol_elements, value_elements);
   stage_begin(kStageFinalize, stream);
