@@ -1124,10 +1124,68 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   for (int first = 0; first < view.steps; first += kBlockRows) {
     const int count = min(kBlockRows, view.steps - first);
     wave_lds_fence();
-    stage_rows<NVW, kRowStats>(view, first, kBlockRows, lane, rows, W);
-    if (needs_utility) {
-      stage_grad_rows<DVP>(view, first, kBlockRows, lane, grads, DVP);
-      stage_value_columns<NVW>(view, first, kBlockRows + kWave, lane, value_columns);
+    {
+      // every global load of the block is issued before the first of them is used
+      const bool row_lane = lane < kBlockRows;
+      const int i = min(first + lane, view.steps - 1);  // rows past the band's end repeat the last
+      const int t = view.diag0 + 1 + i;
+      uint4 symbols = make_uint4(0u, 0u, 0u, 0u);
+      float4 stat = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (row_lane) {
+        symbols.x = view.q[t];
+        symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+        symbols.z = view.k[i];
+        symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
+        stat = view.stats[t];
+      }
+      constexpr int kQuads = DVP / 4;
+      constexpr int kGradParts = (kBlockRows * kQuads + kWave - 1) / kWave;
+      constexpr int kValueParts = ((kBlockRows + kWave) * NVW + kWave - 1) / kWave;
+      float4 grad_in[kGradParts];
+      uint32_t value_in[kValueParts];
+      if (needs_utility) {
+#pragma unroll
+        for (int part = 0; part < kGradParts; ++part) {
+          const int index = part * kWave + lane;
+          const int r = index / kQuads;
+          grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (r < kBlockRows && first + r < view.steps) {
+            grad_in[part] = *reinterpret_cast<const float4*>(
+                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * DVP +
+                4 * (index - r * kQuads));
+          }
+        }
+#pragma unroll
+        for (int part = 0; part < kValueParts; ++part) {
+          const int index = part * kWave + lane;
+          const int column = index / NVW;
+          const int a = first - 63 + column;
+          value_in[part] = (column < kBlockRows + kWave && a >= 1 && a <= view.len - 1)
+              ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (row_lane) {
+        uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
+        row_words[0] = symbols;
+        row_words[1] = make_uint4(__float_as_uint(fmaf(stat.x, kLog2e, stat.w)), 0u, 0u, 0u);
+      }
+      if (needs_utility) {
+#pragma unroll
+        for (int part = 0; part < kGradParts; ++part) {
+          const int index = part * kWave + lane;
+          const int r = index / kQuads;
+          if (r < kBlockRows) {
+            *reinterpret_cast<float4*>(grads + r * DVP + 4 * (index - r * kQuads)) = grad_in[part];
+          }
+        }
+#pragma unroll
+        for (int part = 0; part < kValueParts; ++part) {
+          if (part * kWave + lane < (kBlockRows + kWave) * NVW) {
+            value_columns[part * kWave + lane] = value_in[part];
+          }
+        }
+      }
     }
     for (int local = 0; local < count; local += kChunk) {
       const int rows_here = min(kChunk, count - local);
