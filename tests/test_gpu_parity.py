@@ -145,6 +145,9 @@ VJP_CASES = [
     (1, 120, 1, 4, 1, 4, 8, 30.0, 0.2, 0.5, torch.float32, "periodic"),  # row-maximum pass
     (1, 90, 2, 4, 1, 70, 12, 1.0, 0.1, 3.0, torch.float32, "random"),    # two value slices
     (1, 70, 2, 3, 2, 130, 8, 1.0, 0.0, 3.0, torch.bfloat16, "shifted"),  # three value slices
+    # second symbol tile 4 bits wide, second value tile 8 wide: both flushed on all lanes
+    (1, 150, 2, 20, 1, 24, 20, 1.0, 0.1, 3.0, torch.float32, "random"),
+    (2, 97, 2, 24, 2, 20, 12, 1.0, 0.0, 3.0, torch.float32, "shifted"),
 ]
 
 
