@@ -882,12 +882,24 @@ __device__ __forceinline__ RowSymbols staged_symbols(const uint32_t* row) {
   return RowSymbols{words.x, words.y, words.z, words.w};
 }
 
+// exp2(-c n) of a mismatch count n without the int -> float conversion: 0x3f800000 + n is
+// the float 1 + n 2^-23, and fma(that, -c 2^23, c 2^23) is -c n with the single rounding
+// of the plain product.
+constexpr int kCountBias = 0x3f800000;
+
+__device__ __forceinline__ float decay_of_biased_count(int biased, float gate_log2) {
+  const float slope = gate_log2 * 8388608.0f;
+  return fast_exp2(fmaf(__int_as_float(biased), -slope, slope));
+}
+
 // One forward step of the evidence recurrence S = g (1 + S_prev) - overflow.
 // STEADY: every lane of the wave is past its diagonal's first W + 1 rows, so no
 // lane needs masking (true for all but the first W + 64 rows of a band).
 // QUIET (with STEADY): the caller knows that no overflow term of these rows can move
 // a float32 result; the window is not tracked and the overflow is taken as zero.
-template <int NVW, bool STEADY = false, bool QUIET = false>
+// BIASED: Band::window carries kCountBias on top of the count (the caller adds it when
+// the band starts and removes it where the count leaves the kernel).
+template <int NVW, bool STEADY = false, bool QUIET = false, bool BIASED = false>
 __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbols& symbols, int i,
                                                 int lane, int W, float gate_log2) {
   const int a0 = i + 1;
@@ -895,9 +907,16 @@ __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbol
   StepOut out;
   out.a = a0 - lane;
   const int mismatches = __popc(symbols.query ^ band.key_word);
+  const auto window_decay = [&]() {
+    return BIASED ? decay_of_biased_count(band.window, gate_log2)
+                  : fast_exp2(-gate_log2 * static_cast<float>(band.window));
+  };
+  const float gate = (BIASED || (STEADY && QUIET))
+      ? decay_of_biased_count(mismatches + kCountBias, gate_log2)
+      : fast_exp2(-gate_log2 * static_cast<float>(mismatches));
   if constexpr (STEADY && QUIET) {
     out.active = true;
-    out.gate = fast_exp2(-gate_log2 * static_cast<float>(mismatches));
+    out.gate = gate;
     out.overflow = 0.0f;
     band.evidence = fmaf(out.gate, band.evidence, out.gate);
     out.evidence = band.evidence;
@@ -907,16 +926,16 @@ __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbol
   if constexpr (STEADY) {
     out.active = true;
     band.window += mismatches - __popc(symbols.old_query ^ band.old_key_word);
-    out.gate = fast_exp2(-gate_log2 * static_cast<float>(mismatches));
-    out.overflow = fast_exp2(-gate_log2 * static_cast<float>(band.window));
+    out.gate = gate;
+    out.overflow = window_decay();
     band.evidence = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
   } else {
     out.active = out.a >= 1;
     const int leaving = (out.a >= W + 2) ? __popc(symbols.old_query ^ band.old_key_word) : 0;
-    band.window = out.active ? band.window + mismatches - leaving : 0;
-    out.gate = out.active ? fast_exp2(-gate_log2 * static_cast<float>(mismatches)) : 0.0f;
-    out.overflow =
-        (out.a >= W + 1) ? fast_exp2(-gate_log2 * static_cast<float>(band.window)) : 0.0f;
+    band.window =
+        out.active ? band.window + mismatches - leaving : (BIASED ? kCountBias : 0);
+    out.gate = out.active ? gate : 0.0f;
+    out.overflow = (out.a >= W + 1) ? window_decay() : 0.0f;
     const float next = fmaf(out.gate, band.evidence, out.gate) - out.overflow;
     band.evidence = out.active ? next : 0.0f;
   }
@@ -1114,7 +1133,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   }
   Band<NVW> band;
   band.evidence = 0.0f;
-  band.window = 0;
+  band.window = kCountBias;  // forward_step<..., BIASED>
   load_sliding<NVW>(band, view, 0, lane, W);
   const bool needs_utility = (P.gradient_mask & (ROSA_GRAD_QUERY | ROSA_GRAD_KEY)) != 0;
   uint32_t route_hash = route_hash_of(-lane);
@@ -1195,7 +1214,7 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
             view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
         slot[lane] = band.evidence;
       }
-      const int window_before = band.window;
+      const int window_before = band.window - kCountBias;
       float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
@@ -1223,7 +1242,8 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           }
           const int i = min(chunk_first + r, last_step);
           const int t = view.diag0 + 1 + i;
-          const StepOut s = forward_step<NVW, STEADY>(band, symbols, i, lane, W, P.gate_log2);
+          const StepOut s =
+              forward_step<NVW, STEADY, false, true>(band, symbols, i, lane, W, P.gate_log2);
           peak_overflow = fmaxf(peak_overflow, s.overflow);
           const float one_plus = 1.0f + s.evidence;
           const float root = one_plus * fast_rsq(one_plus);
@@ -1813,7 +1833,7 @@ void vjp_gradients_kernel(VjpParams P) {
             keep_adjoint[r] = live ? adjoint : 0.0f;
             keep_gate[r] = live ? s.gate : 0.0f;
             keep_overflow[r] = live ? s.overflow : 0.0f;
-            keep_evidence[r] = live ? s.evidence + s.overflow : 0.0f;
+            keep_evidence[r] = live ? (QUIET ? s.evidence : s.evidence + s.overflow) : 0.0f;
           }
         };
         const bool steady = first >= W + kWave && rows_here == kChunk;
