@@ -151,6 +151,21 @@ VJP_CASES = [
 ]
 
 
+def test_hard_forward_beyond_65535_rows_uses_the_64_bit_key(cabi, c_oracle):
+    # sequences of 65536 rows and more no longer fit (run, route) into 32 bits: the scan
+    # switches to a 64-bit key and the maximum; narrow symbols give long runs and many ties
+    T, W = 66000, 40
+    query = nonzero_randn((1, T, 1, 2), seed=1)
+    key = nonzero_randn((1, T, 1, 2), seed=2)
+    value = nonzero_randn((1, T, 1, 3), seed=3)
+    out, _, _, routes = cabi.hard_forward(*(t.to(DEVICE) for t in (query, key, value)), W)
+    torch.cuda.synchronize()
+    want_out, want_routes, _ = c_oracle.hard_forward(query, key, value, W)
+    assert int(want_routes.max()) > 65535
+    assert torch.equal(routes.cpu(), want_routes)
+    assert torch.equal(out.cpu(), want_out)
+
+
 @pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,scale,p,ms,dtype,pattern", VJP_CASES)
 def test_surrogate_vjp_matches_oracle(cabi, c_oracle, B, T, H, D, Hv, Dv, W, scale, p, ms, dtype,
                                       pattern):

@@ -206,3 +206,35 @@ def test_state_dict_round_trip_and_async_handle(rosa):
     torch.cuda.synchronize()
     assert torch.equal(ends.cpu(), want[1][:, 25:]) and torch.equal(output.cpu(), want[0][:, 25:])
     second.close()
+
+
+def test_history_beyond_65535_tokens_matches_the_dense_forward(rosa):
+    # past 65535 tokens of history the route scan switches from its 32-bit key to the 64-bit
+    # one; the expected routes come from the training forward's oracle on the same symbols
+    from oracle import c_oracle
+
+    tokens, bits, horizon = 66000, 2, 40
+    query = random_packed((1, tokens, 1), bits, 11)
+    key = random_packed((1, tokens, 1), bits, 12)
+    payload = random_packed((1, tokens, 1), bits, 13)
+
+    def signs(symbols):
+        planes = (symbols.unsqueeze(-1) >> torch.arange(bits, dtype=torch.uint8)) & 1
+        return planes.to(torch.float32) * 2.0 - 1.0  # [1, tokens, 1, bits]
+
+    _, routes, _ = c_oracle.hard_forward(signs(query), signs(key), signs(payload), horizon)
+    routes = routes.reshape(-1).to(torch.int64)
+    want_ends = torch.where(routes > 0, routes - 1, torch.full_like(routes, -1))
+    want_output = torch.where(routes > 0, payload.reshape(-1)[routes.clamp(min=0)].to(torch.int64),
+                              torch.zeros_like(routes))
+    with rosa.RosaRuntime(1, 1, bits, bits, horizon) as runtime:
+        pieces = []
+        for begin, end in ((0, 40000), (40000, 65999), (65999, tokens)):
+            got = runtime.update_packed(query[:, begin:end].to(DEVICE), key[:, begin:end].to(DEVICE),
+                                        payload[:, begin:end].to(DEVICE))
+            pieces.append((got[0].cpu().reshape(-1), got[1].cpu().reshape(-1)))
+    output = torch.cat([piece[0] for piece in pieces]).to(torch.int64)
+    ends = torch.cat([piece[1] for piece in pieces])
+    assert int(ends.max()) > 65535
+    assert torch.equal(ends, want_ends)
+    assert torch.equal(output, want_output)
