@@ -1,0 +1,98 @@
+"""Seeded random sweep of shapes and controls: device path against the C oracle.
+
+The hand-picked cases of test_gpu_parity.py name the code paths; this sweep crosses
+them (symbol and value widths on both sides of the 8/16/32/64 tile limits, lengths around
+the 16-row chunk and 64-row segment sizes, windows shorter and longer than the sequence,
+dropout, gradient masks, packed layouts with empty sequences, the three dtypes), with the
+same bars: routes and outputs bit-exact, gradients to rtol 1e-4.
+"""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from tests.conftest import nonzero_randn
+from tests.test_gpu_parity import assert_gradients_close, make_case, run_device
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from rosa_soft_amd import cabi as module
+
+    module.load()
+    return module
+
+
+def draw_case(rng, lengths):
+    value_heads = rng.choice([1, 2])
+    return dict(
+        D=rng.choice([1, 2, 3, 5, 8, 8, 8, 9, 16, 17, 24, 32]),
+        Dv=rng.choice([1, 4, 8, 8, 8, 9, 16, 17, 32, 33, 64, 65]),
+        Hv=value_heads,
+        H=value_heads * rng.choice([1, 2]),
+        T=rng.choice(lengths),
+        B=rng.choice([1, 2]),
+        W=rng.choice([1, 2, 7, 16, 33, 64, 128, 500]),
+        p=rng.choice([0.0, 0.0, 0.1, 0.5]),
+        scale=rng.choice([0.5, 1.0, 2.0]),
+        ms=rng.choice([1.0, 3.0, 9.0]),
+        dtype=rng.choice([torch.float32, torch.float32, torch.float16, torch.bfloat16]),
+        pattern=rng.choice(["random", "random", "shifted", "periodic", "all_match"]),
+        mask=rng.choice([7, 7, 7, 1, 2, 4, 3, 5, 6]),
+        packed=rng.random() < 0.3,
+    )
+
+
+def check_case(cabi, c_oracle, rng, index, c):
+    seed = rng.randrange(1, 2 ** 62) if c["p"] > 0 else None
+    controls = dict(max_suffix_length=c["W"], scale=c["scale"], dropout_p=c["p"],
+                    mismatch_scale=c["ms"], seed=seed)
+    if not c["packed"]:
+        q, k, v, go = make_case(c["B"], c["T"], c["H"], c["D"], c["Hv"], c["Dv"], c["dtype"],
+                                seed=index, pattern=c["pattern"])
+        out, _, _, routes, grads = run_device(cabi, q, k, v, go, c["W"], c["scale"], c["p"],
+                                              c["ms"], seed, c["mask"])
+        want_out, want_routes, _ = c_oracle.hard_forward(q, k, v, c["W"])
+        want = c_oracle.surrogate_vjp(q, k, v, go, **controls)
+        longest = c["T"]
+    else:
+        parts = [rng.choice([0, 1, 5, 63, 64, 65, 130, 200]) for _ in range(rng.choice([1, 3, 5]))]
+        if sum(parts) == 0:
+            parts.append(7)
+        offsets = [0, *np.cumsum(parts).tolist()]
+        total = offsets[-1]
+        q = nonzero_randn((total, c["H"], c["D"]), seed=index + 1).to(c["dtype"])
+        k = nonzero_randn((total, c["H"], c["D"]), seed=index + 2).to(c["dtype"])
+        if c["pattern"] != "random":
+            k = q.roll(2, dims=0).clone()
+        v = nonzero_randn((total, c["Hv"], c["Dv"]), seed=index + 3).to(c["dtype"])
+        go = nonzero_randn((total, c["H"], c["Dv"]), seed=index + 4, floor=0.0).to(c["dtype"])
+        out, _, _, routes, grads = run_device(cabi, q, k, v, go, c["W"], c["scale"], c["p"],
+                                              c["ms"], seed, c["mask"], offsets)
+        want_out, want_routes = c_oracle.varlen_hard_forward(q, k, v, offsets, c["W"])
+        want = c_oracle.varlen_surrogate_vjp(q, k, v, offsets, go, **controls)
+        longest = max(parts)
+    label = f"case {index}: {c}"
+    assert torch.equal(out.cpu().float(), want_out.float()), label
+    assert torch.equal(routes.cpu(), want_routes), label
+    # the same widening with the logit's magnitude as in test_surrogate_vjp_matches_oracle
+    slack = max(1.0, c["scale"] * max(longest, 8) / 40.0)
+    for bit, got, expected, name in zip((1, 2, 4), grads, want, "qkv"):
+        if c["mask"] & bit:
+            assert_gradients_close(got, expected, f"{label} d{name}", slack=slack)
+
+
+@pytest.mark.parametrize("seed,cases,lengths", [
+    (11, 120, [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 191, 200, 257, 320, 400]),
+    (12, 12, [511, 777, 1024, 1500, 2049]),
+])
+def test_random_shapes_and_controls_match_the_oracle(cabi, c_oracle, seed, cases, lengths):
+    rng = random.Random(seed)
+    for index in range(cases):
+        check_case(cabi, c_oracle, rng, index, draw_case(rng, lengths))
