@@ -238,3 +238,36 @@ def test_history_beyond_65535_tokens_matches_the_dense_forward(rosa):
     assert int(ends.max()) > 65535
     assert torch.equal(ends, want_ends)
     assert torch.equal(output, want_output)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_chunkings_match_the_dense_definition(rosa, seed):
+    # random symbol widths, horizons, head groupings and chunk boundaries: chunks of up to 8
+    # rows take the per-row kernel, longer ones the row-block scan
+    import random
+
+    rng = random.Random(seed)
+    for case in range(10):
+        batch = rng.choice([1, 2, 3])
+        payload_heads = rng.choice([1, 2])
+        heads = payload_heads * rng.choice([1, 2])
+        bits = rng.choice([1, 2, 3, 8])
+        payload_bits = rng.choice([1, 4, 8])
+        horizon = rng.choice([1, 2, 5, 17, 64, 200])
+        tokens = rng.choice([1, 9, 64, 65, 130, 300])
+        query = random_packed((batch, tokens, heads), bits, 100 * seed + 3 * case)
+        key = random_packed((batch, tokens, heads), bits, 100 * seed + 3 * case + 1)
+        payload = random_packed((batch, tokens, payload_heads), payload_bits, 100 * seed + 3 * case + 2)
+        want = expect_dense(query, key, payload, bits, payload_bits, horizon)
+        cuts = sorted({0, tokens, *(rng.randrange(0, tokens + 1) for _ in range(rng.choice([0, 2, 6])))})
+        outputs, positions = [], []
+        with rosa.RosaRuntime(heads, payload_heads, bits, payload_bits, horizon) as runtime:
+            for begin, end in zip(cuts[:-1], cuts[1:]):
+                output, ends = runtime.update_packed(
+                    query[:, begin:end].to(DEVICE), key[:, begin:end].to(DEVICE),
+                    payload[:, begin:end].to(DEVICE))
+                outputs.append(output)
+                positions.append(ends)
+        label = f"seed {seed} case {case}: cuts {cuts}"
+        assert torch.equal(torch.cat(outputs, dim=1).cpu(), want[0]), label
+        assert torch.equal(torch.cat(positions, dim=1).cpu(), want[1]), label
