@@ -98,30 +98,12 @@ __device__ __forceinline__ float dpp_row_shr8(float keep, float src) {
                                                     0x118, 0xf, 0xf, false));
 }
 
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add(float acc, float src) {
-  const int moved =
-      __builtin_amdgcn_update_dpp(0, __float_as_int(src), CTRL, ROW_MASK, 0xf, false);
-  return acc + __int_as_float(moved);
-}
-
-// Sum over the 64 lanes; the total is valid in lane 63 only.
 // The band kernels run one wavefront per block.  LDS instructions of one wave execute in
 // order, so data written by one lane is visible to another lane's later read without a
 // barrier; what is needed is that the compiler keeps the order, and nothing else: a full
 // __syncthreads() would also wait for every outstanding global store and atomic.
 __device__ __forceinline__ void wave_lds_fence() {
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-}
-
-__device__ __forceinline__ float wave_sum_lane63(float v) {
-  v = dpp_add<0x111, 0xf>(v, v);  // row_shr:1
-  v = dpp_add<0x112, 0xf>(v, v);  // row_shr:2
-  v = dpp_add<0x114, 0xf>(v, v);  // row_shr:4
-  v = dpp_add<0x118, 0xf>(v, v);  // row_shr:8
-  v = dpp_add<0x142, 0xa>(v, v);  // row_bcast:15 into rows 1 and 3
-  v = dpp_add<0x143, 0xc>(v, v);  // row_bcast:31 into rows 2 and 3
-  return v;
 }
 
 template <int CTRL, int ROW_MASK>
@@ -132,6 +114,7 @@ __device__ __forceinline__ float dpp_max(float acc, float src) {
   return fmaxf(acc, __int_as_float(moved));
 }
 
+// Maximum over the 64 lanes; the result is valid in lane 63 only.
 __device__ __forceinline__ float wave_max_lane63(float v) {
   v = dpp_max<0x111, 0xf>(v, v);
   v = dpp_max<0x112, 0xf>(v, v);
@@ -144,7 +127,6 @@ __device__ __forceinline__ float wave_max_lane63(float v) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
-__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 template <int DTYPE>
 __device__ __forceinline__ float load_as_float(const void* base, int64_t index) {
@@ -1739,8 +1721,8 @@ void vjp_gradients_kernel(VjpParams P) {
         band.key_word = key_window[local + 63 - lane];
         band.old_key_word = old_key_window[local + 63 - lane];
         const float* grad_tile = grad_rows_lds + local * GP;
-        const int a_first = first + 1;  // column of lane 0 in the chunk's first row
-        const uint32_t* key_tile = key_window + local;  // window column c <-> a = a_first - 64 + c
+        // window column c <-> a = first + 1 - 64 + c (first + 1 is lane 0's column in the first row)
+        const uint32_t* key_tile = key_window + local;
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
@@ -1850,7 +1832,7 @@ void vjp_gradients_kernel(VjpParams P) {
         }
         wave_lds_fence();
 
-        // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = a_first - 64 + c);
+        // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = first + 1 - 64 + c);
         // element (column c, row r) of the skewed matrix is tile[r][64 - c + r].
         if (want_v) {
           // narrow tiles: operands of every product are fetched one k step ahead, without
@@ -2036,7 +2018,7 @@ void vjp_gradients_kernel(VjpParams P) {
             }
           }
         }
-        // the last window tile (columns a_first .. a_first + 15) is complete: park it with
+        // the last window tile (columns first + 1 .. first + 16) is complete: park it with
         // the chunk's row sums, then shift the window up by one tile
 #pragma unroll
         for (int n = 0; n < VT; ++n) done_value[n] = value_acc[kWindowTiles - 1][n];
