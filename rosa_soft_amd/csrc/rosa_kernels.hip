@@ -2334,10 +2334,12 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   constexpr int SEG = gradient_segment(DVP);
   const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
                             SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave;
-  const hipError_t attribute = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(&vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
-      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_floats * sizeof(float)));
-  if (attribute != hipSuccess) return fail_hip(attribute, "gradient kernel LDS size");
+  // At most 20 KB of dynamic LDS per block: below the 64 KB every kernel may use without
+  // raising its limit first.  (Raising it would be a configuration call per launch, and
+  // those are refused while a stream is being captured into a graph.)
+  static_assert((2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP + SEG * kRowWords +
+                 (SEG + kWave) * (2 + NVW) + SEG + kWave) * sizeof(float) <= 64 * 1024,
+                "dynamic LDS of the gradient kernel");
   stage_begin(kStageGradients, stream);
   hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
                      dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave),

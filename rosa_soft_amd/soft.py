@@ -177,6 +177,23 @@ def _needs_backward(*tensors: Tensor) -> bool:
     return torch.is_grad_enabled() and any(tensor.requires_grad for tensor in tensors)
 
 
+def _refuse_training_capture(name: str) -> None:
+    """The no-grad forward can be recorded into a HIP graph; the training step cannot.
+
+    Recording forward + surrogate backward with ``torch.cuda.graph`` ended in a host
+    segmentation fault on this platform whose cause is not known, so the attempt is turned
+    into an error before anything is launched.
+    """
+
+    if torch.compiler.is_compiling():  # tracing: nothing is being launched
+        return
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            f"{name}: the surrogate backward cannot be recorded into a HIP graph in this "
+            "build; capture the forward under torch.no_grad() or run the training step eagerly"
+        )
+
+
 # ---------------------------------------------------------------------------
 # public operators
 # ---------------------------------------------------------------------------
@@ -204,6 +221,7 @@ def rosa_soft(
     _check_device_call("rosa_soft", query, horizon, scale, dropout_p, mismatch_scale)
     if not _needs_backward(query, key, value):
         return torch.ops.rosa_soft.hard_forward(query, key, value, horizon)[0]
+    _refuse_training_capture("rosa_soft")
     seed = make_dropout_seed(query, dropout_p, True)
     return _HardForwardSoftVjpFunction.apply(
         query, key, value, seed, horizon, float(scale), float(dropout_p), float(mismatch_scale)
@@ -233,6 +251,7 @@ def rosa_soft_varlen(
     _check_device_call("rosa_soft_varlen", query, horizon, scale, dropout_p, mismatch_scale)
     if not _needs_backward(query, key, value):
         return torch.ops.rosa_soft.hard_forward_varlen(query, key, value, cu_seqlens, horizon)[0]
+    _refuse_training_capture("rosa_soft_varlen")
     seed = make_dropout_seed(query, dropout_p, True)
     return _HardForwardSoftVjpVarlenFunction.apply(
         query, key, value, cu_seqlens, seed, horizon, float(scale), float(dropout_p),

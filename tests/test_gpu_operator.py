@@ -285,3 +285,40 @@ def test_autocast_gradscaler_and_checkpoint_replay(rosa):
     assert torch.equal(plain[0], replayed[0])
     torch.testing.assert_close(plain[1], replayed[1], rtol=1e-5, atol=1e-7)
     torch.testing.assert_close(plain[2], replayed[2], rtol=1e-5, atol=1e-7)
+
+
+def test_no_grad_forward_replays_from_a_hip_graph(rosa):
+    # every replay is checked against eager work done between the replays, on new inputs
+    # written in place
+    query, key, value, _ = device_inputs(T=300, seed=21)
+    q, k, v = (t.to(DEVICE) for t in (query, key, value))
+    generator = torch.Generator(device=DEVICE).manual_seed(5)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            rosa.rosa_soft(q, k, v, max_suffix_length=32)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = rosa.rosa_soft(q, k, v, max_suffix_length=32)
+        for _ in range(4):
+            q.copy_(torch.randn(q.shape, device=DEVICE, generator=generator))
+            want = rosa.rosa_soft(q, k, v, max_suffix_length=32).clone()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(captured, want)
+
+
+def test_recording_the_training_step_into_a_graph_is_refused(rosa):
+    query, key, value, _ = device_inputs(seed=22)
+    leaves = [t.to(DEVICE).requires_grad_() for t in (query, key, value)]
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be recorded into a HIP graph"):
+        with torch.cuda.graph(graph):
+            rosa.rosa_soft(*leaves, max_suffix_length=12)
+    # the stream is usable again afterwards
+    output = rosa.rosa_soft(*leaves, max_suffix_length=12)
+    assert output.shape == (2, 48, 4, 5)
