@@ -627,10 +627,10 @@ struct VjpParams {
 // grad_output -> float32 head-major rows padded to DVP.  One thread per float of the
 // destination: stores are contiguous, loads are runs of Dv elements.
 template <int DTYPE>
-__global__ __launch_bounds__(256) void prepare_grad_rows_kernel(
-    const void* __restrict__ grad_output, float* __restrict__ grad_rows, int64_t rows, int H,
-    int Dv, int dvp, int T, int N, int varlen, int value_stride, int value_offset) {
-  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void prepare_grad_rows(
+    int64_t index, const void* __restrict__ grad_output, float* __restrict__ grad_rows,
+    int64_t rows, int H, int Dv, int dvp, int T, int N, int varlen, int value_stride,
+    int value_offset) {
   if (index >= rows * dvp) return;
   const int64_t dst = index / dvp;  // head-major row
   const int d = static_cast<int>(index - dst * dvp);
@@ -658,12 +658,12 @@ __device__ __forceinline__ int64_t value_word_row(int64_t row, int Hv, int T, in
 
 // Value sign bits for widths 8, 16, 32 and 64: one lane per element in the order of the
 // tensor, one wave ballot per 64 elements; the lane at the start of a 32-bit group (or of
-// a narrower row) stores that group's word.
+// a narrower row) stores that group's word.  Every lane of the wave must call this.
 template <int DTYPE>
-__global__ __launch_bounds__(256) void pack_value_bits_ballot_kernel(
-    const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
-    int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
-  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void pack_value_bits_ballot(
+    int64_t index, const void* __restrict__ value, uint32_t* __restrict__ value_bits,
+    int64_t rows, int Hv, int Dv, int nvw, int T, int N, int varlen, int value_stride,
+    int value_offset) {
   const bool inside = index < rows * Dv;
   const int64_t row = index / Dv;
   const int d = static_cast<int>(index - row * Dv);
@@ -681,10 +681,9 @@ __global__ __launch_bounds__(256) void pack_value_bits_ballot_kernel(
 // value sign bits, head-major over value heads: word index (seq, hv, t) like the symbol words
 // (any width: one thread per row)
 template <int DTYPE>
-__global__ __launch_bounds__(256) void pack_value_bits_kernel(
-    const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows, int Hv,
-    int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void pack_value_bits_rows(
+    int64_t row, const void* __restrict__ value, uint32_t* __restrict__ value_bits, int64_t rows,
+    int Hv, int Dv, int nvw, int T, int N, int varlen, int value_stride, int value_offset) {
   if (row >= rows) return;  // row = token * Hv + hv
   const int64_t dst = value_word_row(row, Hv, T, N, varlen);
   for (int w = 0; w < nvw; ++w) {
@@ -704,10 +703,9 @@ __global__ __launch_bounds__(256) void pack_value_bits_kernel(
 // max(null, scale*U(min(W, t)) - log t) of every logit of the row, otherwise it
 // starts at the null logit and a separate pass raises it to the row maximum.
 template <bool VARLEN>
-__global__ __launch_bounds__(256) void init_row_stats_kernel(Layout L, float4* __restrict__ stats,
-                                                             float scale, int analytic,
-                                                             int32_t* __restrict__ work_counter) {
-  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void init_row_stats(int64_t index, const Layout& L,
+                                               float4* __restrict__ stats, float scale,
+                                               int analytic, int32_t* __restrict__ work_counter) {
   if (index == 0) *work_counter = 0;
   const int64_t rows = static_cast<int64_t>(L.N) * L.H;
   if (index >= rows) return;
@@ -735,6 +733,61 @@ __global__ __launch_bounds__(256) void init_row_stats_kernel(Layout L, float4* _
   }
   const float base = (scale * kSqrtScale + log_count) * kLog2e;
   stats[index] = make_float4(reference, 0.0f, 0.0f, base);
+}
+
+// Everything the two backward passes need before they start, as one launch: the four
+// parts are independent and own consecutive ranges of the grid.
+struct PrepareParams {
+  Layout L;
+  const void* grad_output;
+  const void* value;
+  float* grad_rows;
+  uint32_t* value_bits;
+  float4* stats;
+  int32_t* work_counter;
+  int64_t symbol_rows, value_rows;
+  int Dv, dvp, nvw, value_stride, value_offset;
+  float scale;
+  int analytic;
+  int ballot;  // value width is 8, 16, 32 or 64: pack signs with wave ballots
+  float* fill[3];  // gradient buffers to clear (null: none), with their lengths
+  int64_t fill_elements[3];
+  unsigned grad_blocks, value_blocks, stats_blocks, fill_blocks;
+};
+
+template <int DTYPE, bool VARLEN>
+__global__ __launch_bounds__(256) void vjp_prepare_kernel(PrepareParams p) {
+  unsigned block = blockIdx.x;
+  const auto element = [&]() { return static_cast<int64_t>(block) * blockDim.x + threadIdx.x; };
+  if (block < p.grad_blocks) {
+    prepare_grad_rows<DTYPE>(element(), p.grad_output, p.grad_rows, p.symbol_rows, p.L.H, p.Dv,
+                             p.dvp, p.L.T, p.L.N, p.L.varlen, p.value_stride, p.value_offset);
+    return;
+  }
+  block -= p.grad_blocks;
+  if (block < p.value_blocks) {
+    if (p.ballot) {
+      pack_value_bits_ballot<DTYPE>(element(), p.value, p.value_bits, p.value_rows, p.L.Hv, p.Dv,
+                                    p.nvw, p.L.T, p.L.N, p.L.varlen, p.value_stride,
+                                    p.value_offset);
+    } else {
+      pack_value_bits_rows<DTYPE>(element(), p.value, p.value_bits, p.value_rows, p.L.Hv, p.Dv,
+                                  p.nvw, p.L.T, p.L.N, p.L.varlen, p.value_stride,
+                                  p.value_offset);
+    }
+    return;
+  }
+  block -= p.value_blocks;
+  if (block < p.stats_blocks) {
+    init_row_stats<VARLEN>(element(), p.L, p.stats, p.scale, p.analytic, p.work_counter);
+    return;
+  }
+  block -= p.stats_blocks;
+  const int64_t stride = static_cast<int64_t>(p.fill_blocks) * blockDim.x;
+  for (int part = 0; part < 3; ++part) {
+    if (p.fill[part] == nullptr) continue;
+    for (int64_t i = element(); i < p.fill_elements[part]; i += stride) p.fill[part][i] = 0.0f;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -2070,18 +2123,6 @@ __global__ __launch_bounds__(256) void finalize_gradients_kernel(
   }
 }
 
-__global__ __launch_bounds__(256) void zero_fill_kernel(float* __restrict__ a, int64_t na,
-                                                        float* __restrict__ b, int64_t nb,
-                                                        float* __restrict__ c, int64_t nc) {
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-       i < na || i < nb || i < nc; i += stride) {
-    if (a != nullptr && i < na) a[i] = 0.0f;
-    if (b != nullptr && i < nb) b[i] = 0.0f;
-    if (c != nullptr && i < nc) c[i] = 0.0f;
-  }
-}
-
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -2392,13 +2433,6 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   const int64_t symbol_elements = view.symbol_rows * L.D;
   const int64_t value_elements = view.value_rows * full_width;
   stage_begin(kStagePrepare, stream);
-  {
-    const int64_t largest = std::max(symbol_elements, value_elements);
-    const unsigned fill_blocks = static_cast<unsigned>(std::min<int64_t>(blocks_for(largest, 256), 8192));
-    hipLaunchKernelGGL(zero_fill_kernel, dim3(fill_blocks), dim3(256), 0, stream, grad_query,
-                       grad_query ? symbol_elements : 0, grad_key, grad_key ? symbol_elements : 0,
-                       grad_value, grad_value ? value_elements : 0);
-  }
   for (int value_offset = 0; value_offset < full_width; value_offset += kValueSlice) {
     L.Dv = std::min(kValueSlice, full_width - value_offset);
     const int dvp = padded_value_width(L.Dv);
@@ -2411,26 +2445,51 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     int32_t* counter = at<int32_t>(workspace, w.header) + 1;
     const bool analytic = analytic_reference_is_safe(L, scale);
 
-    hipLaunchKernelGGL(prepare_grad_rows_kernel<DTYPE>,
-                       dim3(blocks_for(view.symbol_rows * dvp, 256)), dim3(256), 0, stream,
-                       grad_output, grad_rows, view.symbol_rows, L.H, L.Dv, dvp, L.T, L.N, L.varlen,
-                       full_width, value_offset);
-    if (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) {
-      hipLaunchKernelGGL(pack_value_bits_ballot_kernel<DTYPE>,
-                         dim3(blocks_for(view.value_rows * L.Dv, 256)), dim3(256), 0, stream, value,
-                         value_bits, view.value_rows, L.Hv, L.Dv, nvw, L.T, L.N, L.varlen,
-                         full_width, value_offset);
-    } else {
-      hipLaunchKernelGGL(pack_value_bits_kernel<DTYPE>, dim3(blocks_for(view.value_rows, 256)),
-                         dim3(256), 0, stream, value, value_bits, view.value_rows, L.Hv, L.Dv, nvw,
-                         L.T, L.N, L.varlen, full_width, value_offset);
-    }
-    if (L.varlen) {
-      hipLaunchKernelGGL(init_row_stats_kernel<true>, dim3(blocks_for(view.symbol_rows, 256)),
-                         dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
-    } else {
-      hipLaunchKernelGGL(init_row_stats_kernel<false>, dim3(blocks_for(view.symbol_rows, 256)),
-                         dim3(256), 0, stream, L, stats, scale, analytic ? 1 : 0, counter);
+    {
+      PrepareParams prepare;
+      memset(&prepare, 0, sizeof(prepare));
+      prepare.L = L;
+      prepare.grad_output = grad_output;
+      prepare.value = value;
+      prepare.grad_rows = grad_rows;
+      prepare.value_bits = value_bits;
+      prepare.stats = stats;
+      prepare.work_counter = counter;
+      prepare.symbol_rows = view.symbol_rows;
+      prepare.value_rows = view.value_rows;
+      prepare.Dv = L.Dv;
+      prepare.dvp = dvp;
+      prepare.nvw = nvw;
+      prepare.value_stride = full_width;
+      prepare.value_offset = value_offset;
+      prepare.scale = scale;
+      prepare.analytic = analytic ? 1 : 0;
+      prepare.ballot = (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) ? 1 : 0;
+      prepare.grad_blocks = blocks_for(view.symbol_rows * dvp, 256);
+      prepare.value_blocks =
+          blocks_for(prepare.ballot ? view.value_rows * L.Dv : view.value_rows, 256);
+      prepare.stats_blocks = blocks_for(view.symbol_rows, 256);
+      if (value_offset == 0) {  // the gradient buffers are cleared once, before the first slice
+        float* buffers[3] = {grad_query, grad_key, grad_value};
+        const int64_t lengths[3] = {symbol_elements, symbol_elements, value_elements};
+        int64_t largest = 0;
+        for (int part = 0; part < 3; ++part) {
+          prepare.fill[part] = buffers[part];
+          prepare.fill_elements[part] = buffers[part] != nullptr ? lengths[part] : 0;
+          largest = std::max(largest, prepare.fill_elements[part]);
+        }
+        prepare.fill_blocks =
+            static_cast<unsigned>(std::min<int64_t>(blocks_for(largest, 256), 8192));
+      }
+      const unsigned blocks = prepare.grad_blocks + prepare.value_blocks + prepare.stats_blocks +
+                              prepare.fill_blocks;
+      if (L.varlen) {
+        hipLaunchKernelGGL((vjp_prepare_kernel<DTYPE, true>), dim3(blocks), dim3(256), 0, stream,
+                           prepare);
+      } else {
+        hipLaunchKernelGGL((vjp_prepare_kernel<DTYPE, false>), dim3(blocks), dim3(256), 0, stream,
+                           prepare);
+      }
     }
 
     stage_end(kStagePrepare, stream);
