@@ -13,14 +13,22 @@ dropout_p=0.1, mismatch_scale=3.0).  One JSON line is printed.
 Besides whole-step tokens/s the line carries
 
 * ``fwd_tokens_per_s``: forward-only (no-grad) tokens/s;
-* ``roofline``: the dominant kernel (``vjp_gradients``) priced by its
-  algorithmic MFMA-equivalent flops ``2 * pairs * (3 D + 2 Dv)`` over its
-  average launch time, measured with HIP events recorded by the library on the
-  stream the kernel runs on, against the MI355X fp32 matrix peak;
+* ``roofline``: the dominant kernel (``vjp_gradients``) priced by the matrix flops it
+  performs, ``2 * pairs * (2 D + 2 Dv)`` (utilities, dV, dK, dQ), over its average launch
+  time, measured with HIP events recorded by the library on the stream the kernel runs on,
+  against the MI355X fp32 matrix peak; the same for the row-statistics kernel
+  (``2 * pairs * Dv``) and for the whole backward (``2 * pairs * (3 D + 2 Dv)`` over the sum
+  of its stages); ``traffic`` and ``issue`` are counter figures read from the rocprofv3
+  summaries under ``profiles/`` for this workload (absent where none was taken);
 * ``kernels``: average milliseconds and achieved HBM GB/s (algorithmic bytes)
   of every stage;
-* ``cpu_baseline``: the float64 CPU oracle timed on a bounded slice of the same
-  workload on this box's host cores, extrapolated to tokens/s.
+* ``configs`` (default workload only): ms per step, forward ms and the roofline fractions
+  of configurations 1 to 5, timed by the same run;
+* ``cpu_baseline``: the float64 C oracle timed on a bounded slice of the same workload on
+  this box's host cores and scaled by pair count, with ``pytorch`` (the pure-PyTorch
+  restatement of ``rosa_soft_reference``, forward + backward, configuration 1 at full
+  shape) and ``router`` (the reference's own CPU ``RosaRuntime`` built from its source,
+  forward only, the metric shape's 8-bit symbols) beside it.
 """
 
 from __future__ import annotations
@@ -28,6 +36,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -96,12 +105,6 @@ def pair_count(config) -> int:
     if "lengths" in config:
         return config["H"] * sum(n * (n - 1) // 2 for n in config["lengths"])
     return config["B"] * config["H"] * config["T"] * (config["T"] - 1) // 2
-
-
-# HBM bytes per launch of vjp_gradients_kernel, measured with `rocprofv3 --pmc FETCH_SIZE` and
-# `--pmc WRITE_SIZE` runs of this script (scaled by what the same counters read for
-# `--copy-calibration 1024`); only the metric workload has been measured.
-MEASURED_TRAFFIC_BYTES = {"metric": 2.89e9}
 
 
 def token_count(config) -> int:
@@ -189,9 +192,241 @@ def cpu_baseline(name: str, budget_seconds: float = 25.0) -> dict:
         sample=(
             f"float64 C oracle, fwd+bwd, 1 batch x {group} heads x first {rows} rows "
             f"({slice_pairs} pairs, {elapsed:.2f} s, forward {forward_seconds:.3f} s), "
-            "scaled by pair count"
+            f"extrapolated x{pair_count(config) / max(slice_pairs, 1):.1f} by pair count"
         ),
+        extrapolation_factor=pair_count(config) / max(slice_pairs, 1),
     )
+
+
+
+def measure_workload(name: str, steps: int, warmup: int) -> dict:
+    """Time `steps` training steps and as many no-grad forwards of one configuration."""
+
+    import rosa_soft_amd
+    from rosa_soft_amd import cabi
+
+    assert rosa_soft_amd.BUILD_CAPABILITIES.variant == "rocm", "HIP extension is not built"
+    device = torch.device("cuda:0")
+    config, query, key, value, cu_seqlens = make_workload(name, device)
+    leaves = [t.requires_grad_() for t in (query, key, value)]
+    cabi.stage_timing(True)
+    for _ in range(warmup):
+        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
+    torch.cuda.synchronize()
+    stage_totals = {}
+    begin = time.perf_counter()
+    for _ in range(steps):
+        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
+        # the events of this step were recorded on the stream; reading them
+        # waits for the step, which the closing synchronize would do anyway
+        for stage, ms in cabi.stage_times().items():
+            stage_totals[stage] = stage_totals.get(stage, 0.0) + ms
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    cabi.stage_timing(False)
+
+    def forward():
+        if cu_seqlens is None:
+            return rosa_soft_amd.rosa_soft(query, key, value, max_suffix_length=config["W"])
+        return rosa_soft_amd.rosa_soft_varlen(query, key, value, cu_seqlens,
+                                              max_suffix_length=config["W"])
+
+    with torch.no_grad():
+        for _ in range(2):
+            forward()
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(steps):
+            forward()
+        torch.cuda.synchronize()
+        forward_ms = 1e3 * (time.perf_counter() - begin) / steps
+    return dict(
+        name=name, config=config, steps=steps, warmup=warmup,
+        ms_per_step=1e3 * elapsed / steps, forward_ms=forward_ms,
+        stage_ms={stage: total / steps for stage, total in stage_totals.items()},
+    )
+
+
+def roofline_fractions(measured: dict) -> dict:
+    """Matrix flops each backward kernel performs over that kernel's own time.
+
+    Per (row, route) pair the backward contracts five times: the utilities go x sign(v)
+    (2 Dv flop; both backward kernels need them), dV (2 Dv), dK and dQ (2 D each) in the
+    gradient kernel, and q x k (2 D), which this build evaluates as xor + popcount on packed
+    words and therefore does not count for any kernel.  All fractions are against the
+    MI355X float32 matrix peak, whatever pipe executes the products.
+    """
+
+    config, stage_ms = measured["config"], measured["stage_ms"]
+    pairs = pair_count(config)
+    D, Dv = config["D"], config["Dv"]
+    flops = {
+        "vjp_gradients": 2.0 * pairs * (2 * D + 2 * Dv),
+        "vjp_row_stats": 2.0 * pairs * Dv,
+    }
+    out = {}
+    for stage, work in flops.items():
+        ms = stage_ms.get(stage)
+        if ms:
+            tflops = work / (ms * 1e-3) / 1e12
+            out[stage] = dict(ms=ms, flop=work, tflops=tflops, frac=tflops / FP32_MATRIX_PEAK_TFLOPS)
+    backward_ms = sum(ms for stage, ms in stage_ms.items() if stage.startswith("vjp_"))
+    if backward_ms > 0:
+        work = 2.0 * pairs * (3 * D + 2 * Dv)  # the per-pair figure of the five contractions
+        tflops = work / (backward_ms * 1e-3) / 1e12
+        out["whole_backward"] = dict(ms=backward_ms, flop=work, tflops=tflops,
+                                     frac=tflops / FP32_MATRIX_PEAK_TFLOPS)
+    return out
+
+
+def config_summary(measured: dict) -> dict:
+    config = measured["config"]
+    tokens = token_count(config)
+    fractions = roofline_fractions(measured)
+    return dict(
+        workload=", ".join(f"{k}={v}" for k, v in config.items()),
+        steps=measured["steps"],
+        ms_per_step=round(measured["ms_per_step"], 4),
+        fwd_ms=round(measured["forward_ms"], 4),
+        tokens_per_s=round(tokens / (measured["ms_per_step"] * 1e-3), 1),
+        fwd_tokens_per_s=round(tokens / (measured["forward_ms"] * 1e-3), 1),
+        vjp_gradients_ms=round(measured["stage_ms"].get("vjp_gradients", float("nan")), 4),
+        vjp_row_stats_ms=round(measured["stage_ms"].get("vjp_row_stats", float("nan")), 4),
+        vjp_gradients_frac=round(fractions.get("vjp_gradients", {}).get("frac", float("nan")), 4),
+        whole_backward_frac=round(fractions.get("whole_backward", {}).get("frac", float("nan")), 4),
+    )
+
+
+PROFILE_FIGURE = re.compile(r"^bench: (\w+) = ([-+0-9.eE]+)\s*$", re.MULTILINE)
+
+
+def profile_figures(workload: str) -> dict:
+    """Counter figures of a workload's dominant kernel, read from the committed summaries.
+
+    The rocprofv3 summaries under profiles/ end in lines `bench: name = value`; those are
+    what a counter run measured for this workload (HBM bytes per launch of the gradient
+    kernel, busy fractions of the VALU and matrix pipes, issued matrix instructions).
+    A workload without summaries yields an empty dict, never a guess.
+    """
+
+    figures = {}
+    for suffix in ("backward_hbm_traffic", "backward_issue_counters"):
+        path = os.path.join(ROOT, "profiles", f"{workload}_{suffix}.md")
+        if os.path.exists(path):
+            with open(path) as handle:
+                for name, value in PROFILE_FIGURE.findall(handle.read()):
+                    figures[name] = float(value)
+    return figures
+
+
+def training_record(args) -> dict:
+    measured = measure_workload(args.workload, args.steps, args.warmup)
+    config, stage_ms = measured["config"], measured["stage_ms"]
+    tokens = token_count(config)
+    pairs = pair_count(config)
+    ms_per_step, forward_ms = measured["ms_per_step"], measured["forward_ms"]
+    bytes_needed = algorithmic_bytes(config)
+    fractions = roofline_fractions(measured)
+    backward_ms = fractions.get("whole_backward", {}).get("ms", 0.0)
+    kernels = {stage: dict(ms=round(ms, 4)) for stage, ms in stage_ms.items()}
+    if "hard_forward" in stage_ms:
+        kernels["hard_forward"]["hbm_gbs"] = round(
+            bytes_needed["forward"] / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2
+        )
+        kernels["hard_forward"]["gpairs_per_s"] = round(pairs / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2)
+    if backward_ms > 0:
+        kernels["vjp_total"] = dict(
+            ms=round(backward_ms, 4),
+            hbm_gbs=round(bytes_needed["backward"] / (backward_ms * 1e-3) / 1e9, 2),
+            gpairs_per_s=round(pairs / (backward_ms * 1e-3) / 1e9, 2),
+        )
+    dominant = fractions.get("vjp_gradients", dict(tflops=float("nan"), frac=float("nan"), flop=0.0))
+    figures = profile_figures(args.workload)
+    roofline = {
+        "kernel": "vjp_gradients_kernel",
+        "bound": "mfma",
+        "achieved": dominant["tflops"],
+        "peak": FP32_MATRIX_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": dominant["frac"],
+        "traffic": figures.get("traffic_bytes_per_launch"),
+        "flop_per_launch": dominant["flop"],
+        "row_stats_kernel": fractions.get("vjp_row_stats"),
+        "whole_backward": fractions.get("whole_backward"),
+        "note": "achieved = the matrix flops this kernel performs per launch, "
+                "2*pairs*(2D+2Dv) (utilities, dV, dK, dQ; q.k is xor+popcount here), over its "
+                "mean launch time from HIP events on the launch stream; whole_backward = "
+                "2*pairs*(3D+2Dv) over the sum of the backward stages; traffic and issue are "
+                "read from the rocprofv3 summaries under profiles/ (null when this workload "
+                "has none)",
+    }
+    if figures:
+        roofline["issue"] = {k: v for k, v in figures.items() if k != "traffic_bytes_per_launch"}
+    return {
+        "metric": "fwd+bwd tokens/sec",
+        "value": tokens / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if config["dtype"] == "float32" else config["dtype"],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: " + ", ".join(f"{k}={v}" for k, v in config.items()),
+            "loss": "output.float().square().mean()",
+            "tokens_per_step": tokens,
+            "pairs_per_step": pairs,
+        },
+        "fwd_tokens_per_s": tokens / (forward_ms * 1e-3),
+        "fwd_ms": forward_ms,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+
+
+def pytorch_cpu_baseline(budget_seconds: float = 8.0) -> dict:
+    """The pure-PyTorch restatement of rosa_soft_reference (oracle/rosa_oracle.py), forward +
+    backward on configuration 1 at its full shape, on this box's host cores (the reference's
+    own CPU-runnable case: rosa_soft/soft_reference.py:596-635)."""
+
+    from oracle import rosa_oracle
+
+    config, query, key, value, _ = make_workload("config1")
+    leaves = [t.clone().requires_grad_() for t in (query, key, value)]
+    repeats, elapsed = 0, 0.0
+    while (elapsed < budget_seconds and repeats < 50) or repeats < 2:
+        for leaf in leaves:
+            leaf.grad = None
+        begin = time.perf_counter()
+        output = rosa_oracle.rosa_soft_oracle(
+            *leaves, max_suffix_length=config["W"], scale=1.0, dropout_p=config["p"],
+            mismatch_scale=config["ms"])
+        output.square().mean().backward()
+        if repeats > 0:  # the first pass warms the allocator and the thread pool
+            elapsed += time.perf_counter() - begin
+        repeats += 1
+    timed = repeats - 1
+    return dict(
+        value=timed * token_count(config) / elapsed, unit="tokens/s",
+        cores=torch.get_num_threads(), kind="port",
+        sample=(f"oracle/rosa_oracle.py (dense PyTorch restatement), fwd+bwd, config1 at full "
+                f"shape ({', '.join(f'{k}={v}' for k, v in config.items())}), {timed} repeats in "
+                f"{elapsed:.2f} s, torch threads {torch.get_num_threads()}"),
+    )
+
+
+def router_cpu_baseline() -> dict:
+    """The reference's RosaRuntime (its rosa_runtime.cpp built under oracle/_ref), forward only,
+    on the metric shape's 8-bit symbols: the CPU counterpart of the hard forward
+    (benchmarks/rosa_runtime.py:15-46)."""
+
+    config = RUNTIME_WORKLOADS["runtime_prefill"]
+    query, key, payload = runtime_symbols(config, config["T"], 7)
+    return runtime_cpu_baseline(config, query, key, payload)
 
 
 RUNTIME_WORKLOADS = {
@@ -305,6 +540,8 @@ def main() -> None:
     parser.add_argument("--workload", default="metric",
                         choices=sorted(WORKLOADS) + sorted(RUNTIME_WORKLOADS))
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-configs", action="store_true",
+                        help="skip the block that times configurations 1 to 5 beside the metric shape")
     parser.add_argument(
         "--copy-calibration", type=int, default=0, metavar="MIB",
         help="only run a plain device copy of MIB mebibytes three times (reference point for "
@@ -333,111 +570,18 @@ def main() -> None:
         run_runtime_workload(args)
         return
 
-    import rosa_soft_amd
-    from rosa_soft_amd import cabi
-
-    assert rosa_soft_amd.BUILD_CAPABILITIES.variant == "rocm", "HIP extension is not built"
-    device = torch.device("cuda:0")
-    config, query, key, value, cu_seqlens = make_workload(args.workload, device)
-    leaves = [t.requires_grad_() for t in (query, key, value)]
-    tokens = token_count(config)
-
-    cabi.stage_timing(True)
-    for _ in range(args.warmup):
-        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
-    torch.cuda.synchronize()
-    stage_totals = {}
-    begin = time.perf_counter()
-    for _ in range(args.steps):
-        run_step(rosa_soft_amd, config, leaves, cu_seqlens)
-        # the events of this step were recorded on the stream; reading them
-        # waits for the step, which the closing synchronize would do anyway
-        for stage, ms in cabi.stage_times().items():
-            stage_totals[stage] = stage_totals.get(stage, 0.0) + ms
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - begin
-    cabi.stage_timing(False)
-    ms_per_step = 1e3 * elapsed / args.steps
-
-    # forward only
-    with torch.no_grad():
-        for _ in range(2):
-            run_forward = (
-                rosa_soft_amd.rosa_soft(query, key, value, max_suffix_length=config["W"])
-                if cu_seqlens is None
-                else rosa_soft_amd.rosa_soft_varlen(query, key, value, cu_seqlens,
-                                                    max_suffix_length=config["W"])
-            )
-        torch.cuda.synchronize()
-        begin = time.perf_counter()
-        for _ in range(args.steps):
-            if cu_seqlens is None:
-                rosa_soft_amd.rosa_soft(query, key, value, max_suffix_length=config["W"])
-            else:
-                rosa_soft_amd.rosa_soft_varlen(query, key, value, cu_seqlens,
-                                               max_suffix_length=config["W"])
-        torch.cuda.synchronize()
-        forward_ms = 1e3 * (time.perf_counter() - begin) / args.steps
-
-    pairs = pair_count(config)
-    stage_ms = {stage: total / args.steps for stage, total in stage_totals.items()}
-    bytes_needed = algorithmic_bytes(config)
-    flops = 2.0 * pairs * (3 * config["D"] + 2 * config["Dv"])
-    gradient_ms = stage_ms.get("vjp_gradients", float("nan"))
-    achieved_tflops = flops / (gradient_ms * 1e-3) / 1e12
-    backward_ms = sum(ms for stage, ms in stage_ms.items() if stage.startswith("vjp_"))
-    kernels = {
-        stage: dict(ms=round(ms, 4)) for stage, ms in stage_ms.items()
-    }
-    if "hard_forward" in stage_ms:
-        kernels["hard_forward"]["hbm_gbs"] = round(
-            bytes_needed["forward"] / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2
-        )
-        kernels["hard_forward"]["gpairs_per_s"] = round(pairs / (stage_ms["hard_forward"] * 1e-3) / 1e9, 2)
-    if backward_ms > 0:
-        kernels["vjp_total"] = dict(
-            ms=round(backward_ms, 4),
-            hbm_gbs=round(bytes_needed["backward"] / (backward_ms * 1e-3) / 1e9, 2),
-            gpairs_per_s=round(pairs / (backward_ms * 1e-3) / 1e9, 2),
-        )
-
-    record = {
-        "metric": "fwd+bwd tokens/sec",
-        "value": tokens / (ms_per_step * 1e-3),
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32" if config["dtype"] == "float32" else config["dtype"],
-        "data": "synthetic",
-        "config": {
-            "workload": f"{args.workload}: " + ", ".join(f"{k}={v}" for k, v in config.items()),
-            "loss": "output.float().square().mean()",
-            "tokens_per_step": tokens,
-            "pairs_per_step": pairs,
-        },
-        "fwd_tokens_per_s": tokens / (forward_ms * 1e-3),
-        "fwd_ms": forward_ms,
-        "roofline": {
-            "kernel": "vjp_gradients_kernel",
-            "bound": "mfma",
-            "achieved": achieved_tflops,
-            "peak": FP32_MATRIX_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": achieved_tflops / FP32_MATRIX_PEAK_TFLOPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "note": "algorithmic flops 2*pairs*(3D+2Dv) over the kernel's mean launch time; "
-                    "traffic = HBM bytes per launch of this kernel from rocprofv3 FETCH_SIZE + "
-                    "WRITE_SIZE runs of this command, scaled by a 1 GiB device copy",
-        },
-        "kernels": kernels,
-    }
+    record = training_record(args)
+    if not args.no_configs and args.workload == "metric":
+        # the other configurations, timed by this same run (fewer steps each)
+        record["configs"] = {
+            name: config_summary(measure_workload(name, max(2, args.steps // 3), 2))
+            for name in ("config1", "config2", "config3", "config4", "config5")
+        }
     if not args.no_cpu_baseline:
         record["cpu_baseline"] = cpu_baseline(args.workload)
+        if args.workload == "metric":
+            record["cpu_baseline"]["pytorch"] = pytorch_cpu_baseline()
+            record["cpu_baseline"]["router"] = router_cpu_baseline()
     print(json.dumps(record))
 
 

@@ -105,6 +105,35 @@ int rosa_hip_hard_routes(const rosa_problem* problem, const void* query,
                          size_t workspace_bytes, void* stream);
 
 /*
+ * Hard forward whose result leaves as bits instead of ternary elements, for the step that
+ * follows the operator in its callers (the output projection of
+ * examples/fit_soft_reference.py:405-417 reads the output once and can expand it in its
+ * own prologue): `sign_words` uint32 [tokens][H][ceil(Dv/32)], bit d of word w set iff
+ * output[..., 32 w + d] == +1, and `routed` uint8 [tokens][H], 1 where a route was
+ * selected and 0 for the null route (whose words are zero): output = routed ? (bit ? +1
+ * : -1) : 0.  Invalid device cu_seqlens give routed = 0xff everywhere.  Same workspace as
+ * rosa_hip_hard_forward.  The reference has no such output; it replaces the element-wise
+ * tail of hard_forward_cuda (rosa_soft_kernels.cu:509-530) for such a consumer.
+ */
+int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query,
+                               const void* key, const void* value,
+                               uint32_t* sign_words, uint8_t* routed,
+                               int32_t* packed_query, int32_t* packed_key,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Sign symbols of a contiguous [rows][bits] tensor, in row order: bit i of a symbol is
+ * x[row, i] > 0 (so 0, -0, NaN and -inf give 0).  `symbol_bytes` = 1 writes uint8
+ * symbols (bits <= 8), the input format of rosa_hip_router_update; 4 writes uint32 words
+ * (bits <= 32).  Replaces pack_sign_bits of the reference's runtime front end
+ * (rosa_soft/runtime.py:130-146) and, for a caller that fuses the packing into its
+ * projection epilogue, stands for pack_sign_bits_pair_kernel
+ * (rosa_soft_kernels.cu:202-241) without the head-major transposition.
+ */
+int rosa_hip_pack_symbols(int dtype, const void* logits, int64_t rows, int bits,
+                          void* symbols, int symbol_bytes, void* stream);
+
+/*
  * Dense surrogate VJP.  Replaces surrogate_vjp_cuda (rosa_soft_kernels.cu:1923-2379)
  * and surrogate_vjp_varlen_cuda (:2382-2638).  Gradients are float32 in the
  * layout of the corresponding input and are fully overwritten; pass NULL for
@@ -160,12 +189,14 @@ typedef struct rosa_router_update {
 int rosa_hip_router_update(const rosa_router_update* update, void* stream);
 
 /*
- * Asynchronous device-side diagnostics.  Invalid cu_seqlens values (not
- * starting at 0, decreasing, or not ending at N) cannot be seen by the host
- * without a synchronisation, so the kernels clamp them to a safe range, and
- * record the fact in the first int32 of the workspace.  This call copies that
- * word back (it synchronises `stream`) and returns it: 0 = offsets were valid.
- * The reference aborts the process instead (rosa_soft_kernels.cu:287-308).
+ * Invalid device cu_seqlens values (not starting at 0, decreasing, or not ending
+ * at N) cannot be seen by the host without a synchronisation.  The reference
+ * aborts the process with a device assert (rosa_soft_kernels.cu:287-308); here no
+ * kernel touches a token in that case (every sequence is treated as empty) and the
+ * results carry the signal: every element of `output` and of every requested
+ * gradient is NaN.  The fact is also recorded in the first int32 of the workspace;
+ * this call copies that word back (it synchronises `stream`) and returns it:
+ * 0 = offsets were valid.
  */
 int rosa_hip_read_offset_error(const void* workspace, void* stream);
 

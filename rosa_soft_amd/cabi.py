@@ -30,6 +30,8 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_set_record_budget",
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
+    "rosa_hip_hard_forward_bits",
+    "rosa_hip_pack_symbols",
     "rosa_hip_surrogate_vjp",
     "rosa_hip_router_update",
     "rosa_hip_read_offset_error",
@@ -120,6 +122,14 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_hard_routes.restype = ctypes.c_int
     library.rosa_hip_hard_routes.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_hard_forward_bits.restype = ctypes.c_int
+    library.rosa_hip_hard_forward_bits.argtypes = [
+        problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_pack_symbols.restype = ctypes.c_int
+    library.rosa_hip_pack_symbols.argtypes = [
+        ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int, vp, ctypes.c_int, vp,
     ]
     library.rosa_hip_router_update.restype = ctypes.c_int
     library.rosa_hip_router_update.argtypes = [ctypes.POINTER(RosaRouterUpdate), vp]
@@ -221,6 +231,85 @@ def hard_forward(
     return output, packed_q, packed_k, routes
 
 
+def hard_forward_bits(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    max_suffix_length: int,
+    cu_seqlens: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """Hard forward whose output leaves as bits: ``(sign_words, routed)``.
+
+    ``sign_words`` is int32 ``[..., H, ceil(Dv/32)]`` (bit ``d`` of word ``w`` set iff output
+    element ``32 w + d`` is +1) and ``routed`` uint8 ``[..., H]`` (1 where a route was
+    selected); the leading axes are those of the inputs.  ``expand_output_bits`` turns them
+    back into the ternary output.
+    """
+
+    library = load()
+    assert query.is_cuda and query.is_contiguous() and key.is_contiguous() and value.is_contiguous()
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    words = (problem.Dv + 31) // 32
+    if cu_seqlens is None:
+        word_shape = (problem.B, problem.H, problem.T)
+        lead = (problem.B, problem.T, problem.H)
+    else:
+        word_shape = (problem.H, problem.N)
+        lead = (problem.N, problem.H)
+    with torch.cuda.device(query.device):
+        sign_words = torch.empty((*lead, words), dtype=torch.int32, device=query.device)
+        routed = torch.empty(lead, dtype=torch.uint8, device=query.device)
+        packed_q = torch.empty(word_shape, dtype=torch.int32, device=query.device)
+        packed_k = torch.empty(word_shape, dtype=torch.int32, device=query.device)
+        size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
+        workspace = torch.empty(max(size, 256), dtype=torch.uint8, device=query.device)
+        status = library.rosa_hip_hard_forward_bits(
+            ctypes.byref(problem), _ptr(query), _ptr(key), _ptr(value), _ptr(sign_words),
+            _ptr(routed), _ptr(packed_q), _ptr(packed_k), _ptr(workspace), workspace.numel(),
+            _stream(query),
+        )
+    _check(status, "rosa_hip_hard_forward_bits")
+    return sign_words, routed
+
+
+def expand_output_bits(sign_words: Tensor, routed: Tensor, value_dim: int,
+                       dtype: torch.dtype = torch.float32) -> Tensor:
+    """Ternary output from the bit form of ``hard_forward_bits`` (what a consumer's prologue does)."""
+
+    shifts = torch.arange(32, device=sign_words.device, dtype=torch.int32)
+    bits = (sign_words.unsqueeze(-1) >> shifts) & 1          # [..., words, 32]
+    bits = bits.reshape(*sign_words.shape[:-1], -1)[..., :value_dim]
+    signs = bits.to(dtype) * 2 - 1
+    return signs * (routed == 1).unsqueeze(-1).to(dtype)
+
+
+def pack_symbols(logits: Tensor, symbol_dtype: torch.dtype = torch.uint8) -> Tensor:
+    """Sign symbols of the last axis of a device tensor: bit ``i`` = ``logits[..., i] > 0``.
+
+    ``symbol_dtype`` is ``torch.uint8`` (widths up to 8, the streaming router's symbols) or
+    ``torch.int32`` (widths up to 32).  One launch; the result has the shape of ``logits``
+    without its last axis.
+    """
+
+    library = load()
+    if logits.dtype not in _DTYPE_CODES:
+        raise ValueError("pack_symbols supports float32, float16, and bfloat16")
+    if symbol_dtype not in (torch.uint8, torch.int32):
+        raise ValueError("symbols are stored as uint8 or int32")
+    assert logits.is_cuda
+    logits = logits.contiguous()
+    bits = logits.size(-1)
+    rows = logits.numel() // max(bits, 1)
+    with torch.cuda.device(logits.device):
+        symbols = torch.empty(logits.shape[:-1], dtype=symbol_dtype, device=logits.device)
+        status = library.rosa_hip_pack_symbols(
+            _DTYPE_CODES[logits.dtype], _ptr(logits), rows, bits, _ptr(symbols),
+            1 if symbol_dtype == torch.uint8 else 4, _stream(logits),
+        )
+    _check(status, "rosa_hip_pack_symbols")
+    return symbols
+
+
 def hard_routes(
     query: Tensor,
     key: Tensor,
@@ -311,9 +400,9 @@ def surrogate_vjp(
 
 
 def vjp_workspace_bytes(query: Tensor, value: Tensor, max_suffix_length: int,
-                        cu_seqlens: Optional[Tensor] = None) -> int:
+                        cu_seqlens: Optional[Tensor] = None, dropout: bool = False) -> int:
     problem = make_problem(query, value, max_suffix_length, cu_seqlens)
-    return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0))
+    return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, int(dropout)))
 
 
 def router_update(update: RosaRouterUpdate, device: torch.device) -> None:

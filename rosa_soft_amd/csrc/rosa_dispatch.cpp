@@ -18,6 +18,7 @@
 #include <torch/extension.h>
 
 #include <Python.h>
+#include <hip/hip_runtime_api.h>
 
 #include <algorithm>
 #include <cmath>
@@ -263,6 +264,19 @@ Triple vjp_common(Tensor query, Tensor key, Tensor value, const Tensor* cu_seqle
                   Tensor grad_output, Tensor packed_query, Tensor packed_key, Tensor seed,
                   int64_t horizon, const Scalars& scalars, int64_t gradient_mask) {
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(query.device());
+  {
+    // Recording the surrogate backward into a HIP graph has crashed the host process on
+    // this platform (cause unknown), whichever way the backward is reached: refuse before
+    // anything is allocated or launched.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const hipError_t queried = hipStreamIsCapturing(
+        c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(), &capture);
+    TORCH_CHECK(queried == hipSuccess, "surrogate_vjp: hipStreamIsCapturing failed: ",
+                hipGetErrorString(queried));
+    TORCH_CHECK(capture == hipStreamCaptureStatusNone,
+                "surrogate_vjp: the surrogate backward cannot be recorded into a HIP graph in "
+                "this build; run the backward eagerly");
+  }
   query = query.contiguous();
   key = key.contiguous();
   value = value.contiguous();

@@ -154,6 +154,17 @@ __device__ __forceinline__ void store_sign(void* base, int64_t index, int sign) 
   }
 }
 
+template <int DTYPE>
+__device__ __forceinline__ void store_nan(void* base, int64_t index) {
+  if constexpr (DTYPE == ROSA_DTYPE_F32) {
+    static_cast<uint32_t*>(base)[index] = 0x7fc00000u;
+  } else if constexpr (DTYPE == ROSA_DTYPE_F16) {
+    static_cast<uint16_t*>(base)[index] = uint16_t(0x7e00);
+  } else {
+    static_cast<uint16_t*>(base)[index] = uint16_t(0x7fc0);
+  }
+}
+
 // The counter hash (reference rosa_soft_kernels.cu:549-586) is six rounds of
 //   h(x): x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16
 // chained as s = h(s ^ key).  fold16(x) = x ^ (x >> 16) is linear over xor and its own
@@ -308,32 +319,31 @@ __global__ void prepare_sequences_kernel(const int32_t* __restrict__ cu_seqlens,
                                          int64_t* __restrict__ step_prefix, int H,
                                          int64_t checkpoint_capacity,
                                          int32_t* __restrict__ header) {
-  // single block; offsets are clamped into [previous, N] so that no later
-  // kernel can index outside the tensors, and any violation is recorded.
+  // Single block.  Offsets are valid iff they start at 0, end at N and never decrease.
+  // When they are not, every sequence is made empty, so that no later kernel touches a
+  // token, and header[0] is set: the kernels that write results then fill them with NaN.
   __shared__ int bad;
   __shared__ int partial[256];
-  if (threadIdx.x == 0) bad = 0;
+  if (threadIdx.x == 0) bad = (cu_seqlens[0] != 0 || cu_seqlens[S] != N) ? 1 : 0;
   __syncthreads();
   const int per_thread = (S + blockDim.x - 1) / blockDim.x;
   const int first = threadIdx.x * per_thread;
   const int last = min(S, first + per_thread);
   int local_bad = 0;
-  int blocks = 0;
   for (int s = first; s < last; ++s) {
-    const int raw_begin = cu_seqlens[s];
-    const int raw_end = cu_seqlens[s + 1];
-    if (raw_begin > raw_end || raw_begin < 0 || raw_end > N) local_bad = 1;
-    const int begin = min(max(raw_begin, 0), N);
-    const int end = min(max(raw_end, begin), N);
-    seq_start[s] = begin;
-    seq_len[s] = end - begin;
-    blocks += (end - begin + 63) >> 6;
-  }
-  if (threadIdx.x == 0) {
-    if (cu_seqlens[0] != 0) local_bad = 1;
-    if (cu_seqlens[S] != N) local_bad = 1;
+    if (cu_seqlens[s] > cu_seqlens[s + 1]) local_bad = 1;
   }
   if (local_bad) atomicOr(&bad, 1);
+  __syncthreads();
+  const bool valid = bad == 0;
+  int blocks = 0;
+  for (int s = first; s < last; ++s) {
+    const int begin = valid ? cu_seqlens[s] : 0;
+    const int length = valid ? cu_seqlens[s + 1] - begin : 0;
+    seq_start[s] = begin;
+    seq_len[s] = length;
+    blocks += (length + 63) >> 6;
+  }
   partial[threadIdx.x] = blocks;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -560,14 +570,21 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
   source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
 }
 
-// output[token, h, :] = sign(value[source, h / group, :]) or exact zero
+// output[token, h, :] = sign(value[source, h / group, :]) or exact zero.  `offset_error`
+// (packed layout only, else NULL) points at the flag of invalid cu_seqlens: when it is set
+// no row was routed and every output element becomes NaN, so that the mistake cannot pass
+// for a result.
 template <int DTYPE>
 __global__ __launch_bounds__(256) void gather_values_kernel(
     const int32_t* __restrict__ source_token, const void* __restrict__ value,
     void* __restrict__ output, int64_t elements, int H, int Hv, int Dv, int T, int N,
-    int varlen) {
+    int varlen, const int32_t* __restrict__ offset_error) {
   const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (index >= elements) return;
+  if (offset_error != nullptr && *offset_error != 0) {
+    store_nan<DTYPE>(output, index);
+    return;
+  }
   const int d = static_cast<int>(index % Dv);
   const int64_t row = index / Dv;
   const int h = static_cast<int>(row % H);
@@ -588,6 +605,83 @@ __global__ __launch_bounds__(256) void gather_values_kernel(
     sign = x > 0.0f ? 1 : -1;
   }
   store_sign<DTYPE>(output, index, sign);
+}
+
+// The same output as sign and validity bits, for a consumer that expands the ternary
+// values itself (the prologue of the projection that follows the operator): per
+// (token, head) ceil(Dv / 32) words whose bit d is value[source, hv, d] > 0, zero for the
+// null route, and one byte that is 1 when a route was selected.  One thread per word.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void gather_value_bits_kernel(
+    const int32_t* __restrict__ source_token, const void* __restrict__ value,
+    uint32_t* __restrict__ sign_words, uint8_t* __restrict__ routed, int64_t words, int H,
+    int Hv, int Dv, int nvw, int T, int N, int varlen,
+    const int32_t* __restrict__ offset_error) {
+  const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= words) return;
+  const int w = static_cast<int>(index % nvw);
+  const int64_t row = index / nvw;  // token * H + h
+  const int h = static_cast<int>(row % H);
+  const int64_t token = row / H;
+  if (offset_error != nullptr && *offset_error != 0) {
+    // invalid cu_seqlens: bits cannot carry NaN; validity 0xff is the marker
+    sign_words[index] = 0u;
+    if (w == 0) routed[row] = uint8_t(0xff);
+    return;
+  }
+  int64_t word_index;
+  if (varlen) {
+    word_index = static_cast<int64_t>(h) * N + token;
+  } else {
+    const int64_t b = token / T;
+    word_index = (b * H + h) * T + (token - b * T);
+  }
+  const int source = source_token[word_index];
+  uint32_t bits = 0u;
+  if (source >= 0) {
+    const int hv = h / (H / Hv);
+    const int64_t base = (static_cast<int64_t>(source) * Hv + hv) * Dv + 32 * w;
+    const int count = min(32, Dv - 32 * w);
+    for (int d = 0; d < count; ++d) {
+      if (load_as_float<DTYPE>(value, base + d) > 0.0f) bits |= 1u << d;
+    }
+  }
+  sign_words[index] = bits;
+  if (w == 0) routed[row] = source >= 0 ? uint8_t(1) : uint8_t(0);
+}
+
+// Sign symbols of a contiguous [rows][bits] tensor in the order of its rows: bit i of the
+// symbol is x[row, i] > 0.  OUT is uint8_t (bits <= 8, the streaming router's symbols) or
+// uint32_t.  Widths that divide 64 take one lane per element and one ballot per 64
+// elements; other widths take one lane per row.
+template <int DTYPE, typename OUT>
+__global__ __launch_bounds__(256) void pack_rows_ballot_kernel(const void* __restrict__ logits,
+                                                               OUT* __restrict__ symbols,
+                                                               int64_t elements, int bits) {
+  const int64_t element = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool positive = element < elements && load_as_float<DTYPE>(logits, element) > 0.0f;
+  const uint64_t mask = __ballot(positive);
+  const int lane = threadIdx.x & 63;
+  if (lane < 64 / bits) {
+    const int64_t row = (element - lane) / bits + lane;
+    if (row * bits < elements) {
+      const uint32_t field = bits == 32 ? 0xffffffffu : ((1u << bits) - 1u);
+      symbols[row] = static_cast<OUT>(static_cast<uint32_t>(mask >> (lane * bits)) & field);
+    }
+  }
+}
+
+template <int DTYPE, typename OUT>
+__global__ __launch_bounds__(256) void pack_rows_serial_kernel(const void* __restrict__ logits,
+                                                               OUT* __restrict__ symbols,
+                                                               int64_t rows, int bits) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (row >= rows) return;
+  uint32_t symbol = 0u;
+  for (int bit = 0; bit < bits; ++bit) {
+    if (load_as_float<DTYPE>(logits, row * bits + bit) > 0.0f) symbol |= 1u << bit;
+  }
+  symbols[row] = static_cast<OUT>(symbol);
 }
 
 // ---------------------------------------------------------------------------
@@ -2105,8 +2199,18 @@ __global__ __launch_bounds__(256) void finalize_gradients_kernel(
     const void* __restrict__ query, const void* __restrict__ key,
     const void* __restrict__ value, float* __restrict__ grad_query,
     float* __restrict__ grad_key, float* __restrict__ grad_value, int64_t symbol_elements,
-    int64_t value_elements) {
+    int64_t value_elements, const int32_t* __restrict__ offset_error) {
   const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (offset_error != nullptr && *offset_error != 0) {
+    // invalid cu_seqlens (packed layout): nothing was accumulated; every gradient is NaN
+    const float nan = __uint_as_float(0x7fc00000u);
+    if (index < symbol_elements) {
+      if (grad_query != nullptr) grad_query[index] = nan;
+      if (grad_key != nullptr) grad_key[index] = nan;
+    }
+    if (index < value_elements && grad_value != nullptr) grad_value[index] = nan;
+    return;
+  }
   if (index < symbol_elements) {
     if (grad_query != nullptr) {
       const float den = 1.0f + fabsf(load_as_float<DTYPE>(query, index));
@@ -2302,7 +2406,7 @@ template <int DTYPE>
 int run_forward(const rosa_problem* p, const ProblemView& view, const void* query,
                 const void* key, const void* value, void* output, int32_t* packed_query,
                 int32_t* packed_key, int32_t* routes, int32_t* lengths, void* workspace,
-                hipStream_t stream) {
+                hipStream_t stream, uint32_t* sign_words = nullptr, uint8_t* routed = nullptr) {
   Layout L = view.L;
   const ForwardWorkspace w = carve_forward(view);
   stage_begin(kStageForward, stream);
@@ -2343,10 +2447,19 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
                          L, pq, pk, routes, lengths, source_token, shift);
     }
   }
-  const int64_t out_elements = view.symbol_rows * L.Dv;
-  hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)), dim3(256),
-                     0, stream, source_token, value, output, out_elements, L.H, L.Hv, L.Dv, L.T,
-                     L.N, L.varlen);
+  const int32_t* offset_error = L.varlen ? at<const int32_t>(workspace, w.header) : nullptr;
+  if (sign_words != nullptr) {  // the output as sign and validity bits
+    const int nvw = value_words(L.Dv);
+    const int64_t words = view.symbol_rows * nvw;
+    hipLaunchKernelGGL(gather_value_bits_kernel<DTYPE>, dim3(blocks_for(words, 256)), dim3(256),
+                       0, stream, source_token, value, sign_words, routed, words, L.H, L.Hv,
+                       L.Dv, nvw, L.T, L.N, L.varlen, offset_error);
+  } else {
+    const int64_t out_elements = view.symbol_rows * L.Dv;
+    hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)),
+                       dim3(256), 0, stream, source_token, value, output, out_elements, L.H,
+                       L.Hv, L.Dv, L.T, L.N, L.varlen, offset_error);
+  }
   stage_end(kStageForward, stream);
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "hard forward launch");
@@ -2550,7 +2663,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   stage_begin(kStageFinalize, stream);
   hipLaunchKernelGGL(finalize_gradients_kernel<DTYPE>, dim3(blocks_for(finalize_items, 256)),
                      dim3(256), 0, stream, query, key, value, grad_query, grad_key, grad_value,
-                     symbol_elements, value_elements);
+                     symbol_elements, value_elements,
+                     L.varlen ? at<const int32_t>(workspace, w.header) : nullptr);
   stage_end(kStageFinalize, stream);
   const hipError_t launch = hipGetLastError();
   if (launch != hipSuccess) return fail_hip(launch, "surrogate vjp launch");
@@ -2586,6 +2700,7 @@ struct RouterUpdate {
   uint8_t* output;               // [tokens][H]
   int64_t* matched_key_end;      // [tokens][H]
   int tokens;
+  int blocks_per_run;            // blocks of the routing grid that share one (slot, head)
 };
 
 __device__ __forceinline__ int router_chunk_begin(const RouterUpdate& U, int slot) {
@@ -2622,12 +2737,16 @@ __global__ __launch_bounds__(256) void router_append_kernel(RouterUpdate U) {
 // the routes exactly like hard_route_kernel; the first row block starts at the slot's old
 // length, so its predecessor row lies in the history.
 __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
-  const int slot = blockIdx.y / U.H;
-  const int head = blockIdx.y - slot * U.H;
+  // one-dimensional grid: (slot, head) run-major, so that slots * heads is not bounded by
+  // the 65535 blocks of the other grid dimensions
+  const int run = static_cast<int>(blockIdx.x / static_cast<unsigned>(U.blocks_per_run));
+  const int row_block = static_cast<int>(blockIdx.x - static_cast<unsigned>(run) * U.blocks_per_run);
+  const int slot = run / U.H;
+  const int head = run - slot * U.H;
   const int old_length = U.history_lengths[slot];
   const int chunk_begin = router_chunk_begin(U, slot);
   const int new_length = old_length + (router_chunk_begin(U, slot + 1) - chunk_begin);
-  const int t0 = old_length + static_cast<int>(blockIdx.x) * kWave;
+  const int t0 = old_length + row_block * kWave;
   if (t0 >= new_length) return;
   const int lane = threadIdx.x;
   const int64_t run_base = (static_cast<int64_t>(slot) * U.H + head) * U.capacity;
@@ -2656,12 +2775,13 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
 // routes of the row, each comparing its suffixes directly, and the wave keeps the maximum of
 // the packed key (length, route): longest first, latest on ties.
 __global__ __launch_bounds__(kWave) void router_decode_kernel(RouterUpdate U) {
-  const int slot = blockIdx.y / U.H;
-  const int head = blockIdx.y - slot * U.H;
+  const int run = static_cast<int>(blockIdx.x / static_cast<unsigned>(U.blocks_per_run));
+  const int row = static_cast<int>(blockIdx.x - static_cast<unsigned>(run) * U.blocks_per_run);
+  const int slot = run / U.H;
+  const int head = run - slot * U.H;
   const int old_length = U.history_lengths[slot];
   const int chunk_begin = router_chunk_begin(U, slot);
   const int rows = router_chunk_begin(U, slot + 1) - chunk_begin;
-  const int row = blockIdx.x;
   if (row >= rows) return;
   const int lane = threadIdx.x;
   const int t = old_length + row;
@@ -2697,6 +2817,58 @@ __global__ __launch_bounds__(256) void router_advance_kernel(RouterUpdate U) {
   U.history_lengths[slot] += router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot);
 }
 
+int forward_entry(const rosa_problem* problem, const void* query, const void* key,
+                  const void* value, void* output, int32_t* packed_query, int32_t* packed_key,
+                  int32_t* routes, int32_t* lengths, void* workspace, size_t workspace_bytes,
+                  void* stream, uint32_t* sign_words, uint8_t* routed) {
+  ProblemView view;
+  const int bad = check_problem(problem, &view);
+  if (bad != 0) return bad;
+  if (!query || !key || !value || !packed_query || !packed_key || !workspace)
+    return fail(2, "hard_forward: NULL tensor or workspace pointer");
+  if (workspace_bytes < carve_forward(view).total) return fail(3, "hard_forward: workspace too small");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (problem->dtype) {
+    case ROSA_DTYPE_F32:
+      return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
+                                         packed_key, routes, lengths, workspace, s, sign_words,
+                                         routed);
+    case ROSA_DTYPE_F16:
+      return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
+                                         packed_key, routes, lengths, workspace, s, sign_words,
+                                         routed);
+    default:
+      return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
+                                          packed_key, routes, lengths, workspace, s, sign_words,
+                                          routed);
+  }
+}
+
+template <int DTYPE>
+void launch_pack_rows(const void* logits, int64_t rows, int bits, void* symbols, int symbol_bytes,
+                      hipStream_t stream) {
+  const int64_t elements = rows * bits;
+  if (64 % bits == 0) {
+    const dim3 grid(blocks_for(elements, 256));
+    if (symbol_bytes == 1) {
+      hipLaunchKernelGGL((pack_rows_ballot_kernel<DTYPE, uint8_t>), grid, dim3(256), 0, stream,
+                         logits, static_cast<uint8_t*>(symbols), elements, bits);
+    } else {
+      hipLaunchKernelGGL((pack_rows_ballot_kernel<DTYPE, uint32_t>), grid, dim3(256), 0, stream,
+                         logits, static_cast<uint32_t*>(symbols), elements, bits);
+    }
+  } else {
+    const dim3 grid(blocks_for(rows, 256));
+    if (symbol_bytes == 1) {
+      hipLaunchKernelGGL((pack_rows_serial_kernel<DTYPE, uint8_t>), grid, dim3(256), 0, stream,
+                         logits, static_cast<uint8_t*>(symbols), rows, bits);
+    } else {
+      hipLaunchKernelGGL((pack_rows_serial_kernel<DTYPE, uint32_t>), grid, dim3(256), 0, stream,
+                         logits, static_cast<uint32_t*>(symbols), rows, bits);
+    }
+  }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -2730,24 +2902,44 @@ int rosa_hip_hard_routes(const rosa_problem* problem, const void* query, const v
                          const void* value, void* output, int32_t* packed_query,
                          int32_t* packed_key, int32_t* routes, int32_t* lengths,
                          void* workspace, size_t workspace_bytes, void* stream) {
-  ProblemView view;
-  const int bad = check_problem(problem, &view);
-  if (bad != 0) return bad;
-  if (!query || !key || !value || !output || !packed_query || !packed_key || !workspace)
-    return fail(2, "hard_forward: NULL tensor or workspace pointer");
-  if (workspace_bytes < carve_forward(view).total) return fail(3, "hard_forward: workspace too small");
+  if (!output) return fail(2, "hard_forward: NULL tensor or workspace pointer");
+  return forward_entry(problem, query, key, value, output, packed_query, packed_key, routes,
+                       lengths, workspace, workspace_bytes, stream, nullptr, nullptr);
+}
+
+int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query, const void* key,
+                               const void* value, uint32_t* sign_words, uint8_t* routed,
+                               int32_t* packed_query, int32_t* packed_key, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  if (!sign_words || !routed) return fail(2, "hard_forward_bits: NULL output pointer");
+  return forward_entry(problem, query, key, value, nullptr, packed_query, packed_key, nullptr,
+                       nullptr, workspace, workspace_bytes, stream, sign_words, routed);
+}
+
+int rosa_hip_pack_symbols(int dtype, const void* logits, int64_t rows, int bits, void* symbols,
+                          int symbol_bytes, void* stream) {
+  if (dtype < ROSA_DTYPE_F32 || dtype > ROSA_DTYPE_BF16) return fail(1, "unsupported dtype");
+  if (rows < 0) return fail(1, "pack_symbols: negative row count");
+  if (symbol_bytes != 1 && symbol_bytes != 4)
+    return fail(1, "pack_symbols: symbols are stored as 1 or 4 bytes");
+  if (bits < 1 || bits > 8 * symbol_bytes)
+    return fail(1, "pack_symbols: symbol width must be in [1, 8] for bytes and [1, 32] for words");
+  if (rows == 0) return 0;
+  if (!logits || !symbols) return fail(2, "pack_symbols: NULL pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (problem->dtype) {
+  switch (dtype) {
     case ROSA_DTYPE_F32:
-      return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
-                                         packed_key, routes, lengths, workspace, s);
+      launch_pack_rows<ROSA_DTYPE_F32>(logits, rows, bits, symbols, symbol_bytes, s);
+      break;
     case ROSA_DTYPE_F16:
-      return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
-                                         packed_key, routes, lengths, workspace, s);
+      launch_pack_rows<ROSA_DTYPE_F16>(logits, rows, bits, symbols, symbol_bytes, s);
+      break;
     default:
-      return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
-                                          packed_key, routes, lengths, workspace, s);
+      launch_pack_rows<ROSA_DTYPE_BF16>(logits, rows, bits, symbols, symbol_bytes, s);
   }
+  const hipError_t launch = hipGetLastError();
+  if (launch != hipSuccess) return fail_hip(launch, "pack_symbols launch");
+  return 0;
 }
 
 int rosa_hip_hard_forward(const rosa_problem* problem, const void* query, const void* key,
@@ -2821,8 +3013,6 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   if (!u.history_lengths || !u.query_history || !u.key_history ||
       !u.payload_history || !u.query || !u.key || !u.payload || !u.output || !u.matched_key_end)
     return fail(2, "router: NULL pointer");
-  if (static_cast<int64_t>(u.S) * u.H > 65535)
-    return fail(1, "router: slots * heads must not exceed 65535");
   RouterUpdate U;
   U.S = u.S; U.H = u.H; U.Hp = u.Hp; U.W = u.W;
   U.capacity = u.capacity;
@@ -2838,16 +3028,23 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   U.output = u.output;
   U.matched_key_end = u.matched_key_end;
   U.tokens = u.tokens;
+  U.blocks_per_run = 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t symbols = static_cast<int64_t>(u.tokens) * u.H;
   hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
-  const unsigned runs = static_cast<unsigned>(u.S * u.H);
-  if (u.longest_chunk > 0 && u.longest_chunk <= kRouterDecodeRows) {
-    hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(u.longest_chunk), runs),
-                       dim3(kWave), 0, s, U);
-  } else if (u.longest_chunk > 0) {
-    const unsigned row_blocks = static_cast<unsigned>((u.longest_chunk + kWave - 1) / kWave);
-    hipLaunchKernelGGL(router_route_kernel, dim3(row_blocks, runs), dim3(kWave), 0, s, U);
+  const int64_t runs = static_cast<int64_t>(u.S) * u.H;
+  if (u.longest_chunk > 0) {
+    const bool decode = u.longest_chunk <= kRouterDecodeRows;
+    U.blocks_per_run = decode ? u.longest_chunk : (u.longest_chunk + kWave - 1) / kWave;
+    const int64_t blocks = runs * U.blocks_per_run;
+    if (blocks > INT32_MAX) return fail(1, "router: slots * heads * row blocks must fit in int32");
+    if (decode) {
+      hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
+                         s, U);
+    } else {
+      hipLaunchKernelGGL(router_route_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
+                         s, U);
+    }
   }
   hipLaunchKernelGGL(router_advance_kernel, dim3(blocks_for(u.S, 256)), dim3(256), 0, s, U);
   const hipError_t status = hipGetLastError();

@@ -46,15 +46,22 @@ def _integer_parameter(name: str, value: int) -> int:
         raise TypeError(f"{name} must be an integer") from error
 
 
-def _pack_sign_bits(logits: Tensor) -> Tensor:
-    # bit i of the symbol = logits[..., i] > 0 (rosa_soft/runtime.py:130-146)
+def _pack_sign_bits(logits: Tensor, device: torch.device) -> Tensor:
+    """uint8 symbols on ``device``: bit i = logits[..., i] > 0 (rosa_soft/runtime.py:130-146).
+
+    One kernel of the library (``rosa_hip_pack_symbols``); host logits are moved to the
+    device first, so nothing is computed on the host.
+    """
+
     if not logits.is_floating_point():
         raise TypeError("unpacked RosaRuntime inputs must be floating-point")
     bits = logits.size(-1)
     if not 1 <= bits <= 8:
         raise ValueError(f"RosaRuntime supports 1..8 bits, got {bits}")
-    weights = 1 << torch.arange(bits, device=logits.device, dtype=torch.int16)
-    return ((logits > 0).to(torch.int16) * weights).sum(dim=-1).to(torch.uint8).contiguous()
+    logits = logits.to(device)
+    if logits.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        logits = logits.to(torch.float32)  # float64: the sign survives the narrowing
+    return cabi.pack_symbols(logits, torch.uint8)
 
 
 def _unpack_sign_bits(packed: Tensor, bits: int, dtype: torch.dtype) -> Tensor:
@@ -238,6 +245,7 @@ class RosaRuntime:
         self._query_history: Optional[Tensor] = None    # [S, H, capacity] uint8
         self._key_history: Optional[Tensor] = None      # [S, H, capacity] uint8
         self._payload_history: Optional[Tensor] = None  # [S, Hp, capacity] uint8
+        self._last_update = None            # event recorded after the latest update's launches
 
     def _require_open(self) -> None:
         if self._state != "OPEN":
@@ -336,17 +344,31 @@ class RosaRuntime:
         if query_logits.ndim != expected_rank or payload_logits.ndim != expected_rank:
             layout = "dense" if cu_seqlens is None else "varlen"
             raise ValueError(f"{layout} inputs have the wrong rank for RosaRuntime")
-        return self.update_packed(
-            _pack_sign_bits(query_logits), _pack_sign_bits(key_logits),
-            _pack_sign_bits(payload_logits), cu_seqlens=cu_seqlens, stream=stream,
+        if not (query_logits.device == key_logits.device == payload_logits.device):
+            raise ValueError("all inputs must be on the same device")
+        self._require_open()
+        # the symbols are packed on the router's device, results return to the caller's
+        return self._update_symbols(
+            _pack_sign_bits(query_logits, self._device), _pack_sign_bits(key_logits, self._device),
+            _pack_sign_bits(payload_logits, self._device), cu_seqlens, stream=stream,
             async_op=async_op, return_packed=return_packed, output_dtype=payload_logits.dtype,
-            sequence_ids=sequence_ids,
+            sequence_ids=sequence_ids, caller_device=payload_logits.device,
         )
 
     def update_packed(self, query_symbols: Tensor, key_symbols: Tensor, payload_symbols: Tensor,
                       cu_seqlens: Optional[Tensor] = None, *, stream=None,
                       async_op: bool = False, return_packed: bool = True,
                       output_dtype: torch.dtype = torch.float32, sequence_ids=None):
+        return self._update_symbols(
+            query_symbols, key_symbols, payload_symbols, cu_seqlens, stream=stream,
+            async_op=async_op, return_packed=return_packed, output_dtype=output_dtype,
+            sequence_ids=sequence_ids, caller_device=payload_symbols.device,
+        )
+
+    def _update_symbols(self, query_symbols: Tensor, key_symbols: Tensor, payload_symbols: Tensor,
+                        cu_seqlens: Optional[Tensor], *, stream, async_op: bool,
+                        return_packed: bool, output_dtype: torch.dtype, sequence_ids,
+                        caller_device: torch.device):
         query, key, payload, offsets, output_shape, dense = _flatten_packed(
             query_symbols, key_symbols, payload_symbols, cu_seqlens
         )
@@ -356,7 +378,6 @@ class RosaRuntime:
             raise ValueError("packed payload head count must equal num_payload_heads")
         slot_count = len(offsets) - 1
         normalized_ids = _normalize_sequence_ids(sequence_ids, slot_count)
-        caller_device = payload_symbols.device
         if stream is not None and caller_device.type != "cuda":
             raise ValueError("stream requires CUDA inputs")
         if stream is not None and stream.device != caller_device:
@@ -376,6 +397,12 @@ class RosaRuntime:
         if run_stream is not None:
             run_stream.wait_stream(torch.cuda.current_stream(self._device))
         with torch.cuda.stream(run_stream) if run_stream is not None else _NullContext():
+            # Updates are serialised whatever streams they are given (the reference's
+            # runtime does the same): this one starts after the previous one has finished
+            # with the histories, including a growth copy.
+            working_stream = torch.cuda.current_stream(self._device)
+            if self._last_update is not None:
+                working_stream.wait_event(self._last_update)
             output, ends = self._route(
                 query.to(self._device), key.to(self._device), payload.to(self._device), offsets
             )
@@ -388,6 +415,8 @@ class RosaRuntime:
                     ends.unsqueeze(-1) >= 0, unpacked,
                     torch.zeros((), dtype=output_dtype, device=self._device),
                 )
+            self._last_update = torch.cuda.Event()
+            self._last_update.record(working_stream)
             if caller_device != self._device:
                 output, ends = output.to(caller_device), ends.to(caller_device)
             if run_stream is not None:

@@ -123,10 +123,10 @@ def test_packed_config5_full_size(cabi, c_oracle):
     query, key, value, grad_output, cu = (t.cpu() for t in tensors)
     offsets = cu.tolist()
     group = config["H"] // config["Hv"]
-    value_head = 2
-    heads = slice(value_head * group, (value_head + 1) * group)
-    # sequences 0 (1024 tokens) and 4 (512 tokens), all heads of one value group
-    for sequence in (0, 4):
+    # sequences 0 (1024 tokens) and 4 (512 tokens), and the longest one, 5 (8192 tokens: the
+    # long bands, two symbol tiles, dropout), each with all heads of one value group
+    for sequence, value_head in ((0, 2), (4, 2), (5, 6)):
+        heads = slice(value_head * group, (value_head + 1) * group)
         start, end = offsets[sequence], offsets[sequence + 1]
         q = query[start:end, heads].unsqueeze(0)
         k = key[start:end, heads].unsqueeze(0)
@@ -143,8 +143,8 @@ def test_packed_config5_full_size(cabi, c_oracle):
         close(grads[0][start:end, heads], want[0][0], "grad_query")
         close(grads[1][start:end, heads], want[1][0], "grad_key")
         close(grads[2][start:end, value_head:value_head + 1], want[2][0], "grad_value")
-    # forward routes of the longest sequence for one head
-    start, end = offsets[5], offsets[6]
+    # forward routes of the second longest sequence for one head
+    start, end = offsets[1], offsets[2]
     want_out, want_routes, _ = c_oracle.hard_forward(
         query[start:end, 17:18].unsqueeze(0), key[start:end, 17:18].unsqueeze(0),
         value[start:end, 2:3].unsqueeze(0), config["W"],

@@ -94,6 +94,33 @@ def test_packed_operator_matches_oracle(rosa, c_oracle):
         )
 
 
+def test_invalid_device_offsets_give_nan_at_the_operator(rosa):
+    """The reference kills the process on bad device cu_seqlens (tests/test_soft_varlen.py:
+    181-226); here the operator returns, and the mistake shows as NaN in the output, in every
+    gradient and therefore in any loss built on them.  Half-precision outputs carry it too."""
+
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        query = nonzero_randn((64, 2, 4), seed=1).to(dtype)
+        key = nonzero_randn((64, 2, 4), seed=2).to(dtype)
+        value = nonzero_randn((64, 1, 5), seed=3).to(dtype)
+        for offsets in ([0, 50, 30, 64], [0, 20, 70], [1, 64]):
+            cu = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
+            leaves = [t.to(DEVICE).requires_grad_() for t in (query, key, value)]
+            output = rosa.rosa_soft_varlen(*leaves, cu, max_suffix_length=8, dropout_p=0.1)
+            assert output.shape == (64, 2, 5) and bool(torch.isnan(output).all())
+            grads = torch.autograd.grad(output, leaves, torch.ones_like(output))
+            assert all(bool(torch.isnan(g).all()) for g in grads)
+            with torch.no_grad():
+                quiet = rosa.rosa_soft_varlen(*leaves, cu, max_suffix_length=8)
+            assert bool(torch.isnan(quiet).all())
+        good = torch.tensor([0, 20, 64], dtype=torch.int32, device=DEVICE)
+        leaves = [t.to(DEVICE).requires_grad_() for t in (query, key, value)]
+        output = rosa.rosa_soft_varlen(*leaves, good, max_suffix_length=8)
+        grads = torch.autograd.grad(output, leaves, torch.ones_like(output))
+        assert bool(torch.isfinite(output).all())
+        assert all(bool(torch.isfinite(g).all()) for g in grads)
+
+
 def test_no_grad_path_draws_no_seed_and_equals_train_forward(rosa):
     # reference tests/test_soft_cuda.py:745-810
     query, key, value, _ = device_inputs(seed=9)
@@ -322,3 +349,17 @@ def test_recording_the_training_step_into_a_graph_is_refused(rosa):
     # the stream is usable again afterwards
     output = rosa.rosa_soft(*leaves, max_suffix_length=12)
     assert output.shape == (2, 48, 4, 5)
+    # the exported backward operator refuses by itself, before it allocates or launches
+    q, k, v = (t.detach() for t in leaves)
+    _, pq, pk = torch.ops.rosa_soft.hard_forward(q, k, v, 12)
+    grad_output = torch.ones_like(output.detach())
+    empty = torch.empty(0, dtype=torch.int64, device=DEVICE)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be recorded into a HIP graph"):
+        with torch.cuda.graph(graph):
+            torch.ops.rosa_soft.surrogate_vjp_masked(
+                q, k, v, grad_output, pq, pk, empty, 12, 1.0, 0.0, 3.0, 7)
+    gradients = torch.ops.rosa_soft.surrogate_vjp_masked(
+        q, k, v, grad_output, pq, pk, empty, 12, 1.0, 0.0, 3.0, 7)
+    assert all(bool(torch.isfinite(g).all()) for g in gradients)

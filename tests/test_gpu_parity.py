@@ -11,6 +11,8 @@ section goes through the public operators and the dispatcher.  Bars:
   operator has cast gradients to float16 / bfloat16.
 """
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -288,31 +290,157 @@ def test_packed_equals_dense_batch_with_same_seed(cabi):
         torch.testing.assert_close(a.reshape(b.shape), b, rtol=2e-5, atol=2e-6)
 
 
-def test_invalid_device_offsets_are_clamped_and_reported(cabi):
-    """Offsets the host cannot see are sanitised on the device (no fault) and
-    the violation is reported through the workspace flag."""
-
-    import ctypes
+def test_invalid_device_offsets_poison_the_results(cabi, c_oracle):
+    """Offsets the host cannot see are checked on the device.  Invalid ones touch no token
+    (no fault), set the workspace flag and turn every output and gradient element into
+    NaN; valid ones leave the results exactly as the oracle has them.  (The reference
+    aborts the process: rosa_soft_kernels.cu:287-308, tests/test_soft_varlen.py:181-226.)"""
 
     total, H, D, Dv = 40, 2, 4, 3
-    query = nonzero_randn((total, H, D), seed=1).to(DEVICE)
-    value = nonzero_randn((total, 1, Dv), seed=2).to(DEVICE)
+    query = nonzero_randn((total, H, D), seed=1)
+    key = nonzero_randn((total, H, D), seed=3)
+    value = nonzero_randn((total, 1, Dv), seed=2)
+    grad_output = nonzero_randn((total, H, Dv), seed=4, floor=0.0)
+    q, k, v, go = (t.to(DEVICE) for t in (query, key, value, grad_output))
     library = cabi.load()
-    for offsets, bad in (([0, 10, 40], 0), ([0, 30, 20, 40], 1), ([0, 10, 50], 1), ([2, 40], 1)):
+    stream = torch.cuda.current_stream().cuda_stream
+    for offsets, bad in (([0, 10, 40], 0), ([0, 30, 20, 40], 1), ([0, 10, 50], 1), ([2, 40], 1),
+                         ([0, 10, 39], 1), ([0, -3, 40], 1), ([0, 0, 40, 40], 0)):
         cu = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
-        problem = cabi.make_problem(query, value, 8, cu)
+        problem = cabi.make_problem(q, v, 8, cu)
         size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
         workspace = torch.zeros(size, dtype=torch.uint8, device=DEVICE)
         out = torch.empty(total, H, Dv, device=DEVICE)
         words = torch.empty(2, H, total, dtype=torch.int32, device=DEVICE)
-        stream = torch.cuda.current_stream().cuda_stream
         status = library.rosa_hip_hard_forward(
-            ctypes.byref(problem), query.data_ptr(), query.data_ptr(), value.data_ptr(),
+            ctypes.byref(problem), q.data_ptr(), k.data_ptr(), v.data_ptr(),
             out.data_ptr(), words[0].data_ptr(), words[1].data_ptr(), None,
             workspace.data_ptr(), size, stream,
         )
         assert status == 0
         assert library.rosa_hip_read_offset_error(workspace.data_ptr(), stream) == bad
+        grads = cabi.surrogate_vjp(q, k, v, go, words[0], words[1], None, 8, 1.0, 0.0, 3.0, 7, cu)
+        torch.cuda.synchronize()
+        if bad:
+            assert bool(torch.isnan(out).all())
+            assert all(bool(torch.isnan(g).all()) for g in grads)
+        else:
+            want_out, _ = c_oracle.varlen_hard_forward(query, key, value, offsets, 8)
+            assert torch.equal(out.cpu(), want_out.float())
+            want = c_oracle.varlen_surrogate_vjp(query, key, value, offsets, grad_output,
+                                                 max_suffix_length=8)
+            for g, w in zip(grads, want):
+                assert_gradients_close(g, w, f"offsets {offsets}")
+
+
+def test_packed_record_budget_on_both_sides_of_the_device_decision(cabi, c_oracle):
+    """Packed layouts size the chunk records for the worst split of N tokens, capped by the
+    budget, and decide on the device (workspace header word 3) whether the records of the
+    actual lengths fit.  A budget that holds the actual records but not the worst case
+    must use them; one that is non-zero but too small must fall back to recomputation;
+    both must give the oracle's gradients."""
+
+    lengths, H, D, Hv, Dv, W, p, seed = [70, 0, 1, 300, 129], 2, 3, 2, 5, 16, 0.1, 4711
+    total = sum(lengths)
+    query, key, value, grad_output = (t[0] for t in make_case(1, total, H, D, Hv, Dv, seed=5))
+    offsets = [0] + list(np.cumsum(lengths))
+    want = c_oracle.varlen_surrogate_vjp(query, key, value, offsets, grad_output,
+                                         max_suffix_length=W, dropout_p=p, seed=seed)
+
+    def band_steps(length):  # (row, band) steps of one (sequence, head)
+        if length < 2:
+            return 0
+        bands = (length - 2) // 64 + 1
+        return bands * (length - 1) - 32 * bands * (bands - 1)
+
+    record_bytes = 4 * (128 + 32)  # (S, window) of 64 diagonals + 16 keep bits per lane
+    slots = lambda parts: (H * sum(band_steps(n) for n in parts)) // 16 \
+        + H * sum((n + 63) // 64 for n in parts) + 1
+    needed, worst = slots(lengths) * record_bytes, slots([total]) * record_bytes
+    assert needed < worst
+    q, k, v, go = (t.to(DEVICE).contiguous() for t in (query, key, value, grad_output))
+    cu = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
+    seed_tensor = torch.tensor(seed, dtype=torch.int64, device=DEVICE)
+    _, pq, pk, _ = cabi.hard_forward(q, k, v, W, cu)
+    sizes = {}
+    try:
+        for label, budget, fits in (("enough", needed + record_bytes, 1), ("short", needed // 2, 0),
+                                    ("one record", record_bytes, 0)):
+            cabi.set_record_budget(budget)
+            sizes[label] = cabi.vjp_workspace_bytes(q, v, W, cu, dropout=True)
+            workspace = torch.zeros(sizes[label], dtype=torch.uint8, device=DEVICE)
+            grads = cabi.surrogate_vjp(q, k, v, go, pq, pk, seed_tensor, W, 1.0, p, 3.0, 7, cu,
+                                       workspace=workspace)
+            torch.cuda.synchronize()
+            header = workspace[:16].view(torch.int32).cpu().tolist()
+            assert header[0] == 0 and header[3] == fits, (label, header)
+            for name, got, expected in zip("qkv", grads, want):
+                assert_gradients_close(got, expected, f"{label} d{name}")
+        cabi.set_record_budget(None)
+        full = cabi.vjp_workspace_bytes(q, v, W, cu, dropout=True)
+    finally:
+        cabi.set_record_budget(None)
+    assert sizes["one record"] < sizes["short"] < sizes["enough"] < full
+
+
+# --------------------------------------------------------------------------- the operator's edges as bits
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 7, 8, 16, 27, 32])
+def test_pack_symbols_matches_the_closed_form(cabi, bits):
+    # bit i = x[..., i] > 0; zero, -0, NaN and -inf give 0, +inf gives 1 (reference
+    # rosa_soft_kernels.cu:202-241, rosa_soft/runtime.py:130-146)
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        logits = nonzero_randn((3, 41, 5, bits), seed=bits).to(dtype)
+        flat = logits.view(-1)
+        flat[:5] = torch.tensor([0.0, -0.0, float("nan"), float("-inf"), float("inf")]).to(dtype)
+        weights = 1 << torch.arange(bits, dtype=torch.int64)
+        want = ((logits > 0).long() * weights).sum(-1)
+        words = cabi.pack_symbols(logits.to(DEVICE), torch.int32)
+        assert words.shape == (3, 41, 5) and words.dtype == torch.int32
+        assert torch.equal(words.cpu().long() & 0xFFFFFFFF, want)
+        if bits <= 8:
+            symbols = cabi.pack_symbols(logits.to(DEVICE), torch.uint8)
+            assert symbols.dtype == torch.uint8 and torch.equal(symbols.cpu().long(), want)
+        else:
+            with pytest.raises(RuntimeError, match="symbol width"):
+                cabi.pack_symbols(logits.to(DEVICE), torch.uint8)
+    empty = cabi.pack_symbols(torch.empty(0, 4, bits, device=DEVICE), torch.int32)
+    assert empty.shape == (0, 4)
+
+
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,dtype,pattern", FORWARD_CASES)
+def test_bit_form_of_the_output_expands_to_the_oracle_output(cabi, c_oracle, B, T, H, D, Hv, Dv,
+                                                            W, dtype, pattern):
+    query, key, value, _ = make_case(B, T, H, D, Hv, Dv, dtype, seed=T, pattern=pattern)
+    q, k, v = (t.to(DEVICE) for t in (query, key, value))
+    sign_words, routed = cabi.hard_forward_bits(q, k, v, W)
+    torch.cuda.synchronize()
+    want_out, want_routes, _ = c_oracle.hard_forward(query, key, value, W)
+    assert sign_words.shape == (B, T, H, (Dv + 31) // 32) and routed.shape == (B, T, H)
+    assert torch.equal(routed.cpu().bool(), (want_routes > 0).permute(0, 2, 1))
+    assert set(routed.cpu().unique().tolist()) <= {0, 1}
+    got = cabi.expand_output_bits(sign_words, routed, Dv)
+    assert torch.equal(got.cpu(), want_out.float())
+    # words of the null route and the bits beyond Dv are zero
+    assert int((sign_words.cpu()[~routed.cpu().bool()] != 0).sum()) == 0
+    if Dv % 32:
+        last = sign_words.cpu()[..., -1].long() & 0xFFFFFFFF
+        assert int((last >> (Dv % 32)).sum()) == 0
+
+
+def test_bit_form_of_the_packed_output_and_its_invalid_offset_marker(cabi, c_oracle):
+    offsets = [0, 9, 9, 70, 71, 130]
+    query = nonzero_randn((130, 4, 6), seed=1)
+    key = nonzero_randn((130, 4, 6), seed=2)
+    value = nonzero_randn((130, 2, 40), seed=3)
+    q, k, v = (t.to(DEVICE) for t in (query, key, value))
+    cu = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
+    sign_words, routed = cabi.hard_forward_bits(q, k, v, 12, cu)
+    want_out, _ = c_oracle.varlen_hard_forward(query, key, value, offsets, 12)
+    assert torch.equal(cabi.expand_output_bits(sign_words, routed, 40).cpu(), want_out)
+    bad = torch.tensor([0, 80, 60, 130], dtype=torch.int32, device=DEVICE)
+    sign_words, routed = cabi.hard_forward_bits(q, k, v, 12, bad)
+    assert bool((routed == 0xFF).all()) and int(sign_words.abs().sum()) == 0
 
 
 # --------------------------------------------------------------------------- golden vectors on the device

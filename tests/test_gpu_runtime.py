@@ -271,3 +271,69 @@ def test_random_chunkings_match_the_dense_definition(rosa, seed):
         label = f"seed {seed} case {case}: cuts {cuts}"
         assert torch.equal(torch.cat(outputs, dim=1).cpu(), want[0]), label
         assert torch.equal(torch.cat(positions, dim=1).cpu(), want[1]), label
+
+
+def test_logit_updates_pack_on_the_device_and_match_packed_updates(rosa):
+    """``update`` (sign logits, every float dtype, host or device) routes exactly like
+    ``update_packed`` on the symbols ``bit i = logit[..., i] > 0``; host inputs come back on
+    the host (reference rosa_soft/runtime.py:130-146, tests/test_runtime.py:318-345)."""
+
+    batch, tokens, heads, payload_heads, horizon = 2, 37, 4, 2, 6
+    generator = torch.Generator().manual_seed(50)
+    for qk_bits, payload_bits, dtype in ((8, 8, torch.float32), (3, 5, torch.float16),
+                                         (1, 7, torch.bfloat16), (8, 2, torch.float64)):
+        logits = [torch.randn(batch, tokens, h, bits, generator=generator).to(dtype)
+                  for h, bits in ((heads, qk_bits), (heads, qk_bits), (payload_heads, payload_bits))]
+        logits[0][0, 3, 1, 0] = 0.0            # zero, NaN and -inf quantise to bit 0, +inf to 1
+        logits[1][1, 5, 0, 0] = float("nan")
+        logits[2][0, 7, 1, 0] = float("-inf")
+        logits[2][0, 8, 1, 0] = float("inf")
+        symbols = []
+        for tensor in logits:
+            weights = 1 << torch.arange(tensor.size(-1), dtype=torch.int64)
+            symbols.append(((tensor > 0).long() * weights).sum(-1).to(torch.uint8))
+        want = expect_dense(*symbols, qk_bits, payload_bits, horizon)
+        for place in (DEVICE, "cpu"):
+            with rosa.RosaRuntime(heads, payload_heads, qk_bits, payload_bits, horizon) as runtime:
+                output, ends = runtime.update(*(t.to(place) for t in logits), return_packed=True)
+            assert output.device.type == torch.device(place).type
+            assert torch.equal(output.cpu(), want[0]) and torch.equal(ends.cpu(), want[1])
+
+
+def test_many_slots_and_heads_in_one_update(rosa):
+    # slots * heads beyond the 65535 blocks of a grid's second dimension
+    slots, tokens, heads, bits, horizon = 1100, 9, 64, 2, 4
+    query = random_packed((slots, tokens, heads), bits, 61)
+    key = random_packed((slots, tokens, heads), bits, 62)
+    payload = random_packed((slots, tokens, heads), bits, 63)
+    want = expect_dense(query, key, payload, bits, bits, horizon)
+    with rosa.RosaRuntime(heads, heads, bits, bits, horizon) as runtime:
+        first = runtime.update_packed(query[:, :8].to(DEVICE), key[:, :8].to(DEVICE),
+                                      payload[:, :8].to(DEVICE))
+        last = runtime.update_packed(query[:, 8:].to(DEVICE), key[:, 8:].to(DEVICE),
+                                     payload[:, 8:].to(DEVICE))     # decode-sized chunk
+    got_output = torch.cat([first[0], last[0]], dim=1).cpu()
+    got_ends = torch.cat([first[1], last[1]], dim=1).cpu()
+    assert torch.equal(got_output, want[0]) and torch.equal(got_ends, want[1])
+
+
+def test_updates_on_different_streams_are_serialised(rosa):
+    heads, bits, horizon = 2, 2, 7
+    query = random_packed((1, 3000, heads), bits, 71)
+    key = random_packed((1, 3000, heads), bits, 72)
+    payload = random_packed((1, 3000, 1), bits, 73)
+    want = expect_dense(query, key, payload, bits, bits, horizon)
+    q, k, p = (t.to(DEVICE) for t in (query, key, payload))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=DEVICE) for _ in range(3)]
+    pieces = []
+    with rosa.RosaRuntime(heads, 1, bits, bits, horizon) as runtime:
+        bounds = [0, 1500, 1501, 2600, 3000]
+        for index, (begin, end) in enumerate(zip(bounds[:-1], bounds[1:])):
+            stream = streams[index % 3] if index != 2 else None
+            pieces.append(runtime.update_packed(q[:, begin:end], k[:, begin:end], p[:, begin:end],
+                                                stream=stream, async_op=True))
+        results = [work.wait() for work in pieces]
+        torch.cuda.synchronize()
+    assert torch.equal(torch.cat([r[0] for r in results], dim=1).cpu(), want[0])
+    assert torch.equal(torch.cat([r[1] for r in results], dim=1).cpu(), want[1])

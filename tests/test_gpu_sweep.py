@@ -4,7 +4,10 @@ The hand-picked cases of test_gpu_parity.py name the code paths; this sweep cros
 them (symbol and value widths on both sides of the 8/16/32/64 tile limits, lengths around
 the 16-row chunk and 64-row segment sizes, windows shorter and longer than the sequence,
 dropout, gradient masks, packed layouts with empty sequences, the three dtypes), with the
-same bars: routes and outputs bit-exact, gradients to rtol 1e-4.
+same bars: routes and outputs bit-exact, gradients to
+``|got - want| <= 1e-4 |want| + 1e-5 max|want|``, widened only when the logits themselves
+are large (scale * L > 40, L = scale * U(min(W, T)); about 5x in this sweep, for
+scale = 2 with W = 500 on sequences of 500 rows and more).
 """
 
 import random
@@ -81,8 +84,10 @@ def check_case(cabi, c_oracle, rng, index, c):
     label = f"case {index}: {c}"
     assert torch.equal(out.cpu().float(), want_out.float()), label
     assert torch.equal(routes.cpu(), want_routes), label
-    # the same widening with the logit's magnitude as in test_surrogate_vjp_matches_oracle
-    slack = max(1.0, c["scale"] * max(longest, 8) / 40.0)
+    # the same widening with the logit's magnitude L = scale * U(min(W, longest)) as in
+    # test_surrogate_vjp_matches_oracle: none while scale * L <= 40
+    longest_logit = c["scale"] * 2.4142 * ((1.0 + min(c["W"], max(longest, 1))) ** 0.5 - 1.0)
+    slack = max(1.0, c["scale"] * longest_logit / 40.0)
     for bit, got, expected, name in zip((1, 2, 4), grads, want, "qkv"):
         if c["mask"] & bit:
             assert_gradients_close(got, expected, f"{label} d{name}", slack=slack)
