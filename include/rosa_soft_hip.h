@@ -122,6 +122,22 @@ int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query,
                                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * rosa_hip_hard_forward for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The workspace is a 16 MiB array that lives in the
+ * library's device image (one copy per GPU, held until the process ends), so the call
+ * takes no workspace argument and calls no allocator; it handles problems whose forward
+ * workspace fits, i.e. about tokens * H <= 4 190 000, and returns 3 with a message
+ * beyond that.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * on one GPU (different streams or threads) race and must be ordered by the caller.
+ * Outputs and their meaning are those of rosa_hip_hard_forward.
+ */
+int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query,
+                                 const void* key, const void* value, void* output,
+                                 int32_t* packed_query, int32_t* packed_key,
+                                 int32_t* routes, void* stream);
+
+/*
  * Sign symbols of a contiguous [rows][bits] tensor, in row order: bit i of a symbol is
  * x[row, i] > 0 (so 0, -0, NaN and -inf give 0).  `symbol_bytes` = 1 writes uint8
  * symbols (bits <= 8), the input format of rosa_hip_router_update; 4 writes uint32 words

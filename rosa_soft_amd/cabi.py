@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_hard_forward_bits",
+    "rosa_hip_hard_forward_static",
     "rosa_hip_pack_symbols",
     "rosa_hip_surrogate_vjp",
     "rosa_hip_router_update",
@@ -127,6 +128,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_hard_forward_bits.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
     ]
+    library.rosa_hip_hard_forward_static.restype = ctypes.c_int
+    library.rosa_hip_hard_forward_static.argtypes = [problem_p, vp, vp, vp, vp, vp, vp, vp, vp]
     library.rosa_hip_pack_symbols.restype = ctypes.c_int
     library.rosa_hip_pack_symbols.argtypes = [
         ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int, vp, ctypes.c_int, vp,
@@ -228,6 +231,50 @@ def hard_forward(
             _stream(query),
         )
     _check(status, "rosa_hip_hard_forward")
+    return output, packed_q, packed_k, routes
+
+
+def hard_forward_static(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    max_suffix_length: int,
+    cu_seqlens: Optional[Tensor] = None,
+    outputs: Optional[Tuple[Tensor, Tensor, Tensor, Tensor]] = None,
+) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """``hard_forward`` through the entry point that allocates nothing.
+
+    The library call takes no workspace (it uses the scratch array of its device image).
+    ``outputs`` = ``(output, packed_q, packed_k, routes)`` are written in place when given,
+    which is what a caller that cannot allocate does; otherwise they are created here.
+    """
+
+    library = load()
+    assert query.is_cuda and query.is_contiguous() and key.is_contiguous() and value.is_contiguous()
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    if cu_seqlens is None:
+        word_shape = (problem.B, problem.H, problem.T)
+        out_shape = (problem.B, problem.T, problem.H, problem.Dv)
+    else:
+        word_shape = (problem.H, problem.N)
+        out_shape = (problem.N, problem.H, problem.Dv)
+    with torch.cuda.device(query.device):
+        if outputs is None:
+            outputs = (
+                torch.empty(out_shape, dtype=query.dtype, device=query.device),
+                torch.empty(word_shape, dtype=torch.int32, device=query.device),
+                torch.empty(word_shape, dtype=torch.int32, device=query.device),
+                torch.empty(word_shape, dtype=torch.int32, device=query.device),
+            )
+        output, packed_q, packed_k, routes = outputs
+        assert output.shape == out_shape and output.dtype == query.dtype and output.is_contiguous()
+        assert all(w.shape == word_shape and w.dtype == torch.int32 and w.is_contiguous()
+                   for w in (packed_q, packed_k, routes))
+        status = library.rosa_hip_hard_forward_static(
+            ctypes.byref(problem), _ptr(query), _ptr(key), _ptr(value), _ptr(output),
+            _ptr(packed_q), _ptr(packed_k), _ptr(routes), _stream(query),
+        )
+    _check(status, "rosa_hip_hard_forward_static")
     return output, packed_q, packed_k, routes
 
 

@@ -30,6 +30,15 @@
 
 #include "../../include/rosa_soft_hip.h"
 
+#include <mutex>
+
+// Scratch memory of rosa_hip_hard_forward_static: the forward's workspace (route of every
+// row and the packed-sequence tables) for callers that cannot allocate.  Every device the
+// library runs on holds its own copy until the process ends.  In host code the array's name
+// is not a device address: the address of a device's copy comes from hipGetSymbolAddress.
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 constexpr int kWave = 64;
@@ -2844,6 +2853,28 @@ int forward_entry(const rosa_problem* problem, const void* query, const void* ke
   }
 }
 
+// Address of the current device's copy of `scratch`, looked up once per device.
+constexpr int kMaxDevices = 64;
+void* g_scratch_address[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int static_scratch_address(void** address) {
+  int device = -1;
+  const hipError_t current = hipGetDevice(&device);
+  if (current != hipSuccess) return fail_hip(current, "hipGetDevice");
+  if (device < 0 || device >= kMaxDevices) return fail(4, "static scratch: device index out of range");
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (g_scratch_address[device] == nullptr) {
+    void* found = nullptr;
+    const hipError_t status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (status != hipSuccess) return fail_hip(status, "hipGetSymbolAddress(scratch)");
+    if (found == nullptr) return fail(4, "static scratch: no device address");
+    g_scratch_address[device] = found;
+  }
+  *address = g_scratch_address[device];
+  return 0;
+}
+
 template <int DTYPE>
 void launch_pack_rows(const void* logits, int64_t rows, int bits, void* symbols, int symbol_bytes,
                       hipStream_t stream) {
@@ -2914,6 +2945,24 @@ int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query, c
   if (!sign_words || !routed) return fail(2, "hard_forward_bits: NULL output pointer");
   return forward_entry(problem, query, key, value, nullptr, packed_query, packed_key, nullptr,
                        nullptr, workspace, workspace_bytes, stream, sign_words, routed);
+}
+
+int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query, const void* key,
+                                 const void* value, void* output, int32_t* packed_query,
+                                 int32_t* packed_key, int32_t* routes, void* stream) {
+  if (!output) return fail(2, "hard_forward_static: NULL tensor pointer");
+  ProblemView view;
+  const int bad = check_problem(problem, &view);
+  if (bad != 0) return bad;
+  if (carve_forward(view).total > kStaticScratchBytes) {
+    return fail(3, "hard_forward_static: the problem needs more than the 16 MiB of static "
+                   "scratch (4 bytes per token and head); use rosa_hip_hard_forward");
+  }
+  void* address = nullptr;
+  const int status = static_scratch_address(&address);
+  if (status != 0) return status;
+  return forward_entry(problem, query, key, value, output, packed_query, packed_key, routes,
+                       nullptr, address, kStaticScratchBytes, stream, nullptr, nullptr);
 }
 
 int rosa_hip_pack_symbols(int dtype, const void* logits, int64_t rows, int bits, void* symbols,
