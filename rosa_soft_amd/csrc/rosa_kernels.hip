@@ -702,7 +702,9 @@ struct VjpParams {
   const uint32_t* packed_query;
   const uint32_t* packed_key;
   const uint32_t* value_bits;   // [value_words_total][NVW], head-major over value heads
-  const float* grad_rows;       // [head-major row][DVP] float32, zero padded
+  const uint16_t* grad_rows;    // [head-major row][grad_pitch] bfloat16 terms of grad_output
+  int grad_terms;               // terms per element: 3 for float32, 2 for float16, 1 for bfloat16
+  int grad_pitch;               // elements per row: terms * dvp rounded up to whole 32s
   float4* stats;                // [head-major row] (reference logit, denominator, numerator, base)
   const int64_t* dropout_seed;
   float scale, dropout_p, inverse_keep, mismatch_scale;
@@ -727,13 +729,32 @@ struct VjpParams {
   int total_units;
 };
 
-// grad_output -> float32 head-major rows padded to DVP.  One thread per float of the
-// destination: stores are contiguous, loads are runs of Dv elements.
+// Terms of the bfloat16 expansion of a float: x = t0 + t1 + t2 exactly (each term is the
+// bfloat16 nearest to what the terms before it leave), so that products with x can run on
+// the bfloat16 matrix pipe without losing float32 accuracy.  A float16 value needs two
+// terms, a bfloat16 value one.
+__device__ __forceinline__ uint32_t bf16_nearest(float x) {
+  // round to nearest even on the upper 16 bits; NaN stays NaN
+  const uint32_t bits = __float_as_uint(x);
+  if ((bits & 0x7fffffffu) > 0x7f800000u) return (bits >> 16) | 0x40u;
+  return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+}
+
+constexpr int kMaxGradTerms = 3;
+
+__host__ __device__ constexpr int grad_term_pitch(int terms, int dvp) {
+  return ((terms * dvp + 31) / 32) * 32;  // bfloat16 elements per row: whole 32-wide k blocks
+}
+
+// grad_output -> head-major rows of bfloat16 terms, [row][term][dvp] padded with zeros to
+// whole blocks of 32 elements (`pitch` elements per row).  One thread per (row, value
+// dimension of the padded width): loads are runs of Dv elements, stores of one term are
+// contiguous over the threads of a row.
 template <int DTYPE>
 __device__ __forceinline__ void prepare_grad_rows(
-    int64_t index, const void* __restrict__ grad_output, float* __restrict__ grad_rows,
+    int64_t index, const void* __restrict__ grad_output, uint16_t* __restrict__ grad_rows,
     int64_t rows, int H, int Dv, int dvp, int T, int N, int varlen, int value_stride,
-    int value_offset) {
+    int value_offset, int terms, int pitch) {
   if (index >= rows * dvp) return;
   const int64_t dst = index / dvp;  // head-major row
   const int d = static_cast<int>(index - dst * dvp);
@@ -746,9 +767,17 @@ __device__ __forceinline__ void prepare_grad_rows(
     const int64_t b = bh / H;
     source_row = (b * T + (dst - bh * T)) * H + (bh - b * H);
   }
-  grad_rows[index] =
+  float rest =
       d < Dv ? load_as_float<DTYPE>(grad_output, source_row * value_stride + value_offset + d)
              : 0.0f;
+  uint16_t* row = grad_rows + dst * pitch;
+  for (int t = 0; t < terms; ++t) {
+    const uint32_t term = bf16_nearest(rest);
+    row[t * dvp + d] = static_cast<uint16_t>(term);
+    // exact: the term holds the leading bits of `rest`; an infinite or NaN term ends the series
+    rest = (term & 0x7f80u) == 0x7f80u ? 0.0f : rest - __uint_as_float(term << 16);
+  }
+  for (int k = terms * dvp + d; k < pitch; k += dvp) row[k] = uint16_t(0);
 }
 
 __device__ __forceinline__ int64_t value_word_row(int64_t row, int Hv, int T, int N, int varlen) {
@@ -844,12 +873,13 @@ struct PrepareParams {
   Layout L;
   const void* grad_output;
   const void* value;
-  float* grad_rows;
+  uint16_t* grad_rows;
   uint32_t* value_bits;
   float4* stats;
   int32_t* work_counter;
   int64_t symbol_rows, value_rows;
   int Dv, dvp, nvw, value_stride, value_offset;
+  int grad_terms, grad_pitch;  // bfloat16 terms per grad_output element, elements per row
   float scale;
   int analytic;
   int ballot;  // value width is 8, 16, 32 or 64: pack signs with wave ballots
@@ -864,7 +894,8 @@ __global__ __launch_bounds__(256) void vjp_prepare_kernel(PrepareParams p) {
   const auto element = [&]() { return static_cast<int64_t>(block) * blockDim.x + threadIdx.x; };
   if (block < p.grad_blocks) {
     prepare_grad_rows<DTYPE>(element(), p.grad_output, p.grad_rows, p.symbol_rows, p.L.H, p.Dv,
-                             p.dvp, p.L.T, p.L.N, p.L.varlen, p.value_stride, p.value_offset);
+                             p.dvp, p.L.T, p.L.N, p.L.varlen, p.value_stride, p.value_offset,
+                             p.grad_terms, p.grad_pitch);
     return;
   }
   block -= p.grad_blocks;
@@ -911,7 +942,7 @@ struct BandView {
   const uint32_t* q;       // head-major words of this (sequence, head)
   const uint32_t* k;
   const uint32_t* vbits;   // value sign words of this (sequence, value head), NVW per token
-  const float* grad_rows;  // [t][dvp]
+  const uint16_t* grad_rows;  // [t][grad_pitch] bfloat16 terms
   float4* stats;           // [t]
   float* checkpoints;      // chunk records of this band, or NULL
   int record_floats;
@@ -980,22 +1011,23 @@ __device__ __forceinline__ void stage_value_columns(const BandView& view, int fi
   }
 }
 
-// grad_output rows of a block, zero for rows past the band's end; `pitch` floats per row
-template <int DVP>
+// bfloat16 terms of the grad_output rows of a block, zero for rows past the band's end;
+// `pitch` elements per row in LDS, `source_pitch` in the workspace
 __device__ __forceinline__ void stage_grad_rows(const BandView& view, int first, int count,
-                                                int lane, float* dst, int pitch) {
-  constexpr int kQuads = DVP / 4;
-  for (int index = lane; index < count * kQuads; index += kWave) {
-    const int r = index / kQuads;
-    const int quad = index - r * kQuads;
+                                                int lane, uint16_t* dst, int pitch,
+                                                int source_pitch) {
+  const int pieces = source_pitch / 8;  // 16 bytes each
+  for (int index = lane; index < count * pieces; index += kWave) {
+    const int r = index / pieces;
+    const int piece = index - r * pieces;
     const int i = first + r;
-    float4 value = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    uint4 value = make_uint4(0u, 0u, 0u, 0u);
     if (i < view.steps) {
       const int t = view.diag0 + 1 + i;
-      value = *reinterpret_cast<const float4*>(view.grad_rows + static_cast<int64_t>(t) * DVP +
-                                               4 * quad);
+      value = *reinterpret_cast<const uint4*>(view.grad_rows +
+                                              static_cast<int64_t>(t) * source_pitch + 8 * piece);
     }
-    *reinterpret_cast<float4*>(dst + r * pitch + 4 * quad) = value;
+    *reinterpret_cast<uint4*>(dst + r * pitch + 8 * piece) = value;
   }
 }
 
@@ -1111,31 +1143,128 @@ __device__ __forceinline__ float sign_from_bit31(uint32_t x) {
   return __uint_as_float((x & 0x80000000u) | 0x3f800000u);
 }
 
+// The contractions run on the bfloat16 matrix pipe: v_mfma_f32_16x16x32_bf16 multiplies a
+// 16 x 32 by a 32 x 16 matrix in the time v_mfma_f32_16x16x4_f32 takes for a 16 x 4 by
+// 4 x 16 one, with float32 accumulation.  Lane (li, lg) = (lane & 15, lane >> 4) supplies
+// row li of A and column li of B for k = 8 lg .. 8 lg + 7 (element 2 j of the operand is the
+// low half of its dword j) and receives rows 4 lg .. 4 lg + 3 of column li of the product.
+// One factor of every product here is exactly representable (signs, or grad_output as a
+// sum of bfloat16 terms); the other one is split into a leading bfloat16 and the bfloat16
+// nearest to the rest, which keeps 16 to 17 significant bits of it.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ v4f mfma_bf16(v4u a, v4u b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a),
+                                                 __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+}
+
+// [leading | rest << 16] of a float: the bfloat16 nearest to x and the bfloat16 nearest to
+// what it leaves.  Adjacent k indices of a matrix operand, so that a product with an
+// operand that repeats its element for both gives x (to 2^-17) times that element.
+__device__ __forceinline__ uint32_t split_bf16(float x) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+  const v2f twice = {x, x};
+  const uint32_t leading = __builtin_bit_cast(uint32_t, __builtin_convertvector(twice, v2bf));
+  const float head = __uint_as_float(leading << 16);
+  const v2f parts = {head, x - head};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(parts, v2bf));
+}
+
+// Three-term split of a float by truncation: x = leading + middle + rest to 2^-21 of |x|
+// (each term takes the upper 16 bits of what the terms before it leave; the subtractions
+// are exact).  Returns [leading | middle << 16]; `rest` receives the third term in the
+// upper half of its bits.
+__device__ __forceinline__ uint32_t split_bf16_exact(float x, uint32_t& rest) {
+  const uint32_t leading = __float_as_uint(x) & 0xffff0000u;
+  const float after_leading = x - __uint_as_float(leading);
+  const uint32_t middle = __float_as_uint(after_leading) & 0xffff0000u;
+  rest = __float_as_uint(after_leading - __uint_as_float(middle));
+  return __builtin_amdgcn_perm(middle, leading, 0x07060302u);  // leading >> 16 | middle
+}
+
+// 16 x 16 x 16 bfloat16 product: lane (li, lg) supplies k = 4 lg .. 4 lg + 3 (two dwords)
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ v4f mfma_bf16_k16(v2u a, v2u b, v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4s, a),
+                                                   __builtin_bit_cast(v4s, b), c, 0, 0, 0);
+}
+
+// Between matrix instructions of different shapes that share an accumulator: keeps the
+// groups apart for the scheduler and spends the wait states of the longest pipeline.
+__device__ __forceinline__ void mfma_shape_change() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// two 16-bit LDS words as one dword: first | second << 16
+__device__ __forceinline__ uint32_t pair_of(const uint16_t* first, const uint16_t* second) {
+  typedef uint16_t v2h __attribute__((ext_vector_type(2)));
+  const v2h both = {*first, *second};
+  return __builtin_bit_cast(uint32_t, both);
+}
+
+// bfloat16 -1.0 in both halves where bit `bit` of `word` is set, +1.0 where it is clear: the
+// negated symbol for both terms of a split operand; callers fold the sign into their scale.
+__device__ __forceinline__ uint32_t negated_symbol_pair(uint32_t word, int bit) {
+  const int spread = __builtin_amdgcn_sbfe(static_cast<int>(word), bit, 1);  // 0 or all ones
+  return (static_cast<uint32_t>(spread) & 0x80008000u) | 0x3f803f80u;
+}
+
+// Four sign bits -> four bfloat16 values (+1.0 where the bit is set, -1.0 where it is
+// clear) as two dwords: a table of 16 entries, 128 bytes, one entry per LDS bank pair, so
+// that any mix of entries is read without a bank conflict.
+constexpr int kSignTableWords = 32;
+
+__device__ __forceinline__ void fill_sign_table(uint32_t* table, int lane) {
+  if (lane < kSignTableWords) {
+    const int nibble = lane >> 1;
+    const int low = (nibble >> (2 * (lane & 1))) & 1;
+    const int high = (nibble >> (2 * (lane & 1) + 1)) & 1;
+    table[lane] = (low ? 0x3f80u : 0xbf80u) | ((high ? 0x3f80u : 0xbf80u) << 16);
+  }
+}
+
 // Utilities u(t, a) = sum_d grad_output[t, d] * sign(v[a, d]) of 16 rows against
 // their 80 window columns on the matrix cores, written in (row r, lane l)
 // coordinates: out[r * pitch + l] for the pair on diagonal lane l, whose window
-// column is c = 64 - l + r.  `grad_tile` holds the 16 grad_output rows
-// (`grad_pitch` floats each, zero beyond Dv), `value_columns` the sign words of
-// the window columns (NVW per column).  Elements of the first and last column
-// tile that belong to no lane go to `discard` (one float per lane).
+// column is c = 64 - l + r.  `grad_tile` holds the bfloat16 terms of the 16 grad_output
+// rows, `grad_pitch` elements each: k = term * DVP + d, `k_blocks` blocks of 32
+// (zero beyond the last term); the sum over the terms is the float32 product.
+// `value_columns` holds the sign words of the window columns (NVW per column).  Elements
+// of the first and last column tile that belong to no lane go to `discard` (one float
+// per lane).
 template <int NVW, int DVP>
-__device__ __forceinline__ void utility_tile(const float* grad_tile, int grad_pitch,
-                                             const uint32_t* value_columns, float* out,
-                                             int pitch, float* discard, int lane) {
+__device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad_pitch,
+                                             int k_blocks, const uint32_t* value_columns,
+                                             const uint32_t* sign_table, float* out, int pitch,
+                                             float* discard, int lane) {
   const int li = lane & 15;
   const int lg = lane >> 4;
+  const uint16_t* a_row = grad_tile + li * grad_pitch + 8 * lg;
 #pragma unroll
   for (int m = 0; m < 5; ++m) {
-    // inverted and moved down by lg: bit 4 ks of a word is the inverted sign bit 4 ks + lg
     uint32_t words[NVW];
 #pragma unroll
-    for (int w = 0; w < NVW; ++w) words[w] = ~value_columns[(16 * m + li) * NVW + w] >> lg;
+    for (int w = 0; w < NVW; ++w) words[w] = value_columns[(16 * m + li) * NVW + w];
     v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int kBlocksMax = grad_term_pitch(kMaxGradTerms, DVP) / 32;
 #pragma unroll
-    for (int ks = 0; ks < DVP / 4; ++ks) {
-      const float a_value = grad_tile[li * grad_pitch + 4 * ks + lg];
-      const float b_value = sign_from_bit31(words[(4 * ks) >> 5] << (31 - ((4 * ks) & 31)));
-      acc = mfma_16x16x4(a_value, b_value, acc);
+    for (int q = 0; q < kBlocksMax; ++q) {
+      if (q >= k_blocks) break;  // wave-uniform
+      const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
+      // this lane's k = 32 q + 8 lg .. + 7 are eight value dimensions of one term
+      const int d0 = (32 * q + 8 * lg) & (DVP - 1);
+      uint32_t word = words[0];
+      if constexpr (NVW > 1) word = d0 >= 32 ? words[1] : words[0];
+      const uint32_t byte = word >> (d0 & 31);
+      const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
+      const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
+      acc = mfma_bf16(a, v4u{low.x, low.y, high.x, high.y}, acc);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -1163,7 +1292,7 @@ __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, Ban
       ? static_cast<int64_t>(value_head) * P.L.N + u.start
       : (static_cast<int64_t>(u.seq) * P.L.Hv + value_head) * P.L.T;
   view.vbits = P.value_bits + value_base * NVW;
-  view.grad_rows = P.grad_rows + u.word_base * P.dvp;
+  view.grad_rows = P.grad_rows + u.word_base * P.grad_pitch;
   view.stats = P.stats + u.word_base;
   // position of the band in the global (step, band) order of the cached data
   int64_t steps_before, bands_before;
@@ -1253,7 +1382,12 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
   constexpr int kWeightPitch = 68;
   __shared__ __attribute__((aligned(16))) uint32_t rows[kBlockRows * kRowWords];
-  __shared__ __attribute__((aligned(16))) float grads[kBlockRows * DVP];
+  // bfloat16 terms of the block's grad_output rows; sized for three terms, 16 bytes of
+  // padding per row against bank conflicts of the operand reads
+  constexpr int kGradChunksMax = grad_term_pitch(kMaxGradTerms, DVP) / 8;  // 16-byte pieces per row
+  constexpr int kGradPitchMax = 8 * kGradChunksMax + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t grads[kBlockRows * kGradPitchMax];
+  __shared__ __attribute__((aligned(16))) uint32_t sign_table[kSignTableWords];
   __shared__ uint32_t value_columns[(kBlockRows + kWave) * NVW];
   __shared__ __attribute__((aligned(16))) float utilities[kChunk * kUtilityPitch];  // u, then e d u
   __shared__ __attribute__((aligned(16))) float weights[kChunk * kWeightPitch];     // e
@@ -1278,6 +1412,9 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   const int last_step = view.steps - 1;
   // without symbol gradients no utilities are computed and the tile stays zero
   for (int index = lane; index < kChunk * kUtilityPitch; index += kWave) utilities[index] = 0.0f;
+  fill_sign_table(sign_table, lane);
+  const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row actually present
+  const int grad_lds_pitch = P.grad_pitch + 8;
   for (int first = 0; first < view.steps; first += kBlockRows) {
     const int count = min(kBlockRows, view.steps - first);
     wave_lds_fence();
@@ -1295,21 +1432,21 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
         symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
         stat = view.stats[t];
       }
-      constexpr int kQuads = DVP / 4;
-      constexpr int kGradParts = (kBlockRows * kQuads + kWave - 1) / kWave;
+      constexpr int kGradParts = (kBlockRows * kGradChunksMax + kWave - 1) / kWave;
       constexpr int kValueParts = ((kBlockRows + kWave) * NVW + kWave - 1) / kWave;
-      float4 grad_in[kGradParts];
+      uint4 grad_in[kGradParts];
       uint32_t value_in[kValueParts];
       if (needs_utility) {
 #pragma unroll
         for (int part = 0; part < kGradParts; ++part) {
           const int index = part * kWave + lane;
-          const int r = index / kQuads;
-          grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          if (r < kBlockRows && first + r < view.steps) {
-            grad_in[part] = *reinterpret_cast<const float4*>(
-                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * DVP +
-                4 * (index - r * kQuads));
+          const int r = index / kGradChunksMax;
+          const int piece = index - r * kGradChunksMax;
+          grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
+          if (r < kBlockRows && piece < grad_chunks && first + r < view.steps) {
+            grad_in[part] = *reinterpret_cast<const uint4*>(
+                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * P.grad_pitch +
+                8 * piece);
           }
         }
 #pragma unroll
@@ -1331,9 +1468,10 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
 #pragma unroll
         for (int part = 0; part < kGradParts; ++part) {
           const int index = part * kWave + lane;
-          const int r = index / kQuads;
-          if (r < kBlockRows) {
-            *reinterpret_cast<float4*>(grads + r * DVP + 4 * (index - r * kQuads)) = grad_in[part];
+          const int r = index / kGradChunksMax;
+          const int piece = index - r * kGradChunksMax;
+          if (r < kBlockRows && piece < grad_chunks) {
+            *reinterpret_cast<uint4*>(grads + r * grad_lds_pitch + 8 * piece) = grad_in[part];
           }
         }
 #pragma unroll
@@ -1356,8 +1494,9 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
-        utility_tile<NVW, DVP>(grads + local * DVP, DVP, value_columns + local * NVW, utilities,
-                               kUtilityPitch, discard, lane);
+        utility_tile<NVW, DVP>(grads + local * grad_lds_pitch, grad_lds_pitch, P.grad_pitch / 32,
+                               value_columns + local * NVW, sign_table, utilities, kUtilityPitch,
+                               discard, lane);
         wave_lds_fence();
       }
       uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
@@ -1502,7 +1641,13 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
 }
 
 // rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
-constexpr int gradient_segment(int dvp) { return dvp >= 64 ? 32 : 64; }
+constexpr int gradient_segment(int dvp) { return dvp >= 16 ? 32 : 64; }
+
+// bfloat16 elements of padding per staged grad_output row (none at the narrowest width,
+// where the block's LDS decides how many blocks a compute unit holds)
+constexpr int gradient_row_padding(int dvp) { return dvp > 8 ? 8 : 0; }
+
+constexpr int kRestPitch = 100;  // 16-bit elements per row of the third-term plane
 
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
@@ -1510,7 +1655,6 @@ __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr bool kFetchAhead = VT == 1 && DT == 1;  // registers to spare for operands in flight
-  constexpr int GP = DVP;               // pitch of the staged grad_output rows
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds[];
@@ -1518,14 +1662,23 @@ void vjp_gradients_kernel(VjpParams P) {
                                   // row-statistics pass left no records
   int* ck_window = reinterpret_cast<int*>(lds + SEG_CHUNKS * kWave);
   float* tile = lds + 2 * SEG_CHUNKS * kWave;                // [kChunk][kTilePitch]
-  float* grad_rows_lds = tile + kChunk * kTilePitch;         // [SEG][GP]
-  uint32_t* rows = reinterpret_cast<uint32_t*>(grad_rows_lds + SEG * GP);  // [SEG][kRowWords]
+  uint32_t* tile_bits = reinterpret_cast<uint32_t*>(tile);   // the same tile as split operands
+  uint32_t* rows = reinterpret_cast<uint32_t*>(tile + kChunk * kTilePitch);  // [SEG][kRowWords]
   uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
   uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
   uint32_t* query_rows = value_window + (SEG + kWave) * NVW; // [SEG] query words of the rows
   float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
   uint32_t* old_key_window = reinterpret_cast<uint32_t*>(discard + kWave);  // [SEG + 64] key words
                                                              // of the columns W + 1 to the left
+  uint32_t* sign_table = old_key_window + SEG + kWave;       // [kSignTableWords]
+  // third bfloat16 term of the gate adjoints, [kChunk][kRestPitch], same geometry as `tile`
+  uint16_t* rest_plane = reinterpret_cast<uint16_t*>(sign_table + kSignTableWords);
+  // [SEG][GP] bfloat16 terms of the grad_output rows (GP elements per row: the terms in
+  // whole 32-element blocks, plus 16 bytes against bank conflicts where LDS allows)
+  uint16_t* grad_rows_lds = rest_plane + kChunk * kRestPitch;
+  const int GP = P.grad_pitch + gradient_row_padding(DVP);
+  const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row
+  constexpr int kGradChunksMax = grad_term_pitch(kMaxGradTerms, DVP) / 8;
 
   const int lane = threadIdx.x;
   const int li = lane & 15;   // MFMA row (A) / column (B, C) index
@@ -1545,6 +1698,8 @@ void vjp_gradients_kernel(VjpParams P) {
 
   // zero the tile once: its margins are never written again
   for (int index = lane; index < kChunk * kTilePitch; index += kWave) tile[index] = 0.0f;
+  for (int index = lane; index < kChunk * kRestPitch; index += kWave) rest_plane[index] = 0;
+  fill_sign_table(sign_table, lane);
   wave_lds_fence();
 
   for (;;) {
@@ -1794,23 +1949,24 @@ void vjp_gradients_kernel(VjpParams P) {
           store_rows_and_columns();
           __builtin_amdgcn_sched_barrier(0);
         }
-        constexpr int kQuads = DVP / 4;
-        constexpr int kGradParts = SEG * kQuads / kWave;
-        static_assert(kGradParts * kWave == SEG * kQuads, "whole float4s per lane");
+        constexpr int kGradParts = SEG * kGradChunksMax / kWave;
+        static_assert(kGradParts * kWave == SEG * kGradChunksMax, "whole 16-byte pieces per lane");
         // the grad_output rows come in groups that fit the registers free at this point
-        constexpr int kGradGroup = kGradParts;
+        constexpr int kGradGroup = kGradParts % 4 == 0 ? 4 : (kGradParts % 3 == 0 ? 3 : 1);
+        static_assert(kGradParts % kGradGroup == 0, "whole groups");
 #pragma unroll
         for (int group = 0; group < kGradParts; group += kGradGroup) {
-          float4 grad_in[kGradGroup];
+          uint4 grad_in[kGradGroup];
 #pragma unroll
           for (int part = 0; part < kGradGroup; ++part) {
             const int index = (group + part) * kWave + lane;
-            const int r = index / kQuads;
-            grad_in[part] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (seg_first + r < view.steps) {
-              grad_in[part] = *reinterpret_cast<const float4*>(
-                  view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * DVP +
-                  4 * (index - r * kQuads));
+            const int r = index / kGradChunksMax;
+            const int piece = index - r * kGradChunksMax;
+            grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
+            if (piece < grad_chunks && seg_first + r < view.steps) {
+              grad_in[part] = *reinterpret_cast<const uint4*>(
+                  view.grad_rows +
+                  static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * P.grad_pitch + 8 * piece);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -1820,9 +1976,11 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
           for (int part = 0; part < kGradGroup; ++part) {
             const int index = (group + part) * kWave + lane;
-            const int r = index / kQuads;
-            *reinterpret_cast<float4*>(grad_rows_lds + r * GP + 4 * (index - r * kQuads)) =
-                grad_in[part];
+            const int r = index / kGradChunksMax;
+            const int piece = index - r * kGradChunksMax;
+            if (piece < grad_chunks) {
+              *reinterpret_cast<uint4*>(grad_rows_lds + r * GP + 8 * piece) = grad_in[part];
+            }
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -1832,7 +1990,7 @@ void vjp_gradients_kernel(VjpParams P) {
           const int i = seg_first + lane;
           query_rows[lane] = i < view.steps ? view.q[view.diag0 + 1 + i] : 0u;
         }
-        stage_grad_rows<DVP>(view, seg_first, SEG, lane, grad_rows_lds, GP);
+        stage_grad_rows(view, seg_first, SEG, lane, grad_rows_lds, GP, P.grad_pitch);
         for (int index = lane; index < SEG + kWave; index += kWave) {
           const int a = seg_first - 63 + index;  // column; key position a - 1
           key_window[index] = (a >= 1 && a <= view.len - 1) ? view.k[a - 1] : 0u;
@@ -1876,14 +2034,14 @@ void vjp_gradients_kernel(VjpParams P) {
         // sliding registers of the chunk's first step: column first - lane
         band.key_word = key_window[local + 63 - lane];
         band.old_key_word = old_key_window[local + 63 - lane];
-        const float* grad_tile = grad_rows_lds + local * GP;
+        const uint16_t* grad_tile = grad_rows_lds + local * GP;
         // window column c <-> a = first + 1 - 64 + c (first + 1 is lane 0's column in the first row)
         const uint32_t* key_tile = key_window + local;
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
-          utility_tile<NVW, DVP>(grad_tile, GP, value_window + local * NVW, tile + 16, kTilePitch,
-                                 discard, lane);
+          utility_tile<NVW, DVP>(grad_tile, GP, P.grad_pitch / 32, value_window + local * NVW,
+                                 sign_table, tile + 16, kTilePitch, discard, lane);
           wave_lds_fence();
         }
         issue_pending();
@@ -1965,7 +2123,7 @@ void vjp_gradients_kernel(VjpParams P) {
             }
             const float adjoint =
                 (probability * adjoint_gain) * (keep * utility - expected) * inv_root;
-            tile[r * kTilePitch + 16 + lane] = probability * keep;
+            tile_bits[r * kTilePitch + 16 + lane] = split_bf16(probability * keep);
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
             keep_adjoint[r] = live ? adjoint : 0.0f;
@@ -1989,51 +2147,45 @@ void vjp_gradients_kernel(VjpParams P) {
         wave_lds_fence();
 
         // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = first + 1 - 64 + c);
-        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r].
+        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r], a dword
+        // holding the two bfloat16 terms of the pair's value.  One matrix instruction per
+        // tile contracts all 16 rows: k = 2 r + term, lane (li, lg) brings rows 4 lg .. 4 lg + 3
+        // of column 16 m + li.
+        const auto column_operands = [&](v4u (&operands)[kWindowTiles]) {
+#pragma unroll
+          for (int m = 0; m < kWindowTiles; ++m) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int r = 4 * lg + j;
+              operands[m][j] = tile_bits[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+            }
+          }
+        };
         if (want_v) {
-          // narrow tiles: operands of every product are fetched one k step ahead, without
-          // branches, so that the loads of a step fly while the products of the step before
-          // it run (wide tiles have no registers to spare for that)
-          float a_next[kWindowTiles];
-          float grad_next[VT];
-          const auto fetch = [&](int step) {
-            const int r = step + 4 * lg;
+          v4u weights[kWindowTiles];
+          column_operands(weights);
+          // the other factor: grad_output of the same rows, term by term, each element
+          // repeated for the two terms of the weight (the third term of a float32
+          // grad_output is below the accuracy of the split weights and is left out)
+          const int terms = P.grad_terms < 2 ? P.grad_terms : 2;
 #pragma unroll
-            for (int n = 0; n < VT; ++n) {
-              grad_next[n] = grad_tile[r * GP + min(16 * n + li, DVP - 1)];
-            }
+          for (int n = 0; n < VT; ++n) {
+            const int d = 16 * n + li;
+            const uint16_t* source = grad_tile + (4 * lg) * GP + (d < DVP ? d : DVP - 1);
 #pragma unroll
-            for (int m = 0; m < kWindowTiles; ++m) {
-              a_next[m] = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
-            }
-          };
-          if constexpr (kFetchAhead) fetch(0);
+            for (int t = 0; t < 2; ++t) {
+              if (t >= terms) break;  // wave-uniform
+              v4u grads;
 #pragma unroll
-          for (int step = 0; step < kChunk / 4; ++step) {
-            if constexpr (!kFetchAhead) fetch(step);
-            float a_now[kWindowTiles];
-            float grad_now[VT];
+              for (int j = 0; j < 4; ++j) {
+                const uint32_t element = source[j * GP + t * DVP];
+                grads[j] = d < DVP ? element | (element << 16) : 0u;
+              }
 #pragma unroll
-            for (int m = 0; m < kWindowTiles; ++m) a_now[m] = a_next[m];
-#pragma unroll
-            for (int n = 0; n < VT; ++n) grad_now[n] = grad_next[n];
-            if constexpr (kFetchAhead) {
-              if (step + 1 < kChunk / 4) fetch(step + 1);
-              // keep the loads above the products (the scheduler would sink each load to its use)
-              __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int n = 0; n < VT; ++n) {  // columns past the value width are padding
-              if (16 * n + li >= DVP) grad_now[n] = 0.0f;
-            }
-#pragma unroll
-            for (int m = 0; m < kWindowTiles; ++m) {
-#pragma unroll
-              for (int n = 0; n < VT; ++n) {
-                value_acc[m][n] = mfma_16x16x4(a_now[m], grad_now[n], value_acc[m][n]);
+              for (int m = 0; m < kWindowTiles; ++m) {
+                value_acc[m][n] = mfma_bf16(weights[m], grads, value_acc[m][n]);
               }
             }
-            if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
           }
         }
 
@@ -2049,7 +2201,9 @@ void vjp_gradients_kernel(VjpParams P) {
               const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
               adjoint_carry = b;
               gate_below = keep_gate[r];
-              tile[r * kTilePitch + 16 + lane] = b * keep_evidence[r];
+              uint32_t rest;
+              tile_bits[r * kTilePitch + 16 + lane] = split_bf16_exact(b * keep_evidence[r], rest);
+              rest_plane[r * kRestPitch + 16 + lane] = static_cast<uint16_t>(rest >> 16);
             }
           } else {
 #pragma unroll
@@ -2080,97 +2234,89 @@ void vjp_gradients_kernel(VjpParams P) {
             const float h = fmaf(b, keep_evidence[r], -ring_sum);
             if (ring_live == 0) ring_sum = 0.0f;
             const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
-            tile[r * kTilePitch + 16 + lane] = active ? h : 0.0f;
+            uint32_t rest;
+            tile_bits[r * kTilePitch + 16 + lane] = split_bf16_exact(active ? h : 0.0f, rest);
+            rest_plane[r * kRestPitch + 16 + lane] = static_cast<uint16_t>(rest >> 16);
           }
           }
           wave_lds_fence();
 
           if (want_k) {
-            float a_next[kWindowTiles];
-            uint32_t q_next = 0u;
-            const auto fetch = [&](int step) {
-              const int r = step + 4 * lg;
-              q_next = query_rows[local + r];
+            v4u adjoints[kWindowTiles];
+            v2u adjoint_rests[kWindowTiles];  // the third terms: k = r, a product of their own
+            column_operands(adjoints);
+#pragma unroll
+            for (int m = 0; m < kWindowTiles; ++m) {
+              const uint16_t* column = rest_plane + 16 + 64 - (16 * m + li);
+              const int r = 4 * lg;
+              adjoint_rests[m] = v2u{
+                  pair_of(column + r * (kRestPitch + 1), column + (r + 1) * (kRestPitch + 1)),
+                  pair_of(column + (r + 2) * (kRestPitch + 1), column + (r + 3) * (kRestPitch + 1))};
+            }
+            const uint4 q_words = *reinterpret_cast<const uint4*>(query_rows + local + 4 * lg);
+#pragma unroll
+            for (int n = 0; n < DT; ++n) {
+              const int bit = 16 * n + li;
+              const v4u symbols = {negated_symbol_pair(q_words.x, bit), negated_symbol_pair(q_words.y, bit),
+                                   negated_symbol_pair(q_words.z, bit), negated_symbol_pair(q_words.w, bit)};
+              // one element per row for the third terms: low half of one row, high half of the next
+              const v2u symbols_once = {__builtin_amdgcn_perm(symbols[1], symbols[0], 0x07060100u),
+                                        __builtin_amdgcn_perm(symbols[3], symbols[2], 0x07060100u)};
+              // A 16x16x16 product that accumulates onto the result of a 16x16x32 product
+              // must not issue right behind it: the compiler leaves out the wait states
+              // this pair needs (seen as wrong sums), so the two shapes run as separate
+              // groups with the wait states written out between them.
 #pragma unroll
               for (int m = 0; m < kWindowTiles; ++m) {
-                a_next[m] = tile[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+                key_acc[m][n] = mfma_bf16(adjoints[m], symbols, key_acc[m][n]);
               }
-            };
-            if constexpr (kFetchAhead) fetch(0);
-#pragma unroll
-            for (int step = 0; step < kChunk / 4; ++step) {
-              if constexpr (!kFetchAhead) fetch(step);
-              float a_now[kWindowTiles];
-#pragma unroll
-              for (int m = 0; m < kWindowTiles; ++m) a_now[m] = a_next[m];
-              const uint32_t q_word = q_next;
-              if constexpr (kFetchAhead) {
-                if (step + 1 < kChunk / 4) fetch(step + 1);
-              }
-              float query_b[DT];
-#pragma unroll
-              for (int n = 0; n < DT; ++n) query_b[n] = negated_symbol(q_word, 16 * n + li);
-              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
+              mfma_shape_change();
 #pragma unroll
               for (int m = 0; m < kWindowTiles; ++m) {
-#pragma unroll
-                for (int n = 0; n < DT; ++n) {
-                  key_acc[m][n] = mfma_16x16x4(a_now[m], query_b[n], key_acc[m][n]);
-                }
+                key_acc[m][n] = mfma_bf16_k16(adjoint_rests[m], symbols_once, key_acc[m][n]);
               }
-              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
+              mfma_shape_change();
             }
           }
           // row sums: rows are complete for this band after the chunk
           if (want_q) {
-            // four interleaved partial sums: no product waits for the one before it
-            constexpr int kParts = 4;
-            v4f query_part[kParts][DT];
+            // k slice lg of step s <-> window columns 20 lg + 4 s .. + 3 (both terms of each):
+            // every lane reads 20 consecutive key words, and the skewed tile reads of the 64
+            // lanes fall into different banks
+            // the third terms accumulate apart (see above: one instruction shape per
+            // accumulator chain)
+            v4f query_part[3][DT];
 #pragma unroll
-            for (int part = 0; part < kParts; ++part) {
+            for (int part = 0; part < 3; ++part) {
 #pragma unroll
               for (int n = 0; n < DT; ++n) query_part[part][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             }
-            // k slice lg of step s <-> window column 20 lg + s: every lane reads 20
-            // consecutive key words
-            uint32_t key_words[4 * kWindowTiles];
 #pragma unroll
-            for (int quad = 0; quad < kWindowTiles; ++quad) {
-              const uint4 four =
-                  *reinterpret_cast<const uint4*>(key_tile + 4 * kWindowTiles * lg + 4 * quad);
-              key_words[4 * quad] = four.x;
-              key_words[4 * quad + 1] = four.y;
-              key_words[4 * quad + 2] = four.z;
-              key_words[4 * quad + 3] = four.w;
-            }
-            // the tile column of step s, fetched kAhead steps before its product
-            constexpr int kAhead = kFetchAhead ? 8 : 1;
-            float a_ahead[kAhead];
-            const auto tile_value = [&](int step) {
-              const int c = 4 * kWindowTiles * lg + step;
-              return tile[li * kTilePitch + 16 + 64 - c + li];
-            };
+            for (int step = 0; step < kWindowTiles; ++step) {
+              const uint4 k_words =
+                  *reinterpret_cast<const uint4*>(key_tile + 4 * kWindowTiles * lg + 4 * step);
+              v4u adjoints;
+              const int c0 = 4 * kWindowTiles * lg + 4 * step;
 #pragma unroll
-            for (int step = 0; step < kAhead; ++step) a_ahead[step] = tile_value(step);
-#pragma unroll
-            for (int step = 0; step < 4 * kWindowTiles; ++step) {
-              const float a_value = a_ahead[step % kAhead];
-              if (step + kAhead < 4 * kWindowTiles) {
-                a_ahead[step % kAhead] = tile_value(step + kAhead);
+              for (int j = 0; j < 4; ++j) {
+                adjoints[j] = tile_bits[li * kTilePitch + 16 + 64 - (c0 + j) + li];
               }
-              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
+              const uint16_t* rests = rest_plane + li * kRestPitch + 16 + 64 - c0 + li;
+              const v2u adjoint_rests = {pair_of(rests, rests - 1), pair_of(rests - 2, rests - 3)};
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
-                query_part[step % kParts][n] =
-                    mfma_16x16x4(a_value, negated_symbol(key_words[step], 16 * n + li),
-                                 query_part[step % kParts][n]);
+                const int bit = 16 * n + li;
+                const v4u symbols = {negated_symbol_pair(k_words.x, bit), negated_symbol_pair(k_words.y, bit),
+                                     negated_symbol_pair(k_words.z, bit), negated_symbol_pair(k_words.w, bit)};
+                const v2u symbols_once = {__builtin_amdgcn_perm(symbols[1], symbols[0], 0x07060100u),
+                                          __builtin_amdgcn_perm(symbols[3], symbols[2], 0x07060100u)};
+                query_part[step & 1][n] = mfma_bf16(adjoints, symbols, query_part[step & 1][n]);
+                query_part[2][n] = mfma_bf16_k16(adjoint_rests, symbols_once, query_part[2][n]);
               }
-              if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int n = 0; n < DT; ++n) {
-              done_query[n] = (query_part[0][n] + query_part[1][n]) +
-                              (query_part[2][n] + query_part[3][n]);
+              done_query[n] = (query_part[0][n] + query_part[1][n]) + query_part[2][n];
             }
           }
         }
@@ -2247,6 +2393,7 @@ struct ProblemView {
   int64_t tokens;        // B*T or N
   int64_t symbol_rows;   // tokens * H
   int64_t value_rows;    // tokens * Hv
+  int grad_terms;        // bfloat16 terms that represent a grad_output element exactly
 };
 
 int check_problem(const rosa_problem* p, ProblemView* out) {
@@ -2281,6 +2428,7 @@ int check_problem(const rosa_problem* p, ProblemView* out) {
   const int bound = L.varlen ? L.N : L.T;
   if (L.W > bound) L.W = bound;
   out->L = L;
+  out->grad_terms = p->dtype == ROSA_DTYPE_F32 ? 3 : (p->dtype == ROSA_DTYPE_F16 ? 2 : 1);
   out->tokens = tokens;
   out->symbol_rows = tokens * p->H;
   out->value_rows = tokens * p->Hv;
@@ -2346,7 +2494,8 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   const int slice_width = std::min(v.L.Dv, kValueSlice);
   const int dvp = padded_value_width(slice_width);
   w.stats = cursor; cursor += align_up(sizeof(float) * 4 * rows);
-  w.grad_rows = cursor; cursor += align_up(sizeof(float) * rows * dvp);
+  w.grad_rows = cursor;
+  cursor += align_up(sizeof(uint16_t) * rows * grad_term_pitch(v.grad_terms, dvp));
   w.value_bits = cursor;
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(slice_width));
   // Chunk records written by the row-statistics pass for the gradient pass, which
@@ -2493,20 +2642,23 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
                        stream, P.stats, rows, P.null_logit);
   }
   stage_end(kStageRowStats, stream);
-  constexpr int GP = DVP;
   constexpr int SEG = gradient_segment(DVP);
-  const size_t lds_floats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP +
-                            SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave;
-  // At most 20 KB of dynamic LDS per block: below the 64 KB every kernel may use without
+  constexpr size_t kFixedFloats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch +
+                                  SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave +
+                                  kSignTableWords + kChunk * kRestPitch / 2;
+  // the staged grad_output rows: bfloat16 terms
+  const size_t lds_bytes = kFixedFloats * sizeof(float) +
+                           sizeof(uint16_t) * SEG * (P.grad_pitch + gradient_row_padding(DVP));
+  // At most 27 KB of dynamic LDS per block: below the 64 KB every kernel may use without
   // raising its limit first.  (Raising it would be a configuration call per launch, and
   // those are refused while a stream is being captured into a graph.)
-  static_assert((2 * (SEG / kChunk) * kWave + kChunk * kTilePitch + SEG * GP + SEG * kRowWords +
-                 (SEG + kWave) * (2 + NVW) + SEG + kWave) * sizeof(float) <= 64 * 1024,
-                "dynamic LDS of the gradient kernel");
+  static_assert(kFixedFloats * sizeof(float) +
+                    sizeof(uint16_t) * SEG * (grad_term_pitch(kMaxGradTerms, DVP) + 8) <=
+                64 * 1024, "dynamic LDS of the gradient kernel");
   stage_begin(kStageGradients, stream);
   hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
-                     dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave),
-                     lds_floats * sizeof(float), stream, P);
+                     dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave), lds_bytes,
+                     stream, P);
   stage_end(kStageGradients, stream);
   return 0;
 }
@@ -2562,7 +2714,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     if (value_offset > 0) stage_begin(kStagePrepare, stream);
 
     float4* stats = at<float4>(workspace, w.stats);
-    float* grad_rows = at<float>(workspace, w.grad_rows);
+    uint16_t* grad_rows = at<uint16_t>(workspace, w.grad_rows);
+    const int grad_pitch = grad_term_pitch(view.grad_terms, dvp);
     uint32_t* value_bits = at<uint32_t>(workspace, w.value_bits);
     int32_t* counter = at<int32_t>(workspace, w.header) + 1;
     const bool analytic = analytic_reference_is_safe(L, scale);
@@ -2584,6 +2737,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
       prepare.nvw = nvw;
       prepare.value_stride = full_width;
       prepare.value_offset = value_offset;
+      prepare.grad_terms = view.grad_terms;
+      prepare.grad_pitch = grad_pitch;
       prepare.scale = scale;
       prepare.analytic = analytic ? 1 : 0;
       prepare.ballot = (L.Dv == 8 || L.Dv == 16 || L.Dv == 32 || L.Dv == 64) ? 1 : 0;
@@ -2623,6 +2778,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     P.packed_key = reinterpret_cast<const uint32_t*>(packed_key);
     P.value_bits = value_bits;
     P.grad_rows = grad_rows;
+    P.grad_terms = view.grad_terms;
+    P.grad_pitch = grad_pitch;
     P.stats = stats;
     P.dropout_seed = dropout_seed;
     P.scale = scale;
