@@ -1413,6 +1413,10 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   // without symbol gradients no utilities are computed and the tile stays zero
   for (int index = lane; index < kChunk * kUtilityPitch; index += kWave) utilities[index] = 0.0f;
   fill_sign_table(sign_table, lane);
+  // windows with at least this many mismatching bits at the start of a chunk stay above the
+  // count whose overflow term exp2(-gate_log2 * count) reaches tail_threshold
+  const int quiet_window =
+      static_cast<int>(ceilf(-__log2f(P.tail_threshold) / P.gate_log2)) + kChunk * P.L.D + 1;
   const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row actually present
   const int grad_lds_pitch = P.grad_pitch + 8;
   for (int first = 0; first < view.steps; first += kBlockRows) {
@@ -1501,8 +1505,14 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       }
       uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
       // compiled twice: once every lane is past its window fill no masking is needed
-      auto run_chunk = [&](auto steady_tag) {
+      auto run_chunk = [&](auto steady_tag, auto quiet_tag) {
         constexpr bool STEADY = decltype(steady_tag)::value;
+        // QUIET (steady chunks only): no window of the chunk can get small enough for its
+        // overflow term to reach `tail_threshold`, so the terms are left out (they could not
+        // move a float32 result) and the window counts are only kept up to date: the
+        // entering and the leaving mismatches are summed and applied after the chunk.
+        constexpr bool QUIET = decltype(quiet_tag)::value;
+        uint32_t entering = 0u, leaving = 0u;
         const uint32_t* row = rows + local * kRowWords;
         uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
         float next_shift = __uint_as_float(row[4]);
@@ -1519,9 +1529,22 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           }
           const int i = min(chunk_first + r, last_step);
           const int t = view.diag0 + 1 + i;
-          const StepOut s =
-              forward_step<NVW, STEADY, false, true>(band, symbols, i, lane, W, P.gate_log2);
-          peak_overflow = fmaxf(peak_overflow, s.overflow);
+          StepOut s;
+          if constexpr (QUIET) {
+            band.key_word = dpp_wave_shr1(symbols.key, band.key_word);
+            band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
+            const uint32_t differing = symbols.query ^ band.key_word;
+            const float gate =
+                decay_of_biased_count(__popc(differing) + kCountBias, P.gate_log2);
+            band.evidence = fmaf(gate, band.evidence, gate);
+            entering += __popc(differing);
+            leaving += __popc(symbols.old_query ^ band.old_key_word);
+            s.evidence = band.evidence;
+            s.active = true;
+          } else {
+            s = forward_step<NVW, STEADY, false, true>(band, symbols, i, lane, W, P.gate_log2);
+            peak_overflow = fmaxf(peak_overflow, s.overflow);
+          }
           const float one_plus = 1.0f + s.evidence;
           const float root = one_plus * fast_rsq(one_plus);
           const bool live = STEADY || (s.active && r < rows_here);
@@ -1537,11 +1560,18 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
           weights[r * kWeightPitch + lane] = weight;
           utilities[r * kUtilityPitch + lane] = weight * keep * utility;
         }
+        if constexpr (QUIET) band.window += static_cast<int>(entering - leaving);
       };
       if (chunk_first >= W + kWave && rows_here == kChunk) {
-        run_chunk(std::true_type{});
+        // a window loses at most D mismatches per row
+        const bool quiet = __ballot(window_before < quiet_window) == 0ull;
+        if (quiet) {
+          run_chunk(std::true_type{}, std::true_type{});
+        } else {
+          run_chunk(std::true_type{}, std::false_type{});
+        }
       } else {
-        run_chunk(std::false_type{});
+        run_chunk(std::false_type{}, std::false_type{});
       }
       wave_lds_fence();
       {
