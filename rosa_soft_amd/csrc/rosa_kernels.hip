@@ -26,6 +26,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <type_traits>
 
 #include "../../include/rosa_soft_hip.h"
@@ -113,6 +114,12 @@ __device__ __forceinline__ float dpp_row_shr8(float keep, float src) {
 // __syncthreads() would also wait for every outstanding global store and atomic.
 __device__ __forceinline__ void wave_lds_fence() {
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
+// Meeting point of the waves of a block that exchange data through LDS only: the LDS
+// traffic of the wave is complete, global stores and atomics stay in flight.
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 template <int CTRL, int ROW_MASK>
@@ -727,6 +734,8 @@ struct VjpParams {
   int64_t block_scratch_floats;
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
   int total_units;
+  int wave_lds_floats;          // LDS floats each wave of a gradient block owns
+  int exchange_tile_floats;     // LDS floats of an accumulator tile passed between waves
 };
 
 // Terms of the bfloat16 expansion of a float: x = t0 + t1 + t2 exactly (each term is the
@@ -1654,6 +1663,7 @@ __global__ __launch_bounds__(256) void finalize_row_records_kernel(float4* __res
 // skewed reads of the column sums (k slice lg <-> row step + 4 lg) and of the row sums
 // (row li, stride pitch + 1 = 36 (mod 64)) both touch 64 different LDS banks.
 constexpr int kTilePitch = 99;
+constexpr int kCheckpointChunksMax = 4;  // chunks per staged segment at most
 constexpr int kWindowTiles = 5;  // 80 window columns
 
 // -1.0f where symbol bit `bit` of `word` is set, +1.0f where it is clear: the negated
@@ -1673,34 +1683,80 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
 // rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
 constexpr int gradient_segment(int dvp) { return dvp >= 16 ? 32 : 64; }
 
+// waves per block of the gradient kernel for a tile shape (ROSA_GRADIENT_WAVES overrides)
+int gradient_block_waves(int dvp, int symbol_tiles) {
+  static const int forced = [] {
+    const char* text = getenv("ROSA_GRADIENT_WAVES");
+    return text != nullptr ? atoi(text) : 0;
+  }();
+  if (forced == 1 || forced == 2) return forced;
+  return (dvp >= 16 || symbol_tiles > 1) ? 2 : 1;
+}
+
+// Waves per block of the gradient kernel.  The waves of a block own neighbouring bands of
+// one (sequence, head) and walk them in step: at the same band-local step every band
+// completes the same 16 columns, so the column sums of all bands are added in LDS and leave
+// in one set of global atomics; the rows of a band are the rows its neighbour (64 diagonals
+// further) handles four chunks later, so row sums travel from band to band through a short
+// LDS queue and only the last band adds them to memory.  Global float atomics are bounded
+// by the number of 64-byte row segments they touch (about 21 G segments per second on the
+// whole chip, whatever the number of lanes), which made them the limit of the wide tiles.
+constexpr int kQueueSlots = 5;  // a row tile is read four chunks after it was written
+
+// The queues of row tiles are kept where they fit beside four blocks per compute unit.
+constexpr bool gradient_row_queue(int waves, int value_tiles, int symbol_tiles) {
+  return waves > 1 && value_tiles + symbol_tiles <= 3;
+}
+
+// floats of the shared LDS area of a block before the exchange tiles: window columns and,
+// with several waves, the work index
+constexpr int gradient_shared_fixed_floats(int segment, int value_words_per_column, int waves) {
+  return (segment + kWave) * (2 + value_words_per_column) + (waves > 1 ? 64 : 0);
+}
+
+// floats of a 16 x 16 accumulator tile on its way through LDS (lane (li, lg) owns rows
+// 4 lg .. 4 lg + 3 of column li): all 64 lanes, or the 32 lanes of columns 0 .. 7 when no
+// tile has more than 8 live columns
+constexpr int exchange_tile_floats(bool narrow) { return narrow ? 2 * kWave : 4 * kWave; }
+
 // bfloat16 elements of padding per staged grad_output row (none at the narrowest width,
 // where the block's LDS decides how many blocks a compute unit holds)
 constexpr int gradient_row_padding(int dvp) { return dvp > 8 ? 8 : 0; }
 
 constexpr int kRestPitch = 100;  // 16-bit elements per row of the third-term plane
 
-template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
-__global__ __launch_bounds__(kWave)
+template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT, int NW>
+__global__ __launch_bounds__(kWave * NW)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr bool kFetchAhead = VT == 1 && DT == 1;  // registers to spare for operands in flight
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
-  extern __shared__ float lds[];
-  float* ck_evidence = lds;       // [SEG_CHUNKS][64] (S, window) before each chunk when the
-                                  // row-statistics pass left no records
-  int* ck_window = reinterpret_cast<int*>(lds + SEG_CHUNKS * kWave);
-  float* tile = lds + 2 * SEG_CHUNKS * kWave;                // [kChunk][kTilePitch]
+  extern __shared__ float lds_all[];
+  // LDS: first what the waves of a block share, then one region per wave.  Shared are the
+  // window columns of a segment (every band of the block meets the same columns at the same
+  // band-local step; each wave stores them, with the same values), the work index, the
+  // column tiles on their way to wave 0 and the queues of row tiles.
+  const int wave = NW > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6) : 0;
+  constexpr bool kRowQueue = gradient_row_queue(NW, VT, DT);
+  constexpr int kSharedFixed = gradient_shared_fixed_floats(SEG, NVW, NW);
+  uint32_t* key_window = reinterpret_cast<uint32_t*>(lds_all);  // [SEG + 64] key words of the columns
+  uint32_t* old_key_window = key_window + SEG + kWave;       // [SEG + 64] key words of the columns
+                                                             // W + 1 to the left
+  uint32_t* value_window = old_key_window + SEG + kWave;     // [SEG + 64][NVW] value sign words
+  int* shared_unit = reinterpret_cast<int*>(value_window + (SEG + kWave) * NVW);  // [2] (+ padding)
+  float* lds = lds_all + kSharedFixed + wave * P.wave_lds_floats;  // this wave's own region
+  float* column_exchange = lds_all + kSharedFixed + NW * P.wave_lds_floats;
+                                                    // [NW - 1][VT + DT][exchange_tile_floats]
+  float* row_queue = column_exchange + (NW - 1) * (VT + DT) * P.exchange_tile_floats;
+                                                    // [NW - 1][kQueueSlots][DT][exchange_tile_floats]
+  float* tile = lds;                                         // [kChunk][kTilePitch]
   uint32_t* tile_bits = reinterpret_cast<uint32_t*>(tile);   // the same tile as split operands
   uint32_t* rows = reinterpret_cast<uint32_t*>(tile + kChunk * kTilePitch);  // [SEG][kRowWords]
-  uint32_t* key_window = rows + SEG * kRowWords;             // [SEG + 64] key words of the columns
-  uint32_t* value_window = key_window + SEG + kWave;         // [SEG + 64][NVW] value sign words
-  uint32_t* query_rows = value_window + (SEG + kWave) * NVW; // [SEG] query words of the rows
+  uint32_t* query_rows = rows + SEG * kRowWords;             // [SEG] query words of the rows
   float* discard = reinterpret_cast<float*>(query_rows + SEG); // [64] sink of the utility tile
-  uint32_t* old_key_window = reinterpret_cast<uint32_t*>(discard + kWave);  // [SEG + 64] key words
-                                                             // of the columns W + 1 to the left
-  uint32_t* sign_table = old_key_window + SEG + kWave;       // [kSignTableWords]
+  uint32_t* sign_table = reinterpret_cast<uint32_t*>(discard + kWave);  // [kSignTableWords]
   // third bfloat16 term of the gate adjoints, [kChunk][kRestPitch], same geometry as `tile`
   uint16_t* rest_plane = reinterpret_cast<uint16_t*>(sign_table + kSignTableWords);
   // [SEG][GP] bfloat16 terms of the grad_output rows (GP elements per row: the terms in
@@ -1710,9 +1766,17 @@ void vjp_gradients_kernel(VjpParams P) {
   const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row
   constexpr int kGradChunksMax = grad_term_pitch(kMaxGradTerms, DVP) / 8;
 
-  const int lane = threadIdx.x;
-  const int li = lane & 15;   // MFMA row (A) / column (B, C) index
-  const int lg = lane >> 4;   // MFMA k index (A, B) / row group (C)
+  // The wide tiles have no registers for the many addresses and offsets that derive from
+  // the lane number alone: there the lane number is made opaque once per chunk, so that
+  // they are recomputed where they are used instead of being kept (and spilled) across
+  // the whole kernel.
+  constexpr bool kRecomputeLaneValues = VT > 1 || DT > 1;
+  // completed tiles wait in registers for the next chunk's replay to cover their atomics
+  constexpr bool kFlushAtOnce = false;
+  const int lane_id = threadIdx.x & (kWave - 1);
+  int lane = lane_id;
+  int li = lane & 15;   // MFMA row (A) / column (B, C) index
+  int lg = lane >> 4;   // MFMA k index (A, B) / row group (C)
   const int W = P.L.W;
   const int D = P.L.D;
   const int Dv = P.L.Dv;
@@ -1723,8 +1787,13 @@ void vjp_gradients_kernel(VjpParams P) {
   const float adjoint_gain = 0.5f * kSqrtScale * P.scale;  // scale * U'(S) * sqrt(1 + S)
   // the contractions run on negated symbols
   const float symbol_scale = -0.5f * P.mismatch_scale / static_cast<float>(D);
-  float* ring = P.block_scratch + static_cast<int64_t>(blockIdx.x) * P.block_scratch_floats;
-  float* seg_ck = ring + static_cast<int64_t>(P.ring_rows) * kWave;  // [(S, window)][64] per segment
+  float* ring = P.block_scratch +
+      (static_cast<int64_t>(blockIdx.x) * NW + wave) * P.block_scratch_floats;
+  // without chunk records: (S, window) before every chunk of the current segment, then
+  // before every segment of the band
+  float* ck_evidence = ring + static_cast<int64_t>(P.ring_rows) * kWave;   // [SEG_CHUNKS][64]
+  int* ck_window = reinterpret_cast<int*>(ck_evidence + SEG_CHUNKS * kWave);
+  float* seg_ck = ck_evidence + 2 * kCheckpointChunksMax * kWave;  // [(S, window)][64] per segment
 
   // zero the tile once: its margins are never written again
   for (int index = lane; index < kChunk * kTilePitch; index += kWave) tile[index] = 0.0f;
@@ -1732,16 +1801,35 @@ void vjp_gradients_kernel(VjpParams P) {
   fill_sign_table(sign_table, lane);
   wave_lds_fence();
 
+  int pulls = 0;
   for (;;) {
     int unit_index = 0;
-    if (lane == 0) unit_index = atomicAdd(P.work_counter, 1);
+    if constexpr (NW == 1) {
+      if (lane == 0) unit_index = atomicAdd(P.work_counter, 1);
+    } else {
+      // one pull per block; the two slots alternate, so that a wave that is still reading
+      // the previous index is not overtaken by the next pull
+      if (threadIdx.x == 0) shared_unit[pulls & 1] = atomicAdd(P.work_counter, 1);
+      block_barrier();
+      unit_index = shared_unit[pulls & 1];
+      ++pulls;
+    }
     unit_index = __builtin_amdgcn_readfirstlane(unit_index);
     if (unit_index >= P.total_units) break;
-    const Unit u = decode_unit<VARLEN>(P.L, unit_index);
-    if (!u.valid) continue;
+    // The unit names the first band of the block's group of NW neighbouring bands (the
+    // longest of them); wave w takes band w of the group.  Everything that decides how often
+    // the block meets at a barrier derives from the first band, which all waves know.
+    const Unit lead = decode_unit<VARLEN>(P.L, unit_index);
+    if (!lead.valid) continue;
+    if (NW > 1 && lead.block % NW != 0) continue;
+    const int lead_steps = lead.len - 1 - lead.block * kWave;
+    if (lead_steps <= 0) continue;
+    Unit u = lead;
+    u.block += wave;
     BandView view;
     int hv;
-    if (!make_view<NVW, VARLEN>(P, u, view, hv)) continue;
+    const bool have_band = make_view<NVW, VARLEN>(P, u, view, hv);
+    const int my_steps = have_band ? view.steps : 0;  // a wave without a band only keeps step
     DropoutKey key;
     if constexpr (DROPOUT) {
       key = make_dropout_key(static_cast<uint64_t>(*P.dropout_seed), u.head, u.seq, P.dropout_p);
@@ -1758,12 +1846,13 @@ void vjp_gradients_kernel(VjpParams P) {
       for (int n = 0; n < DT; ++n) key_acc[m][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    const int segments = (view.steps + SEG - 1) / SEG;
+    const int lead_segments = (lead_steps + SEG - 1) / SEG;
+    const int segments = (my_steps + SEG - 1) / SEG;
     Band<NVW> band;
     // Without stored checkpoints, a band-level forward sweep leaves (S, window) before the
     // first row of every segment and a segment-level one before every chunk.
-    const bool stored = view.checkpoints != nullptr;
-    if (!stored && segments > 1) {
+    const bool stored = have_band && view.checkpoints != nullptr;
+    if (have_band && !stored && segments > 1) {
       band.evidence = 0.0f;
       band.window = 0;
       load_sliding<NVW>(band, view, 0, lane, W);
@@ -1787,7 +1876,7 @@ void vjp_gradients_kernel(VjpParams P) {
     float ring_sum = 0.0f;        // sum of b * overflow over the next W + 1 rows
     int ring_live = 0;            // rows for which the ring still holds non-zero terms
     int ring_fresh = 0;           // ring reads that must be treated as zero
-    const int last_step = view.steps - 1;
+    const int last_step = my_steps - 1;
     // The global atomics of a chunk are issued one chunk later, right before the next
     // chunk's replay, so that their latency is covered by arithmetic instead of being
     // waited for at the next chunk's first register reuse.
@@ -1796,6 +1885,11 @@ void vjp_gradients_kernel(VjpParams P) {
     v4f done_query[DT];
     int done_first = -1;  // first step of the chunk whose results are pending (-1: none)
     int done_rows = 0;
+    // which of the pending results this wave adds to memory itself (in a block of several
+    // waves column sums leave through wave 0 and row sums through the last band that holds
+    // the rows)
+    bool done_flush_columns = true;
+    bool done_flush_rows = true;
     // step 0 of the band: row diag0 + 1 (query gradients), column 1 (value gradients, key
     // position 0)
     const uint32_t symbol_stride = static_cast<uint32_t>(P.L.H) * D;
@@ -1845,21 +1939,21 @@ void vjp_gradients_kernel(VjpParams P) {
       float* value_base =
           band_value_base + static_cast<uint64_t>(static_cast<uint32_t>(done_first)) * value_stride;
       const auto add_all = [&](auto full_tag, int rows_left, int columns_left) {
-        if (want_q) {
+        if (want_q && (NW == 1 || done_flush_rows)) {
 #pragma unroll
           for (int n = 0; n < DT; ++n) {
             add_tile(full_tag, query_base + 16 * n, symbol_stride, D - 16 * n, done_query[n],
                      symbol_scale, rows_left);
           }
         }
-        if (want_v) {
+        if (want_v && (NW == 1 || done_flush_columns)) {
 #pragma unroll
           for (int n = 0; n < VT; ++n) {
             add_tile(full_tag, value_base + 16 * n, value_stride, Dv - 16 * n, done_value[n], 1.0f,
                      columns_left);
           }
         }
-        if (want_k) {
+        if (want_k && (NW == 1 || done_flush_columns)) {
 #pragma unroll
           for (int n = 0; n < DT; ++n) {
             add_tile(full_tag, key_base + 16 * n, symbol_stride, D - 16 * n, done_key[n],
@@ -1890,11 +1984,15 @@ void vjp_gradients_kernel(VjpParams P) {
         record_kept = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
       }
     };
-    if (stored) fetch_record((view.steps - 1) / kChunk);
+    if (stored) fetch_record((my_steps - 1) / kChunk);
 
-    for (int segment = segments - 1; segment >= 0; --segment) {
+    for (int segment = lead_segments - 1; segment >= 0; --segment) {
       const int seg_first = segment * SEG;
-      const int seg_last = min(view.steps, seg_first + SEG);
+      const int seg_last = min(my_steps, seg_first + SEG);
+      // chunks of the first band in this segment: the trip count of every wave
+      const int chunks = (min(lead_steps, seg_first + SEG) - seg_first + kChunk - 1) / kChunk;
+      const bool segment_active = NW == 1 || seg_first < my_steps;
+      if (segment_active) {
       if (!stored) {
         if (segments > 1) {
           band.evidence = seg_ck[(2 * segment) * kWave + lane];
@@ -1907,7 +2005,6 @@ void vjp_gradients_kernel(VjpParams P) {
       }
       // one round trip brings in everything the segment needs
       wave_lds_fence();
-      const int chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
       constexpr bool kHeavy = VT > 2 || DT > 1;
       if constexpr (!kHeavy) {
         // Every global load of the segment is issued before the first of them is used, so
@@ -2030,20 +2127,30 @@ void vjp_gradients_kernel(VjpParams P) {
       }
       wave_lds_fence();
       // segment-level forward sweep: checkpoint before every chunk
-      for (int chunk = 0; !stored && chunk < chunks; ++chunk) {
+      const int own_chunks = (seg_last - seg_first + kChunk - 1) / kChunk;
+      for (int chunk = 0; !stored && chunk < own_chunks; ++chunk) {
         ck_evidence[chunk * kWave + lane] = band.evidence;
         ck_window[chunk * kWave + lane] = band.window;
-        if (chunk + 1 < chunks) {
+        if (chunk + 1 < own_chunks) {
           const int local = chunk * kChunk;
           sweep_rows<NVW>(band, rows + local * kRowWords, seg_first + local, kChunk, lane, W,
                           P.gate_log2);
         }
       }
+      }  // segment_active
 
       for (int chunk = chunks - 1; chunk >= 0; --chunk) {
         const int local = chunk * kChunk;               // first row of the chunk inside the segment
         const int first = seg_first + local;            // step index of the chunk's first row
         const int rows_here = min(kChunk, seg_last - first);  // < kChunk only for the band's last rows
+        const bool chunk_active = NW == 1 || first < my_steps;
+        if constexpr (kRecomputeLaneValues) {
+          lane = lane_id;
+          asm volatile("" : "+v"(lane));
+          li = lane & 15;
+          lg = lane >> 4;
+        }
+        if (chunk_active) {
         int window_word;
         uint32_t kept_bits = 0u;  // bit r: row r kept
         if (stored) {
@@ -2052,11 +2159,19 @@ void vjp_gradients_kernel(VjpParams P) {
           band.evidence = record_evidence;
           window_word = record_window;
           kept_bits = record_kept;
+          // the copies are made before the loads set out, so that the loads can land in the
+          // record registers (copies after the loads would wait for them)
+          asm volatile("" : "+v"(band.evidence), "+v"(window_word), "+v"(kept_bits));
           if (first >= kChunk) fetch_record(first / kChunk - 1);
           __builtin_amdgcn_sched_barrier(0);
         } else {
-          band.evidence = ck_evidence[chunk * kWave + lane];
-          window_word = ck_window[chunk * kWave + lane];
+          // (a use inside this branch: the wait for these loads must not end up behind the
+          // branch, where it would also wait for the record loads of the other path)
+          float evidence_in = ck_evidence[chunk * kWave + lane];
+          int window_in = ck_window[chunk * kWave + lane];
+          asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3"
+                       : "=&v"(band.evidence), "=&v"(window_word)
+                       : "v"(evidence_in), "v"(window_in));
         }
         band.window = window_word & INT32_MAX;
         // stored records say whether any overflow term of the chunk matters
@@ -2358,8 +2473,6 @@ void vjp_gradients_kernel(VjpParams P) {
         for (int n = 0; n < DT; ++n) done_key[n] = key_acc[kWindowTiles - 1][n];
         done_first = first;
         done_rows = rows_here;
-        // wide tiles have no registers to spare for carrying the results across a chunk
-        if constexpr (VT > 1 || DT > 1) issue_pending();
 #pragma unroll
         for (int m = kWindowTiles - 1; m > 0; --m) {
 #pragma unroll
@@ -2372,6 +2485,97 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
         for (int n = 0; n < DT; ++n) key_acc[0][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         wave_lds_fence();
+        }  // chunk_active
+
+        if constexpr (NW > 1) {
+          // Every band of the block has just completed the same 16 columns (same band-local
+          // step) and, of its rows, a tile that the next band meets four chunks from now.
+          const int g = first / kChunk;
+          const int tile_floats = P.exchange_tile_floats;
+          // a tile in LDS: 16 bytes per lane, only the lanes of columns 0 .. 7 when narrow
+          const bool narrow_tiles = tile_floats == exchange_tile_floats(true);
+          const bool tile_lane = !narrow_tiles || li < 8;
+          const int tile_offset = narrow_tiles ? 4 * (8 * lg + (li & 7)) : 4 * lane;
+          if (chunk_active) {
+            done_flush_columns = wave == 0;
+            done_flush_rows = true;
+            if constexpr (kRowQueue) {
+              if (want_q) {
+                if (wave > 0 && tile_lane) {  // what the band before this one summed over these rows
+                  const float* slot = row_queue +
+                      (((wave - 1) * kQueueSlots + (g + 4) % kQueueSlots) * DT) * tile_floats +
+                      tile_offset;
+#pragma unroll
+                  for (int n = 0; n < DT; ++n) {
+                    done_query[n] += *reinterpret_cast<const v4f*>(slot + n * tile_floats);
+                  }
+                }
+                // rows above the first row of the next band (its chunks 0 .. 3 of this band)
+                // and the rows of the block's last band go to memory from here
+                if (wave + 1 < NW && g >= 4 && lead_steps - (wave + 1) * kWave > 0) {
+                  float* slot = row_queue +
+                      ((wave * kQueueSlots + g % kQueueSlots) * DT) * tile_floats + tile_offset;
+                  if (tile_lane) {
+#pragma unroll
+                    for (int n = 0; n < DT; ++n) {
+                      *reinterpret_cast<v4f*>(slot + n * tile_floats) = done_query[n];
+                    }
+                  }
+                  done_flush_rows = false;
+                }
+              }
+            }
+            if (wave > 0 && tile_lane) {
+              float* out = column_exchange + ((wave - 1) * (VT + DT)) * tile_floats + tile_offset;
+              if (want_v) {
+#pragma unroll
+                for (int n = 0; n < VT; ++n) {
+                  *reinterpret_cast<v4f*>(out + n * tile_floats) = done_value[n];
+                }
+              }
+              if (want_k) {
+#pragma unroll
+                for (int n = 0; n < DT; ++n) {
+                  *reinterpret_cast<v4f*>(out + (VT + n) * tile_floats) = done_key[n];
+                }
+              }
+            }
+          }
+          block_barrier();
+          if (wave == 0 && chunk_active && tile_lane) {
+            for (int other = 1; other < NW; ++other) {
+              if (first >= lead_steps - other * kWave) break;  // shorter bands have no such chunk
+              const float* in =
+                  column_exchange + ((other - 1) * (VT + DT)) * tile_floats + tile_offset;
+              if (want_v) {
+#pragma unroll
+                for (int n = 0; n < VT; ++n) {
+                  done_value[n] += *reinterpret_cast<const v4f*>(in + n * tile_floats);
+                }
+              }
+              if (want_k) {
+#pragma unroll
+                for (int n = 0; n < DT; ++n) {
+                  done_key[n] += *reinterpret_cast<const v4f*>(in + (VT + n) * tile_floats);
+                }
+              }
+            }
+          }
+          // the column tiles have been taken over: the other waves may store their next ones
+          block_barrier();
+        }
+        // wide tiles have no registers to spare for carrying the results across a chunk
+        if constexpr (kFlushAtOnce) {
+          if (chunk_active) {
+            // The record of the next chunk has been on its way for a whole chunk: it is
+            // taken in now, so that the next chunk does not wait for it behind the atomics
+            // issued here (memory operations of a wave are counted in order).
+            if (stored) {
+              asm volatile("" : : "v"(record_evidence), "v"(record_window), "v"(record_kept));
+            }
+            issue_pending();
+          }
+        }
       }
     }
     issue_pending();
@@ -2548,10 +2752,12 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.ring_rows = std::min(v.L.W, longest) + 1;
   const int segment_rows = gradient_segment(dvp);
   const int max_segments = (longest + segment_rows - 1) / segment_rows + 1;
-  w.block_scratch_floats =
-      static_cast<int64_t>(w.ring_rows) * kWave + static_cast<int64_t>(max_segments) * 2 * kWave;
+  w.block_scratch_floats = static_cast<int64_t>(w.ring_rows) * kWave +
+                           2 * kCheckpointChunksMax * kWave +
+                           static_cast<int64_t>(max_segments) * 2 * kWave;
   const int64_t units = static_cast<int64_t>(v.L.slots) * v.L.H;
-  w.resident_blocks = static_cast<int>(std::min<int64_t>(units, kMaxResidentBlocks));
+  // resident waves of the gradient kernel (an even number: its blocks hold one or two waves)
+  w.resident_blocks = static_cast<int>(std::min<int64_t>((units + 1) & ~int64_t(1), kMaxResidentBlocks));
   // keep the scratch pool below 2 GiB by running fewer resident blocks for huge windows
   const int64_t budget_floats = (int64_t(1) << 31) / 4;
   while (w.resident_blocks > 64 &&
@@ -2673,22 +2879,46 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   }
   stage_end(kStageRowStats, stream);
   constexpr int SEG = gradient_segment(DVP);
-  constexpr size_t kFixedFloats = 2 * (SEG / kChunk) * kWave + kChunk * kTilePitch +
-                                  SEG * kRowWords + (SEG + kWave) * (2 + NVW) + SEG + kWave +
+  constexpr int VT = (DVP + 15) / 16;
+  // per wave: tile, row words, query words, sink, sign table, third-term plane and the
+  // staged grad_output rows (bfloat16 terms), in whole 16-byte units
+  constexpr size_t kFixedFloats = kChunk * kTilePitch + SEG * kRowWords + SEG + kWave +
                                   kSignTableWords + kChunk * kRestPitch / 2;
-  // the staged grad_output rows: bfloat16 terms
-  const size_t lds_bytes = kFixedFloats * sizeof(float) +
-                           sizeof(uint16_t) * SEG * (P.grad_pitch + gradient_row_padding(DVP));
-  // At most 27 KB of dynamic LDS per block: below the 64 KB every kernel may use without
-  // raising its limit first.  (Raising it would be a configuration call per launch, and
-  // those are refused while a stream is being captured into a graph.)
-  static_assert(kFixedFloats * sizeof(float) +
-                    sizeof(uint16_t) * SEG * (grad_term_pitch(kMaxGradTerms, DVP) + 8) <=
-                64 * 1024, "dynamic LDS of the gradient kernel");
+  const size_t wave_floats =
+      (kFixedFloats + (SEG * (P.grad_pitch + gradient_row_padding(DVP)) + 1) / 2 + 3) / 4 * 4;
+  const bool narrow_tiles = DVP == 8 && P.L.D <= 8;
+  const size_t tile_floats = exchange_tile_floats(narrow_tiles);
   stage_begin(kStageGradients, stream);
-  hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT>),
-                     dim3(static_cast<unsigned>(w.resident_blocks)), dim3(kWave), lds_bytes,
-                     stream, P);
+  const auto launch = [&](auto waves_tag) {
+    constexpr int NW = decltype(waves_tag)::value;
+    // shared by the waves of a block: window columns, work index, column tiles on their way
+    // to wave 0, row tile queues
+    const size_t shared_floats =
+        gradient_shared_fixed_floats(SEG, NVW, NW) +
+        (NW - 1) * ((VT + DT) + (gradient_row_queue(NW, VT, DT) ? kQueueSlots * DT : 0)) * tile_floats;
+    // At most 64 KB of dynamic LDS per block: what every kernel may use without raising its
+    // limit first.  (Raising it would be a configuration call per launch, and those are
+    // refused while a stream is being captured into a graph.)
+    constexpr size_t kWaveFloatsMax =
+        (kFixedFloats + SEG * (grad_term_pitch(kMaxGradTerms, DVP) + 8) / 2 + 3) / 4 * 4;
+    static_assert(NW > 1 || (kWaveFloatsMax + gradient_shared_fixed_floats(SEG, NVW, 1)) *
+                                    sizeof(float) <= 64 * 1024,
+                  "dynamic LDS of the gradient kernel");
+    VjpParams Q = P;
+    Q.wave_lds_floats = static_cast<int>(wave_floats);
+    Q.exchange_tile_floats = static_cast<int>(tile_floats);
+    const size_t lds_bytes = (NW * wave_floats + shared_floats) * sizeof(float);
+    if (lds_bytes > 64 * 1024) return false;
+    const unsigned blocks = static_cast<unsigned>(std::max(1, w.resident_blocks / NW));
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, NW>), dim3(blocks),
+                       dim3(kWave * NW), lds_bytes, stream, Q);
+    return true;
+  };
+  // two waves per block where that fits the LDS of a block (float32 rows of the widest
+  // tile do not)
+  if (gradient_block_waves(DVP, DT) != 2 || !launch(std::integral_constant<int, 2>{})) {
+    launch(std::integral_constant<int, 1>{});
+  }
   stage_end(kStageGradients, stream);
   return 0;
 }
