@@ -1683,14 +1683,20 @@ constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
 // rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
 constexpr int gradient_segment(int dvp) { return dvp >= 16 ? 32 : 64; }
 
-// waves per block of the gradient kernel for a tile shape (ROSA_GRADIENT_WAVES overrides)
-int gradient_block_waves(int dvp, int symbol_tiles) {
+// resident waves of the persistent gradient kernel: two per SIMD of the 256 compute units
+constexpr int kMaxResidentBlocks = 2048;
+
+// Waves per block of the gradient kernel (ROSA_GRADIENT_WAVES overrides, for measurements).
+// Two waves halve the column atomics, which bound the wide tiles; the narrow tile is bound
+// by its arithmetic, and with few bands per resident wave the kernel's time is that of
+// its longest band, which a block of two waves walks more slowly than a single wave.
+int gradient_block_waves(int dvp, int symbol_tiles, int64_t units) {
   static const int forced = [] {
     const char* text = getenv("ROSA_GRADIENT_WAVES");
     return text != nullptr ? atoi(text) : 0;
   }();
   if (forced == 1 || forced == 2) return forced;
-  return (dvp >= 16 || symbol_tiles > 1) ? 2 : 1;
+  return ((dvp >= 16 || symbol_tiles > 1) && units >= 2 * kMaxResidentBlocks) ? 2 : 1;
 }
 
 // Waves per block of the gradient kernel.  The waves of a block own neighbouring bands of
@@ -1730,7 +1736,7 @@ __global__ __launch_bounds__(kWave * NW)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
-  constexpr bool kFetchAhead = VT == 1 && DT == 1;  // registers to spare for operands in flight
+  constexpr bool kFetchAhead = true;  // row words and operands are fetched ahead of their use
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
   constexpr int SEG_CHUNKS = SEG / kChunk;
   extern __shared__ float lds_all[];
@@ -2713,7 +2719,6 @@ struct VjpWorkspace {
   int ring_rows;
 };
 
-constexpr int kMaxResidentBlocks = 2048;
 
 VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   VjpWorkspace w;
@@ -2916,7 +2921,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   };
   // two waves per block where that fits the LDS of a block (float32 rows of the widest
   // tile do not)
-  if (gradient_block_waves(DVP, DT) != 2 || !launch(std::integral_constant<int, 2>{})) {
+  if (gradient_block_waves(DVP, DT, P.total_units) != 2 || !launch(std::integral_constant<int, 2>{})) {
     launch(std::integral_constant<int, 1>{});
   }
   stage_end(kStageGradients, stream);
