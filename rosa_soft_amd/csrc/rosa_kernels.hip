@@ -752,6 +752,7 @@ struct VjpParams {
   int total_units;
   int wave_lds_floats;          // LDS floats each wave of a gradient block owns
   int exchange_tile_floats;     // LDS floats of an accumulator tile passed between waves
+  int row_queue;                // row tiles travel from band to band through LDS (two-wave blocks)
 };
 
 // Terms of the bfloat16 expansion of a float: x = t0 + t1 + t2 exactly (each term is the
@@ -1730,12 +1731,13 @@ int gradient_block_waves(int dvp, int symbol_tiles, int64_t units) {
 // LDS queue and only the last band adds them to memory.  Global float atomics are bounded
 // by the number of 64-byte row segments they touch (about 21 G segments per second on the
 // whole chip, whatever the number of lanes), which made them the limit of the wide tiles.
-constexpr int kQueueSlots = 5;  // a row tile is read four chunks after it was written
+constexpr int kQueueSlots = 4;  // a row tile is read four chunks after it was written: the
+                                // reader takes it before the barrier, the writer refills the
+                                // slot behind the barrier
 
-// The queues of row tiles are kept where they fit beside four blocks per compute unit.
-constexpr bool gradient_row_queue(int waves, int value_tiles, int symbol_tiles) {
-  return waves > 1 && value_tiles + symbol_tiles <= 3;
-}
+// LDS bytes of a block of the gradient kernel up to which four blocks share a compute unit;
+// the queues of row tiles are kept where the block stays within them
+constexpr size_t kGradientBlockLdsBudget = 40 * 1024;
 
 // floats of the shared LDS area of a block before the exchange tiles: window columns and,
 // with several waves, the work index
@@ -1758,6 +1760,7 @@ template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT, int NW>
 __global__ __launch_bounds__(kWave * NW)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
+  static_assert(NW == 1 || NW == 2, "blocks of one or two waves");
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr bool kFetchAhead = true;  // row words and operands are fetched ahead of their use
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
@@ -1768,7 +1771,7 @@ void vjp_gradients_kernel(VjpParams P) {
   // band-local step; each wave stores them, with the same values), the work index, the
   // column tiles on their way to wave 0 and the queues of row tiles.
   const int wave = NW > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6) : 0;
-  constexpr bool kRowQueue = gradient_row_queue(NW, VT, DT);
+  const bool row_queue_on = NW > 1 && P.row_queue != 0;
   constexpr int kSharedFixed = gradient_shared_fixed_floats(SEG, NVW, NW);
   uint32_t* key_window = reinterpret_cast<uint32_t*>(lds_all);  // [SEG + 64] key words of the columns
   uint32_t* old_key_window = key_window + SEG + kWave;       // [SEG + 64] key words of the columns
@@ -1916,10 +1919,11 @@ void vjp_gradients_kernel(VjpParams P) {
     v4f done_query[DT];
     int done_first = -1;  // first step of the chunk whose results are pending (-1: none)
     int done_rows = 0;
-    // which of the pending results this wave adds to memory itself (in a block of several
-    // waves column sums leave through wave 0 and row sums through the last band that holds
-    // the rows)
-    bool done_flush_columns = true;
+    // which of the pending results this wave adds to memory itself (in a block of two waves
+    // the value column sums leave through wave 0, the key column sums through wave 1, and
+    // row sums through the last band that holds the rows)
+    bool done_flush_value = true;
+    bool done_flush_key = true;
     bool done_flush_rows = true;
     // step 0 of the band: row diag0 + 1 (query gradients), column 1 (value gradients, key
     // position 0)
@@ -1977,14 +1981,14 @@ void vjp_gradients_kernel(VjpParams P) {
                      symbol_scale, rows_left);
           }
         }
-        if (want_v && (NW == 1 || done_flush_columns)) {
+        if (want_v && (NW == 1 || done_flush_value)) {
 #pragma unroll
           for (int n = 0; n < VT; ++n) {
             add_tile(full_tag, value_base + 16 * n, value_stride, Dv - 16 * n, done_value[n], 1.0f,
                      columns_left);
           }
         }
-        if (want_k && (NW == 1 || done_flush_columns)) {
+        if (want_k && (NW == 1 || done_flush_key)) {
 #pragma unroll
           for (int n = 0; n < DT; ++n) {
             add_tile(full_tag, key_base + 16 * n, symbol_stride, D - 16 * n, done_key[n],
@@ -2531,43 +2535,33 @@ void vjp_gradients_kernel(VjpParams P) {
           const bool tile_lane = !narrow_tiles || li < 8;
           const int tile_offset = narrow_tiles ? 4 * (8 * lg + (li & 7)) : 4 * lane;
           if (chunk_active) {
-            done_flush_columns = wave == 0;
+            // both waves have this chunk: each takes over one kind of column sums
+            const bool both = first < lead_steps - kWave;
+            done_flush_value = wave == 0;
+            done_flush_key = wave == 1 || !both;
             done_flush_rows = true;
-            if constexpr (kRowQueue) {
-              if (want_q) {
-                if (wave > 0 && tile_lane) {  // what the band before this one summed over these rows
-                  const float* slot = row_queue +
-                      (((wave - 1) * kQueueSlots + (g + 4) % kQueueSlots) * DT) * tile_floats +
-                      tile_offset;
+            if (row_queue_on && want_q) {
+              if (wave == 1 && tile_lane) {  // what band 0 summed over these rows, four chunks ago
+                const float* slot = row_queue + ((g % kQueueSlots) * DT) * tile_floats + tile_offset;
 #pragma unroll
-                  for (int n = 0; n < DT; ++n) {
-                    done_query[n] += *reinterpret_cast<const v4f*>(slot + n * tile_floats);
-                  }
-                }
-                // rows above the first row of the next band (its chunks 0 .. 3 of this band)
-                // and the rows of the block's last band go to memory from here
-                if (wave + 1 < NW && g >= 4 && lead_steps - (wave + 1) * kWave > 0) {
-                  float* slot = row_queue +
-                      ((wave * kQueueSlots + g % kQueueSlots) * DT) * tile_floats + tile_offset;
-                  if (tile_lane) {
-#pragma unroll
-                    for (int n = 0; n < DT; ++n) {
-                      *reinterpret_cast<v4f*>(slot + n * tile_floats) = done_query[n];
-                    }
-                  }
-                  done_flush_rows = false;
+                for (int n = 0; n < DT; ++n) {
+                  done_query[n] += *reinterpret_cast<const v4f*>(slot + n * tile_floats);
                 }
               }
+              // Rows above the first row of band 1 (chunks 0 .. 3 of band 0) and the rows of
+              // band 1 go to memory from here; the others wait in the queue for band 1.
+              if (wave == 0 && g >= 4 && lead_steps - kWave > 0) done_flush_rows = false;
             }
-            if (wave > 0 && tile_lane) {
-              float* out = column_exchange + ((wave - 1) * (VT + DT)) * tile_floats + tile_offset;
-              if (want_v) {
+            // value tiles of wave 1 go to wave 0, key tiles of wave 0 to wave 1
+            if (both && tile_lane) {
+              float* out = column_exchange + tile_offset;
+              if (wave == 1 && want_v) {
 #pragma unroll
                 for (int n = 0; n < VT; ++n) {
                   *reinterpret_cast<v4f*>(out + n * tile_floats) = done_value[n];
                 }
               }
-              if (want_k) {
+              if (wave == 0 && want_k) {
 #pragma unroll
                 for (int n = 0; n < DT; ++n) {
                   *reinterpret_cast<v4f*>(out + (VT + n) * tile_floats) = done_key[n];
@@ -2576,26 +2570,30 @@ void vjp_gradients_kernel(VjpParams P) {
             }
           }
           block_barrier();
-          if (wave == 0 && chunk_active && tile_lane) {
-            for (int other = 1; other < NW; ++other) {
-              if (first >= lead_steps - other * kWave) break;  // shorter bands have no such chunk
-              const float* in =
-                  column_exchange + ((other - 1) * (VT + DT)) * tile_floats + tile_offset;
-              if (want_v) {
+          if (row_queue_on && want_q && wave == 0 && chunk_active && !done_flush_rows && tile_lane) {
+            // band 1 has taken the slot's old tile in front of the barrier
+            float* slot = row_queue + ((g % kQueueSlots) * DT) * tile_floats + tile_offset;
 #pragma unroll
-                for (int n = 0; n < VT; ++n) {
-                  done_value[n] += *reinterpret_cast<const v4f*>(in + n * tile_floats);
-                }
+            for (int n = 0; n < DT; ++n) {
+              *reinterpret_cast<v4f*>(slot + n * tile_floats) = done_query[n];
+            }
+          }
+          if (chunk_active && tile_lane && first < lead_steps - kWave) {
+            const float* in = column_exchange + tile_offset;
+            if (wave == 0 && want_v) {
+#pragma unroll
+              for (int n = 0; n < VT; ++n) {
+                done_value[n] += *reinterpret_cast<const v4f*>(in + n * tile_floats);
               }
-              if (want_k) {
+            }
+            if (wave == 1 && want_k) {
 #pragma unroll
-                for (int n = 0; n < DT; ++n) {
-                  done_key[n] += *reinterpret_cast<const v4f*>(in + (VT + n) * tile_floats);
-                }
+              for (int n = 0; n < DT; ++n) {
+                done_key[n] += *reinterpret_cast<const v4f*>(in + (VT + n) * tile_floats);
               }
             }
           }
-          // the column tiles have been taken over: the other waves may store their next ones
+          // the column tiles have been taken over: the waves may store their next ones
           block_barrier();
         }
         // wide tiles have no registers to spare for carrying the results across a chunk
@@ -2926,9 +2924,12 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
     constexpr int NW = decltype(waves_tag)::value;
     // shared by the waves of a block: window columns, work index, column tiles on their way
     // to wave 0, row tile queues
-    const size_t shared_floats =
-        gradient_shared_fixed_floats(SEG, NVW, NW) +
-        (NW - 1) * ((VT + DT) + (gradient_row_queue(NW, VT, DT) ? kQueueSlots * DT : 0)) * tile_floats;
+    size_t shared_floats =
+        gradient_shared_fixed_floats(SEG, NVW, NW) + (NW - 1) * (VT + DT) * tile_floats;
+    const size_t queue_floats = (NW - 1) * kQueueSlots * DT * tile_floats;
+    const bool row_queue = NW > 1 && (NW * wave_floats + shared_floats + queue_floats) *
+                                             sizeof(float) <= kGradientBlockLdsBudget;
+    if (row_queue) shared_floats += queue_floats;
     // At most 64 KB of dynamic LDS per block: what every kernel may use without raising its
     // limit first.  (Raising it would be a configuration call per launch, and those are
     // refused while a stream is being captured into a graph.)
@@ -2940,6 +2941,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
     VjpParams Q = P;
     Q.wave_lds_floats = static_cast<int>(wave_floats);
     Q.exchange_tile_floats = static_cast<int>(tile_floats);
+    Q.row_queue = row_queue ? 1 : 0;
     const size_t lds_bytes = (NW * wave_floats + shared_floats) * sizeof(float);
     if (lds_bytes > 64 * 1024) return false;
     const unsigned blocks = static_cast<unsigned>(std::max(1, w.resident_blocks / NW));
