@@ -73,6 +73,15 @@ size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_ma
 void rosa_hip_set_record_budget(size_t bytes);
 
 /*
+ * Waves per block of the backward's gradient kernel: 1, 2, or 0 for the library's choice by
+ * shape (the default).  With two waves the blocks own pairs of neighbouring diagonal bands
+ * and add their column sums in LDS before the global atomics.  The reference has no
+ * counterpart (one block per row there); the knob exists for measurements and so that
+ * tests can run both forms on small problems.
+ */
+void rosa_hip_set_gradient_block_waves(int waves);
+
+/*
  * Exact hard forward.  Replaces hard_forward_cuda (rosa_soft_kernels.cu:1766-1834)
  * and hard_forward_varlen_cuda (:1837-1920): sign-packs query and key into
  * head-major int32 words (dense [B,H,T], packed [H,N]), finds the

@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_forward_workspace_bytes",
     "rosa_hip_vjp_workspace_bytes",
     "rosa_hip_set_record_budget",
+    "rosa_hip_set_gradient_block_waves",
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_hard_forward_bits",
@@ -114,6 +115,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_vjp_workspace_bytes.argtypes = [
         problem_p, ctypes.c_int, ctypes.c_float, ctypes.c_int,
     ]
+    library.rosa_hip_set_gradient_block_waves.restype = None
+    library.rosa_hip_set_gradient_block_waves.argtypes = [ctypes.c_int]
     library.rosa_hip_set_record_budget.restype = None
     library.rosa_hip_set_record_budget.argtypes = [ctypes.c_size_t]
     library.rosa_hip_hard_forward.restype = ctypes.c_int
@@ -467,6 +470,12 @@ def set_record_budget(limit_bytes: Optional[int]) -> None:
 
     load().rosa_hip_set_record_budget(ctypes.c_size_t(-1).value if limit_bytes is None
                                       else int(limit_bytes))
+
+
+def set_gradient_block_waves(waves: Optional[int]) -> None:
+    """Waves per block of the gradient kernel: 1, 2, or ``None`` for the library's choice."""
+
+    load().rosa_hip_set_gradient_block_waves(0 if waves is None else int(waves))
 
 
 def stage_timing(enable: bool) -> None:

@@ -26,7 +26,6 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
-#include <cstdlib>
 #include <type_traits>
 
 #include "../../include/rosa_soft_hip.h"
@@ -1710,16 +1709,14 @@ constexpr int gradient_segment(int dvp) { return dvp >= 16 ? 32 : 64; }
 // resident waves of the persistent gradient kernel: two per SIMD of the 256 compute units
 constexpr int kMaxResidentBlocks = 2048;
 
-// Waves per block of the gradient kernel (ROSA_GRADIENT_WAVES overrides, for measurements).
+// Waves per block of the gradient kernel (rosa_hip_set_gradient_block_waves overrides).
 // Two waves halve the column atomics, which bound the wide tiles; the narrow tile is bound
 // by its arithmetic, and with few bands per resident wave the kernel's time is that of
 // its longest band, which a block of two waves walks more slowly than a single wave.
+int g_gradient_block_waves = 0;  // 0: by shape
+
 int gradient_block_waves(int dvp, int symbol_tiles, int64_t units) {
-  static const int forced = [] {
-    const char* text = getenv("ROSA_GRADIENT_WAVES");
-    return text != nullptr ? atoi(text) : 0;
-  }();
-  if (forced == 1 || forced == 2) return forced;
+  if (g_gradient_block_waves == 1 || g_gradient_block_waves == 2) return g_gradient_block_waves;
   return ((dvp >= 16 || symbol_tiles > 1) && units >= 2 * kMaxResidentBlocks) ? 2 : 1;
 }
 
@@ -3551,6 +3548,10 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "router launch");
   return 0;
+}
+
+void rosa_hip_set_gradient_block_waves(int waves) {
+  g_gradient_block_waves = (waves == 1 || waves == 2) ? waves : 0;
 }
 
 void rosa_hip_set_record_budget(size_t bytes) {

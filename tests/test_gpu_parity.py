@@ -34,6 +34,16 @@ def cabi():
     return module
 
 
+@pytest.fixture(params=[None, 2], ids=["waves_by_shape", "two_wave_blocks"])
+def block_waves(request, cabi):
+    """Both forms of the gradient kernel: the library's choice (one wave per block at these
+    sizes) and blocks of two waves that own neighbouring bands and exchange tiles in LDS."""
+
+    cabi.set_gradient_block_waves(request.param)
+    yield request.param
+    cabi.set_gradient_block_waves(None)
+
+
 def assert_gradients_close(got, want, label="", slack=1.0):
     got = got.detach().cpu().double()
     want = want.double()
@@ -169,8 +179,8 @@ def test_hard_forward_beyond_65535_rows_uses_the_64_bit_key(cabi, c_oracle):
 
 
 @pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,scale,p,ms,dtype,pattern", VJP_CASES)
-def test_surrogate_vjp_matches_oracle(cabi, c_oracle, B, T, H, D, Hv, Dv, W, scale, p, ms, dtype,
-                                      pattern):
+def test_surrogate_vjp_matches_oracle(cabi, c_oracle, block_waves, B, T, H, D, Hv, Dv, W, scale,
+                                      p, ms, dtype, pattern):
     query, key, value, grad_output = make_case(B, T, H, D, Hv, Dv, dtype, seed=7 * T + D, pattern=pattern)
     seed = 0x5DEECE66D1234567 if p > 0 else None
     out, _, _, _, grads = run_device(cabi, query, key, value, grad_output, W, scale, p, ms, seed)
@@ -196,7 +206,7 @@ def test_surrogate_vjp_matches_oracle(cabi, c_oracle, B, T, H, D, Hv, Dv, W, sca
 
 
 @pytest.mark.parametrize("mask", range(1, 8))
-def test_gradient_masks(cabi, c_oracle, mask):
+def test_gradient_masks(cabi, c_oracle, block_waves, mask):
     # reference tests/test_soft_cuda.py:510-567
     query, key, value, grad_output = make_case(1, 70, 2, 5, 1, 6, seed=mask)
     seed = 4242 + mask
@@ -247,7 +257,8 @@ PACKED_CASES = [
 
 
 @pytest.mark.parametrize("lengths,H,D,Hv,Dv,W,p,dtype", PACKED_CASES)
-def test_packed_layout_matches_oracle(cabi, c_oracle, lengths, H, D, Hv, Dv, W, p, dtype):
+def test_packed_layout_matches_oracle(cabi, c_oracle, block_waves, lengths, H, D, Hv, Dv, W, p,
+                                      dtype):
     # reference tests/test_soft_varlen.py:42-141, :392-475, :860-915
     offsets = [0, *np.cumsum(lengths).tolist()]
     total = offsets[-1]
@@ -538,7 +549,7 @@ def test_selected_routes_of_a_packed_batch(cabi, c_oracle):
     (1, 0, 2, 3, 2, 5, 16, 0.1, "random", [70, 0, 1, 300, 129]),
 ])
 def test_backward_without_chunk_records_recomputes_to_the_same_gradients(
-        cabi, c_oracle, B, T, H, D, Hv, Dv, W, p, pattern, lengths):
+        cabi, c_oracle, block_waves, B, T, H, D, Hv, Dv, W, p, pattern, lengths):
     # with the records forbidden the gradient pass sweeps forward again and hashes again
     seed = 99 if p > 0 else None
     if lengths is None:

@@ -3,7 +3,8 @@
 The hand-picked cases of test_gpu_parity.py name the code paths; this sweep crosses
 them (symbol and value widths on both sides of the 8/16/32/64 tile limits, lengths around
 the 16-row chunk and 64-row segment sizes, windows shorter and longer than the sequence,
-dropout, gradient masks, packed layouts with empty sequences, the three dtypes), with the
+dropout, gradient masks, packed layouts with empty sequences, the three dtypes, one- and
+two-wave blocks of the gradient kernel), with the
 same bars: routes and outputs bit-exact, gradients to
 ``|got - want| <= 1e-4 |want| + 1e-5 max|want|``, widened only when the logits themselves
 are large (scale * L > 40, L = scale * U(min(W, T)); about 5x in this sweep, for
@@ -99,5 +100,12 @@ def check_case(cabi, c_oracle, rng, index, c):
 ])
 def test_random_shapes_and_controls_match_the_oracle(cabi, c_oracle, seed, cases, lengths):
     rng = random.Random(seed)
-    for index in range(cases):
-        check_case(cabi, c_oracle, rng, index, draw_case(rng, lengths))
+    try:
+        for index in range(cases):
+            # every other case runs the gradient kernel with two-wave blocks (pairs of
+            # neighbouring bands that exchange tiles through LDS), which the library would
+            # only choose for much larger problems
+            cabi.set_gradient_block_waves(2 if index % 2 else None)
+            check_case(cabi, c_oracle, rng, index, draw_case(rng, lengths))
+    finally:
+        cabi.set_gradient_block_waves(None)
