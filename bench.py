@@ -240,10 +240,12 @@ def measure_workload(name: str, steps: int, warmup: int) -> dict:
             forward()
         torch.cuda.synchronize()
         forward_ms = 1e3 * (time.perf_counter() - begin) / steps
+    plan = cabi.gradient_block_plan(query, value, config["W"], cu_seqlens)
     return dict(
         name=name, config=config, steps=steps, warmup=warmup,
         ms_per_step=1e3 * elapsed / steps, forward_ms=forward_ms,
         stage_ms={stage: total / steps for stage, total in stage_totals.items()},
+        gradient_block_plan=plan,
     )
 
 
@@ -279,6 +281,34 @@ def roofline_fractions(measured: dict) -> dict:
     return out
 
 
+def atomic_row_segments(config, plan: dict) -> int:
+    """64-byte row segments the float atomics of one gradient-kernel launch touch.
+
+    Global float atomics are bounded by the row segments they touch, not by their number
+    (`rosa_hip_measure_atomic_rate`).  A band of 64 diagonals with n rows adds n completed
+    rows of dQ and n completed columns of dK and dV to memory, a row or column of w floats
+    being ceil(4 w / 64) segments; a block of two waves adds the columns of its two bands
+    once, and with the row queue also the rows they share.
+    """
+
+    lengths = config.get("lengths") or [config["T"]] * config["B"]
+    D, Dv = config["D"], config["Dv"]
+    symbol_segments = -(-4 * D // 64)
+    value_segments = sum(-(-4 * min(64, Dv - first) // 64) for first in range(0, Dv, 64))
+    rows = columns = 0
+    for length in lengths:
+        steps = [length - 1 - 64 * band for band in range((length + 63) // 64)]
+        steps = [n for n in steps if n > 0]
+        if plan["waves"] == 2:
+            leads = steps[0::2]
+            columns += sum(leads)
+            rows += sum(leads) if plan["row_queue"] else sum(steps)
+        else:
+            columns += sum(steps)
+            rows += sum(steps)
+    return config["H"] * (columns * (symbol_segments + value_segments) + rows * symbol_segments)
+
+
 def config_summary(measured: dict) -> dict:
     config = measured["config"]
     tokens = token_count(config)
@@ -294,6 +324,8 @@ def config_summary(measured: dict) -> dict:
         vjp_row_stats_ms=round(measured["stage_ms"].get("vjp_row_stats", float("nan")), 4),
         vjp_gradients_frac=round(fractions.get("vjp_gradients", {}).get("frac", float("nan")), 4),
         whole_backward_frac=round(fractions.get("whole_backward", {}).get("frac", float("nan")), 4),
+        waves_per_block=measured["gradient_block_plan"]["waves"],
+        atomic_row_segments=atomic_row_segments(config, measured["gradient_block_plan"]),
     )
 
 
@@ -362,6 +394,24 @@ def training_record(args) -> dict:
     }
     if figures:
         roofline["issue"] = {k: v for k, v in figures.items() if k != "traffic_bytes_per_launch"}
+    # the other bound of the gradient kernel: its global float atomics, priced against the
+    # rate measured on this GPU in this run
+    from rosa_soft_amd import cabi
+
+    plan = measured["gradient_block_plan"]
+    segments = atomic_row_segments(config, plan)
+    row_floats = config["Hv"] * config["Dv"]
+    rate = cabi.measure_atomic_rate(max(row_floats, 16), min(16, config["Dv"]))
+    roofline["atomics"] = {
+        "row_segments_per_launch": segments,
+        "segments_per_s_measured": rate,
+        "floor_ms": 1e3 * segments / rate,
+        "kernel_ms": stage_ms.get("vjp_gradients"),
+        "waves_per_block": plan["waves"],
+        "row_queue": plan["row_queue"],
+        "note": "global float atomics are bounded by the 64-byte row segments they touch; "
+                "the rate is measured by rosa_hip_measure_atomic_rate in the flush pattern",
+    }
     return {
         "metric": "fwd+bwd tokens/sec",
         "value": tokens / (ms_per_step * 1e-3),

@@ -82,6 +82,27 @@ void rosa_hip_set_record_budget(size_t bytes);
 void rosa_hip_set_gradient_block_waves(int waves);
 
 /*
+ * How the backward's gradient kernel will be launched for `problem` (no counterpart in the
+ * reference): waves per block (1 or 2), whether row tiles are queued between the two bands
+ * of a block, and the dynamic LDS of a block in bytes.  Any of the three may be NULL.
+ * Benchmarks use it to count the global atomics of a launch.
+ */
+int rosa_hip_gradient_block_plan(const rosa_problem* problem, int* waves, int* row_queue,
+                                 size_t* lds_bytes);
+
+/*
+ * Measurement aid, no counterpart in the reference: the rate at which this GPU performs
+ * global float atomic adds in the access pattern of the backward's gradient flush
+ * (16 x 16 tiles at random rows of `buffer`, rows `row_floats` floats apart, `columns` <= 16
+ * floats of every row touched).  The result is in row segments per second: the atomics of
+ * one wave instruction that fall into one row count once, whatever their number, which is
+ * how the hardware bounds them.  `buffer` is device memory of `buffer_bytes` bytes that the
+ * call overwrites; the call synchronises the stream.
+ */
+int rosa_hip_measure_atomic_rate(void* buffer, size_t buffer_bytes, int row_floats, int columns,
+                                 double* segments_per_second, void* stream);
+
+/*
  * Exact hard forward.  Replaces hard_forward_cuda (rosa_soft_kernels.cu:1766-1834)
  * and hard_forward_varlen_cuda (:1837-1920): sign-packs query and key into
  * head-major int32 words (dense [B,H,T], packed [H,N]), finds the

@@ -29,6 +29,8 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_vjp_workspace_bytes",
     "rosa_hip_set_record_budget",
     "rosa_hip_set_gradient_block_waves",
+    "rosa_hip_measure_atomic_rate",
+    "rosa_hip_gradient_block_plan",
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_hard_forward_bits",
@@ -117,6 +119,15 @@ def load() -> ctypes.CDLL:
     ]
     library.rosa_hip_set_gradient_block_waves.restype = None
     library.rosa_hip_set_gradient_block_waves.argtypes = [ctypes.c_int]
+    library.rosa_hip_gradient_block_plan.restype = ctypes.c_int
+    library.rosa_hip_gradient_block_plan.argtypes = [
+        problem_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+        ctypes.POINTER(ctypes.c_size_t),
+    ]
+    library.rosa_hip_measure_atomic_rate.restype = ctypes.c_int
+    library.rosa_hip_measure_atomic_rate.argtypes = [
+        vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), vp,
+    ]
     library.rosa_hip_set_record_budget.restype = None
     library.rosa_hip_set_record_budget.argtypes = [ctypes.c_size_t]
     library.rosa_hip_hard_forward.restype = ctypes.c_int
@@ -476,6 +487,31 @@ def set_gradient_block_waves(waves: Optional[int]) -> None:
     """Waves per block of the gradient kernel: 1, 2, or ``None`` for the library's choice."""
 
     load().rosa_hip_set_gradient_block_waves(0 if waves is None else int(waves))
+
+
+def gradient_block_plan(query: Tensor, value: Tensor, max_suffix_length: int,
+                        cu_seqlens: Optional[Tensor] = None) -> dict:
+    """Launch form of the gradient kernel for a problem: waves per block, row queue, LDS bytes."""
+
+    problem = make_problem(query, value, max_suffix_length, cu_seqlens)
+    waves, queue, lds = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+    status = load().rosa_hip_gradient_block_plan(
+        ctypes.byref(problem), ctypes.byref(waves), ctypes.byref(queue), ctypes.byref(lds))
+    _check(status, "rosa_hip_gradient_block_plan")
+    return dict(waves=waves.value, row_queue=bool(queue.value), lds_bytes=lds.value)
+
+
+def measure_atomic_rate(row_floats: int, columns: int = 16, device: str = "cuda:0") -> float:
+    """Row segments per second of global float atomics in the gradient flush's pattern."""
+
+    buffer = torch.zeros(1 << 26, dtype=torch.float32, device=device)  # 256 MiB
+    rate = ctypes.c_double(0.0)
+    status = load().rosa_hip_measure_atomic_rate(
+        _ptr(buffer), buffer.numel() * 4, int(row_floats), int(columns), ctypes.byref(rate),
+        _stream(buffer),
+    )
+    _check(status, "rosa_hip_measure_atomic_rate")
+    return rate.value
 
 
 def stage_timing(enable: bool) -> None:

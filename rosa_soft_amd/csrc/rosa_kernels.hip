@@ -1715,10 +1715,6 @@ constexpr int kMaxResidentBlocks = 2048;
 // its longest band, which a block of two waves walks more slowly than a single wave.
 int g_gradient_block_waves = 0;  // 0: by shape
 
-int gradient_block_waves(int dvp, int symbol_tiles, int64_t units) {
-  if (g_gradient_block_waves == 1 || g_gradient_block_waves == 2) return g_gradient_block_waves;
-  return ((dvp >= 16 || symbol_tiles > 1) && units >= 2 * kMaxResidentBlocks) ? 2 : 1;
-}
 
 // Waves per block of the gradient kernel.  The waves of a block own neighbouring bands of
 // one (sequence, head) and walk them in step: at the same band-local step every band
@@ -1752,6 +1748,60 @@ constexpr int exchange_tile_floats(bool narrow) { return narrow ? 2 * kWave : 4 
 constexpr int gradient_row_padding(int dvp) { return dvp > 8 ? 8 : 0; }
 
 constexpr int kRestPitch = 100;  // 16-bit elements per row of the third-term plane
+
+// LDS floats a wave of the gradient kernel owns: tile, row words, query words, sink, sign
+// table, third-term plane and the staged grad_output rows (bfloat16 terms, `grad_pitch`
+// elements per row plus padding), in whole 16-byte units
+constexpr size_t gradient_wave_floats(int dvp, int grad_pitch) {
+  const size_t segment = gradient_segment(dvp);
+  const size_t fixed = kChunk * kTilePitch + segment * kRowWords + segment + kWave +
+                       kSignTableWords + kChunk * kRestPitch / 2;
+  return (fixed + (segment * (grad_pitch + gradient_row_padding(dvp)) + 1) / 2 + 3) / 4 * 4;
+}
+
+// How the gradient kernel is launched for a tile shape: waves per block, whether row tiles
+// are queued between the bands of a block, and the LDS of a block.
+struct GradientBlockPlan {
+  int waves;
+  bool row_queue;
+  size_t wave_floats, tile_floats, lds_bytes;
+};
+
+int gradient_block_waves(int dvp, int symbol_tiles, int64_t units) {
+  if (g_gradient_block_waves == 1 || g_gradient_block_waves == 2) return g_gradient_block_waves;
+  return ((dvp >= 16 || symbol_tiles > 1) && units >= 2 * kMaxResidentBlocks) ? 2 : 1;
+}
+
+GradientBlockPlan plan_gradient_blocks(int dvp, int D, int value_words_per_column, int grad_pitch,
+                                       int64_t units) {
+  const int segment = gradient_segment(dvp);
+  const int value_tiles = (dvp + 15) / 16;
+  const int symbol_tiles = D > 16 ? 2 : 1;
+  GradientBlockPlan plan;
+  plan.wave_floats = gradient_wave_floats(dvp, grad_pitch);
+  plan.tile_floats = exchange_tile_floats(dvp == 8 && D <= 8);
+  // two waves: column tiles on their way to the other wave and, where the block stays within
+  // its budget, the queue of row tiles
+  if (gradient_block_waves(dvp, symbol_tiles, units) == 2) {
+    size_t shared = gradient_shared_fixed_floats(segment, value_words_per_column, 2) +
+                    (value_tiles + symbol_tiles) * plan.tile_floats;
+    const size_t queue = kQueueSlots * symbol_tiles * plan.tile_floats;
+    plan.row_queue =
+        (2 * plan.wave_floats + shared + queue) * sizeof(float) <= kGradientBlockLdsBudget;
+    if (plan.row_queue) shared += queue;
+    plan.lds_bytes = (2 * plan.wave_floats + shared) * sizeof(float);
+    if (plan.lds_bytes <= 64 * 1024) {
+      plan.waves = 2;
+      return plan;
+    }
+  }
+  plan.waves = 1;  // also where two waves would not fit (float32 rows of the widest tile)
+  plan.row_queue = false;
+  plan.lds_bytes =
+      (plan.wave_floats + gradient_shared_fixed_floats(segment, value_words_per_column, 1)) *
+      sizeof(float);
+  return plan;
+}
 
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT, int NW>
 __global__ __launch_bounds__(kWave * NW)
@@ -2645,6 +2695,29 @@ __global__ __launch_bounds__(256) void finalize_gradients_kernel(
   }
 }
 
+// Measurement aid: the rate of global float atomics in the access pattern of the gradient
+// flush.  Every wave adds 16 x 16 tiles (lane (li, lg) adds rows 4 lg .. 4 lg + 3 of column
+// li, four instructions per tile) at pseudo-random rows of a buffer whose rows are
+// `row_stride` floats apart; `columns` <= 16 lanes of every row are active.  One
+// instruction touches four rows, i.e. four 64-byte segments.
+__global__ __launch_bounds__(kWave) void atomic_rate_kernel(float* buffer, uint32_t rows,
+                                                            uint32_t row_stride, int columns,
+                                                            int tiles) {
+  const int lane = threadIdx.x;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  uint32_t state = blockIdx.x * 2654435761u + 12345u;
+  for (int tile = 0; tile < tiles; ++tile) {
+    state = state * 1664525u + 1013904223u;
+    const uint32_t first_row = (state >> 8) % (rows - 16u);
+    if (li < columns) {
+      float* base = buffer + static_cast<size_t>(first_row + 4 * lg) * row_stride + li;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) atomicAdd(base + e * row_stride, 1.0f);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -2907,49 +2980,26 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   }
   stage_end(kStageRowStats, stream);
   constexpr int SEG = gradient_segment(DVP);
-  constexpr int VT = (DVP + 15) / 16;
-  // per wave: tile, row words, query words, sink, sign table, third-term plane and the
-  // staged grad_output rows (bfloat16 terms), in whole 16-byte units
-  constexpr size_t kFixedFloats = kChunk * kTilePitch + SEG * kRowWords + SEG + kWave +
-                                  kSignTableWords + kChunk * kRestPitch / 2;
-  const size_t wave_floats =
-      (kFixedFloats + (SEG * (P.grad_pitch + gradient_row_padding(DVP)) + 1) / 2 + 3) / 4 * 4;
-  const bool narrow_tiles = DVP == 8 && P.L.D <= 8;
-  const size_t tile_floats = exchange_tile_floats(narrow_tiles);
+  // At most 64 KB of dynamic LDS per block: what every kernel may use without raising its
+  // limit first.  (Raising it would be a configuration call per launch, and those are
+  // refused while a stream is being captured into a graph.)
+  static_assert((gradient_wave_floats(DVP, grad_term_pitch(kMaxGradTerms, DVP)) +
+                 gradient_shared_fixed_floats(SEG, NVW, 1)) * sizeof(float) <= 64 * 1024,
+                "dynamic LDS of the gradient kernel");
+  const GradientBlockPlan plan =
+      plan_gradient_blocks(DVP, P.L.D, NVW, P.grad_pitch, P.total_units);
+  VjpParams Q = P;
+  Q.wave_lds_floats = static_cast<int>(plan.wave_floats);
+  Q.exchange_tile_floats = static_cast<int>(plan.tile_floats);
+  Q.row_queue = plan.row_queue ? 1 : 0;
+  const unsigned blocks = static_cast<unsigned>(std::max(1, w.resident_blocks / plan.waves));
   stage_begin(kStageGradients, stream);
-  const auto launch = [&](auto waves_tag) {
-    constexpr int NW = decltype(waves_tag)::value;
-    // shared by the waves of a block: window columns, work index, column tiles on their way
-    // to wave 0, row tile queues
-    size_t shared_floats =
-        gradient_shared_fixed_floats(SEG, NVW, NW) + (NW - 1) * (VT + DT) * tile_floats;
-    const size_t queue_floats = (NW - 1) * kQueueSlots * DT * tile_floats;
-    const bool row_queue = NW > 1 && (NW * wave_floats + shared_floats + queue_floats) *
-                                             sizeof(float) <= kGradientBlockLdsBudget;
-    if (row_queue) shared_floats += queue_floats;
-    // At most 64 KB of dynamic LDS per block: what every kernel may use without raising its
-    // limit first.  (Raising it would be a configuration call per launch, and those are
-    // refused while a stream is being captured into a graph.)
-    constexpr size_t kWaveFloatsMax =
-        (kFixedFloats + SEG * (grad_term_pitch(kMaxGradTerms, DVP) + 8) / 2 + 3) / 4 * 4;
-    static_assert(NW > 1 || (kWaveFloatsMax + gradient_shared_fixed_floats(SEG, NVW, 1)) *
-                                    sizeof(float) <= 64 * 1024,
-                  "dynamic LDS of the gradient kernel");
-    VjpParams Q = P;
-    Q.wave_lds_floats = static_cast<int>(wave_floats);
-    Q.exchange_tile_floats = static_cast<int>(tile_floats);
-    Q.row_queue = row_queue ? 1 : 0;
-    const size_t lds_bytes = (NW * wave_floats + shared_floats) * sizeof(float);
-    if (lds_bytes > 64 * 1024) return false;
-    const unsigned blocks = static_cast<unsigned>(std::max(1, w.resident_blocks / NW));
-    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, NW>), dim3(blocks),
-                       dim3(kWave * NW), lds_bytes, stream, Q);
-    return true;
-  };
-  // two waves per block where that fits the LDS of a block (float32 rows of the widest
-  // tile do not)
-  if (gradient_block_waves(DVP, DT, P.total_units) != 2 || !launch(std::integral_constant<int, 2>{})) {
-    launch(std::integral_constant<int, 1>{});
+  if (plan.waves == 2) {
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 2>), dim3(blocks),
+                       dim3(kWave * 2), plan.lds_bytes, stream, Q);
+  } else {
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 1>), dim3(blocks),
+                       dim3(kWave), plan.lds_bytes, stream, Q);
   }
   stage_end(kStageGradients, stream);
   return 0;
@@ -3590,6 +3640,52 @@ int rosa_hip_stage_times(float* milliseconds, int count) {
       return fail(5, "event elapsed failed");
     milliseconds[i] = ms;
   }
+  return 0;
+}
+
+int rosa_hip_gradient_block_plan(const rosa_problem* problem, int* waves, int* row_queue,
+                                 size_t* lds_bytes) {
+  ProblemView view;
+  const int status = check_problem(problem, &view);
+  if (status != 0) return status;
+  const int slice_width = std::min(view.L.Dv, kValueSlice);
+  const int dvp = padded_value_width(slice_width);
+  const GradientBlockPlan plan =
+      plan_gradient_blocks(dvp, view.L.D, value_words(slice_width),
+                           grad_term_pitch(view.grad_terms, dvp),
+                           static_cast<int64_t>(view.L.slots) * view.L.H);
+  if (waves != nullptr) *waves = plan.waves;
+  if (row_queue != nullptr) *row_queue = plan.row_queue ? 1 : 0;
+  if (lds_bytes != nullptr) *lds_bytes = plan.lds_bytes;
+  return 0;
+}
+
+int rosa_hip_measure_atomic_rate(void* buffer, size_t buffer_bytes, int row_floats, int columns,
+                                 double* segments_per_second, void* stream) {
+  if (buffer == nullptr || segments_per_second == nullptr) return fail(1, "NULL argument");
+  if (row_floats < 16 || columns < 1 || columns > 16) return fail(1, "row_floats >= 16, 1 <= columns <= 16");
+  const size_t rows = buffer_bytes / (sizeof(float) * static_cast<size_t>(row_floats));
+  if (rows < 64 || rows > UINT32_MAX) return fail(1, "buffer holds too few or too many rows");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipEvent_t begin, end;
+  if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess)
+    return fail(5, "hipEventCreate failed");
+  const int waves = kMaxResidentBlocks, tiles = 2000;
+  // one short launch to warm up, then the timed one
+  hipLaunchKernelGGL(atomic_rate_kernel, dim3(waves), dim3(kWave), 0, s, static_cast<float*>(buffer),
+                     static_cast<uint32_t>(rows), static_cast<uint32_t>(row_floats), columns, 20);
+  (void)hipEventRecord(begin, s);
+  hipLaunchKernelGGL(atomic_rate_kernel, dim3(waves), dim3(kWave), 0, s, static_cast<float*>(buffer),
+                     static_cast<uint32_t>(rows), static_cast<uint32_t>(row_floats), columns, tiles);
+  (void)hipEventRecord(end, s);
+  float ms = 0.0f;
+  const bool ok = hipEventSynchronize(end) == hipSuccess &&
+                  hipEventElapsedTime(&ms, begin, end) == hipSuccess && ms > 0.0f;
+  (void)hipEventDestroy(begin);
+  (void)hipEventDestroy(end);
+  if (!ok) return fail(5, "timing the atomic kernel failed");
+  // 16 row segments per tile
+  *segments_per_second = static_cast<double>(waves) * tiles * 16.0 / (ms * 1e-3);
   return 0;
 }
 
