@@ -1257,13 +1257,13 @@ __device__ __forceinline__ void fill_sign_table(uint32_t* table, int lane) {
 // Utilities u(t, a) = sum_d grad_output[t, d] * sign(v[a, d]) of 16 rows against
 // their 80 window columns on the matrix cores, written in (row r, lane l)
 // coordinates: out[r * pitch + l] for the pair on diagonal lane l, whose window
-// column is c = 64 - l + r.  `grad_tile` holds the bfloat16 terms of the 16 grad_output
+// column is c = 64 - l + r (BY_COLUMN: out[r * pitch + c], pitch a multiple of 4).  `grad_tile` holds the bfloat16 terms of the 16 grad_output
 // rows, `grad_pitch` elements each: k = term * DVP + d, `k_blocks` blocks of 32
 // (zero beyond the last term); the sum over the terms is the float32 product.
 // `value_columns` holds the sign words of the window columns (NVW per column).  Elements
 // of the first and last column tile that belong to no lane go to `discard` (one float
 // per lane).
-template <int NVW, int DVP>
+template <int NVW, int DVP, bool BY_COLUMN = false>
 __device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad_pitch,
                                              int k_blocks, const uint32_t* value_columns,
                                              const uint32_t* sign_table, float* out, int pitch,
@@ -1280,7 +1280,7 @@ __device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad
     constexpr int kBlocksMax = grad_term_pitch(kMaxGradTerms, DVP) / 32;
 #pragma unroll
     for (int q = 0; q < kBlocksMax; ++q) {
-      if (q >= k_blocks) break;  // wave-uniform
+      if (q > 0 && q >= k_blocks) break;  // wave-uniform; there is always a first block
       const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
       // this lane's k = 32 q + 8 lg .. + 7 are eight value dimensions of one term
       const int d0 = (32 * q + 8 * lg) & (DVP - 1);
@@ -1289,16 +1289,36 @@ __device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad
       const uint32_t byte = word >> (d0 & 31);
       const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
       const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
-      acc = mfma_bf16(a, v4u{low.x, low.y, high.x, high.y}, acc);
+      const v4u signs = {low.x, low.y, high.x, high.y};
+      // BY_COLUMN takes the transposed product: lane (li, lg) then holds columns
+      // 16 m + 4 lg .. + 3 of row li, four neighbours of one tile row
+      acc = BY_COLUMN ? mfma_bf16(signs, a, acc) : mfma_bf16(a, signs, acc);
     }
+    // The product is read right behind a branch of the loop above, where the compiler has
+    // been seen to leave out the wait states a matrix result needs before vector or LDS
+    // instructions may read it (wrong utilities): they are spent here.
+    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(acc));
+    if constexpr (BY_COLUMN) {
+      // out[r][c]: one aligned 16-byte store; columns outside r + 1 .. r + 64 belong to no
+      // lane and stay zero
+      const int r = li;
+      const int c = 16 * m + 4 * lg;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int r = 4 * lg + e;
-      const int l = 64 - (16 * m + li) + r;
-      float* target = out + r * pitch + l;
-      if (m == 0) target = l < kWave ? target : discard + lane;
-      if (m == 4) target = l >= 0 ? target : discard + lane;
-      *target = acc[e];
+      for (int e = 0; e < 4; ++e) {
+        if (m == 0 && c + e < r + 1) acc[e] = 0.0f;
+        if (m == 4 && c + e > r + kWave) acc[e] = 0.0f;
+      }
+      *reinterpret_cast<v4f*>(out + r * pitch + c) = acc;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int r = 4 * lg + e;
+        const int l = 64 - (16 * m + li) + r;
+        float* target = out + r * pitch + l;
+        if (m == 0) target = l < kWave ? target : discard + lane;
+        if (m == 4) target = l >= 0 ? target : discard + lane;
+        *target = acc[e];
+      }
     }
   }
 }
@@ -1682,10 +1702,12 @@ __global__ __launch_bounds__(256) void finalize_row_records_kernel(float4* __res
 // tile (the 16 highest columns), which is flushed with global atomics, and the
 // other four shift up by one tile for the next chunk, so column sums live in
 // accumulator registers for their whole life.
-// 16 zero + 64 lanes + 16 zero, padded to 99: with 4 * (pitch + 1) = 16 (mod 64) the
-// skewed reads of the column sums (k slice lg <-> row step + 4 lg) and of the row sums
-// (row li, stride pitch + 1 = 36 (mod 64)) both touch 64 different LDS banks.
-constexpr int kTilePitch = 99;
+// The tile is stored by window column: pair (r, lane l) at [r][c], c = 64 - l + r, so row r
+// holds its 64 pairs in columns r + 1 .. r + 64 and zeros elsewhere.  Pitch 84: with
+// 4 * pitch = 16 (mod 64) the reads of the column sums (lane (li, lg) reads rows
+// 4 lg .. 4 lg + 3 of column li) touch 64 different LDS banks, and the row sums read four
+// neighbouring columns of row li as one aligned 16-byte word, rows 20 (mod 64) banks apart.
+constexpr int kTilePitch = 84;
 constexpr int kCheckpointChunksMax = 4;  // chunks per staged segment at most
 constexpr int kWindowTiles = 5;  // 80 window columns
 
@@ -1747,7 +1769,7 @@ constexpr int exchange_tile_floats(bool narrow) { return narrow ? 2 * kWave : 4 
 // where the block's LDS decides how many blocks a compute unit holds)
 constexpr int gradient_row_padding(int dvp) { return dvp > 8 ? 8 : 0; }
 
-constexpr int kRestPitch = 100;  // 16-bit elements per row of the third-term plane
+constexpr int kRestPitch = 84;  // 16-bit elements per row of the third-term plane
 
 // LDS floats a wave of the gradient kernel owns: tile, row words, query words, sink, sign
 // table, third-term plane and the staged grad_output rows (bfloat16 terms, `grad_pitch`
@@ -2270,8 +2292,8 @@ void vjp_gradients_kernel(VjpParams P) {
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
-          utility_tile<NVW, DVP>(grad_tile, GP, P.grad_pitch / 32, value_window + local * NVW,
-                                 sign_table, tile + 16, kTilePitch, discard, lane);
+          utility_tile<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32, value_window + local * NVW,
+                                 sign_table, tile, kTilePitch, discard, lane);
           wave_lds_fence();
         }
         issue_pending();
@@ -2281,7 +2303,7 @@ void vjp_gradients_kernel(VjpParams P) {
         }
         if (!want_qk) {  // no utilities were written: the replay must still read finite values
 #pragma unroll
-          for (int r = 0; r < kChunk; ++r) tile[r * kTilePitch + 16 + lane] = 0.0f;
+          for (int r = 0; r < kChunk; ++r) tile[r * (kTilePitch + 1) + 64 - lane] = 0.0f;
         }
         float keep_evidence[kChunk];  // S + overflow
         float keep_overflow[kChunk];
@@ -2298,7 +2320,7 @@ void vjp_gradients_kernel(VjpParams P) {
           constexpr bool CACHED = decltype(cached_tag)::value;  // keep decisions are read back
           constexpr bool QUIET = decltype(quiet_tag)::value;    // overflow terms are negligible
           const uint32_t* row = rows + local * kRowWords;
-          const float* slot = tile + 16 + lane;
+          const float* slot = tile + 64 - lane;  // this lane's pair of row r: + r * (pitch + 1)
           // row words and utilities are fetched kRowsAhead rows before their use
           constexpr int kRowsAhead = kFetchAhead ? 2 : 1;
           uint4 ahead_symbols[kRowsAhead];
@@ -2308,7 +2330,7 @@ void vjp_gradients_kernel(VjpParams P) {
           for (int r = 0; r < kRowsAhead; ++r) {
             ahead_symbols[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords);
             ahead_extra[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords + 4);
-            ahead_utility[r] = slot[r * kTilePitch];
+            ahead_utility[r] = slot[r * (kTilePitch + 1)];
           }
 #pragma unroll
           for (int r = 0; r < kChunk; ++r) {
@@ -2324,7 +2346,7 @@ void vjp_gradients_kernel(VjpParams P) {
                   *reinterpret_cast<const uint4*>(row + ahead * kRowWords);
               ahead_extra[r % kRowsAhead] =
                   *reinterpret_cast<const uint4*>(row + ahead * kRowWords + 4);
-              ahead_utility[r % kRowsAhead] = slot[ahead * kTilePitch];
+              ahead_utility[r % kRowsAhead] = slot[ahead * (kTilePitch + 1)];
             }
             // the loads stay here, ahead of their use (the scheduler would sink them)
             if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
@@ -2353,7 +2375,7 @@ void vjp_gradients_kernel(VjpParams P) {
             }
             const float adjoint =
                 (probability * adjoint_gain) * (keep * utility - expected) * inv_root;
-            tile_bits[r * kTilePitch + 16 + lane] = split_bf16(probability * keep);
+            tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16(probability * keep);
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
             keep_adjoint[r] = live ? adjoint : 0.0f;
@@ -2377,7 +2399,7 @@ void vjp_gradients_kernel(VjpParams P) {
         wave_lds_fence();
 
         // Column sums.  Tile m covers window columns 16m .. 16m+15 (a = first + 1 - 64 + c);
-        // element (column c, row r) of the skewed matrix is tile[r][64 - c + r], a dword
+        // element (column c, row r) of the matrix is tile[r][c], a dword
         // holding the two bfloat16 terms of the pair's value.  One matrix instruction per
         // tile contracts all 16 rows: k = 2 r + term, lane (li, lg) brings rows 4 lg .. 4 lg + 3
         // of column 16 m + li.
@@ -2387,7 +2409,7 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               const int r = 4 * lg + j;
-              operands[m][j] = tile_bits[r * kTilePitch + 16 + 64 - (16 * m + li) + r];
+              operands[m][j] = tile_bits[r * kTilePitch + 16 * m + li];
             }
           }
         };
@@ -2432,8 +2454,8 @@ void vjp_gradients_kernel(VjpParams P) {
               adjoint_carry = b;
               gate_below = keep_gate[r];
               uint32_t rest;
-              tile_bits[r * kTilePitch + 16 + lane] = split_bf16_exact(b * keep_evidence[r], rest);
-              rest_plane[r * kRestPitch + 16 + lane] = static_cast<uint16_t>(rest >> 16);
+              tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(b * keep_evidence[r], rest);
+              rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
             }
           } else {
 #pragma unroll
@@ -2465,8 +2487,8 @@ void vjp_gradients_kernel(VjpParams P) {
             if (ring_live == 0) ring_sum = 0.0f;
             const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
             uint32_t rest;
-            tile_bits[r * kTilePitch + 16 + lane] = split_bf16_exact(active ? h : 0.0f, rest);
-            rest_plane[r * kRestPitch + 16 + lane] = static_cast<uint16_t>(rest >> 16);
+            tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(active ? h : 0.0f, rest);
+            rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
           }
           }
           wave_lds_fence();
@@ -2477,11 +2499,11 @@ void vjp_gradients_kernel(VjpParams P) {
             column_operands(adjoints);
 #pragma unroll
             for (int m = 0; m < kWindowTiles; ++m) {
-              const uint16_t* column = rest_plane + 16 + 64 - (16 * m + li);
+              const uint16_t* column = rest_plane + 16 * m + li;
               const int r = 4 * lg;
               adjoint_rests[m] = v2u{
-                  pair_of(column + r * (kRestPitch + 1), column + (r + 1) * (kRestPitch + 1)),
-                  pair_of(column + (r + 2) * (kRestPitch + 1), column + (r + 3) * (kRestPitch + 1))};
+                  pair_of(column + r * kRestPitch, column + (r + 1) * kRestPitch),
+                  pair_of(column + (r + 2) * kRestPitch, column + (r + 3) * kRestPitch)};
             }
             const uint4 q_words = *reinterpret_cast<const uint4*>(query_rows + local + 4 * lg);
 #pragma unroll
@@ -2511,8 +2533,7 @@ void vjp_gradients_kernel(VjpParams P) {
           // row sums: rows are complete for this band after the chunk
           if (want_q) {
             // k slice lg of step s <-> window columns 20 lg + 4 s .. + 3 (both terms of each):
-            // every lane reads 20 consecutive key words, and the skewed tile reads of the 64
-            // lanes fall into different banks
+            // every lane reads 20 consecutive key words and 20 consecutive columns of its row
             // the third terms accumulate apart (see above: one instruction shape per
             // accumulator chain)
             v4f query_part[3][DT];
@@ -2525,14 +2546,12 @@ void vjp_gradients_kernel(VjpParams P) {
             for (int step = 0; step < kWindowTiles; ++step) {
               const uint4 k_words =
                   *reinterpret_cast<const uint4*>(key_tile + 4 * kWindowTiles * lg + 4 * step);
-              v4u adjoints;
+              // four neighbouring columns of row li: one aligned 16-byte word of the tile and
+              // one aligned 8-byte word of the third terms
               const int c0 = 4 * kWindowTiles * lg + 4 * step;
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                adjoints[j] = tile_bits[li * kTilePitch + 16 + 64 - (c0 + j) + li];
-              }
-              const uint16_t* rests = rest_plane + li * kRestPitch + 16 + 64 - c0 + li;
-              const v2u adjoint_rests = {pair_of(rests, rests - 1), pair_of(rests - 2, rests - 3)};
+              const v4u adjoints = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
+              const v2u adjoint_rests =
+                  *reinterpret_cast<const v2u*>(rest_plane + li * kRestPitch + c0);
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
                 const int bit = 16 * n + li;
