@@ -1427,11 +1427,11 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
   constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
   constexpr int kWeightPitch = 68;
   __shared__ __attribute__((aligned(16))) uint32_t rows[kBlockRows * kRowWords];
-  // bfloat16 terms of the block's grad_output rows; sized for three terms, 16 bytes of
-  // padding per row against bank conflicts of the operand reads
+  // bfloat16 terms of the block's grad_output rows, 16 bytes of padding per row against
+  // bank conflicts of the operand reads; sized at the launch for the terms the input type
+  // needs (row_stats_dynamic_lds), because the LDS of a block bounds the waves per SIMD
   constexpr int kGradChunksMax = grad_term_pitch(kMaxGradTerms, DVP) / 8;  // 16-byte pieces per row
-  constexpr int kGradPitchMax = 8 * kGradChunksMax + 8;
-  __shared__ __attribute__((aligned(16))) uint16_t grads[kBlockRows * kGradPitchMax];
+  extern __shared__ __attribute__((aligned(16))) uint16_t grads[];  // [kBlockRows][grad_pitch + 8]
   __shared__ __attribute__((aligned(16))) uint32_t sign_table[kSignTableWords];
   __shared__ uint32_t value_columns[(kBlockRows + kWave) * NVW];
   __shared__ __attribute__((aligned(16))) float utilities[kChunk * kUtilityPitch];  // u, then e d u
@@ -1695,7 +1695,7 @@ __global__ __launch_bounds__(256) void finalize_row_records_kernel(float4* __res
 //   dV[a, :]   += sum_t  d p(t, a) go[t, :]
 //   dK[a-1, :] += c sum_t h(t, a) z(q[t, :])
 //   dQ[t, :]   += c sum_a h(t, a) z(k[a-1, :]),   c = mismatch_scale / (2 D)
-// are formed on the matrix cores (v_mfma_f32_16x16x4_f32).  In the chunk's own
+// are formed on the matrix cores (v_mfma_f32_16x16x32_bf16, split operands).  In the chunk's own
 // (row r, window column c) coordinates the pair (r, lane l) sits at
 // c = 64 - l + r, i.e. the tile read with a skew is an ordinary matrix.  The
 // window spans 80 columns = 5 MFMA tiles; a chunk completes exactly the last
@@ -2980,6 +2980,12 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   return 0;
 }
 
+// bytes of the staged grad_output rows of a block of the row-statistics kernel
+size_t row_stats_dynamic_lds(int grad_pitch) {
+  constexpr int kBlockRows = 32;
+  return sizeof(uint16_t) * kBlockRows * static_cast<size_t>(grad_pitch + 8);
+}
+
 template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT>
 int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
                       hipStream_t stream) {
@@ -2991,7 +2997,7 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   }
   stage_begin(kStageRowStats, stream);
   hipLaunchKernelGGL((vjp_row_stats_kernel<NVW, DVP, VARLEN, DROPOUT>), dim3(units), dim3(kWave),
-                     0, stream, P);
+                     row_stats_dynamic_lds(P.grad_pitch), stream, P);
   {
     const int64_t rows = static_cast<int64_t>(P.L.N) * P.L.H;
     hipLaunchKernelGGL(finalize_row_records_kernel, dim3(blocks_for(rows, 256)), dim3(256), 0,
