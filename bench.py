@@ -293,8 +293,11 @@ def atomic_row_segments(config, plan: dict) -> int:
 
     lengths = config.get("lengths") or [config["T"]] * config["B"]
     D, Dv = config["D"], config["Dv"]
-    symbol_segments = -(-4 * D // 64)
-    value_segments = sum(-(-4 * min(64, Dv - first) // 64) for first in range(0, Dv, 64))
+    # rows of at most 8 floats are accumulated head-major, where two neighbouring rows
+    # share a segment and leave in one instruction
+    symbol_segments = 0.5 if D <= 8 else -(-4 * D // 64)
+    value_segments = 0.5 if Dv <= 8 else sum(
+        -(-4 * min(64, Dv - first) // 64) for first in range(0, Dv, 64))
     rows = columns = 0
     for length in lengths:
         steps = [length - 1 - 64 * band for band in range((length + 63) // 64)]
@@ -306,7 +309,7 @@ def atomic_row_segments(config, plan: dict) -> int:
         else:
             columns += sum(steps)
             rows += sum(steps)
-    return config["H"] * (columns * (symbol_segments + value_segments) + rows * symbol_segments)
+    return int(config["H"] * (columns * (symbol_segments + value_segments) + rows * symbol_segments))
 
 
 def config_summary(measured: dict) -> dict:

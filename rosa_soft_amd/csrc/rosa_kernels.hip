@@ -736,9 +736,18 @@ struct VjpParams {
   float tail_threshold;         // window products below this are treated as zero in the reverse sweep
   int gradient_mask;
   int dvp;                      // padded value width
-  float* grad_query;            // symbol-space accumulators, token-major
-  float* grad_key;
-  float* grad_value;
+  float* grad_query;            // symbol-space accumulators: the gradient tensors themselves
+  float* grad_key;              //   (token-major) or, for rows of at most 8 floats, head-major
+  float* grad_value;            //   accumulators in the workspace (see symbols_by_head)
+  // Global float atomics cost one operation per 64-byte segment an instruction touches.  A
+  // row of at most 8 floats is half a segment, and in a token-major tensor the rows a band
+  // completes lie H * D floats apart; in a head-major accumulator [sequence, head][position][D]
+  // they are neighbours, so that two rows leave in one segment.  Query rows are stored one
+  // position down (row t at t - 1) and value rows likewise (route a at a - 1): the first
+  // row of a chunk then starts a segment, and the slot of the last position of every
+  // (sequence, head) run stays zero.  finalize_gradients_kernel moves the sums to the tensors.
+  int symbols_by_head;          // grad_query / grad_key point to head-major accumulators
+  int values_by_head;           // grad_value points to a head-major accumulator
   int32_t* work_counter;
   const int32_t* header;        // [0] offsets flag, [1] work counter, [3] chunk records fit
   float* checkpoints;           // one record per (band, 16-row chunk), or NULL
@@ -1889,7 +1898,9 @@ void vjp_gradients_kernel(VjpParams P) {
   const float logit_gain = in_vector_register(P.logit_gain);
   const float inverse_keep = in_vector_register(P.inverse_keep);
   // the contractions run on negated symbols
-  const float symbol_scale = -0.5f * P.mismatch_scale / static_cast<float>(D);
+  // dQ and dK are linear in the route adjoints, so the constant factor of every adjoint
+  // (adjoint_gain) is applied here, once per flushed element, instead of once per pair
+  const float symbol_scale = -0.5f * P.mismatch_scale / static_cast<float>(D) * adjoint_gain;
   float* ring = P.block_scratch +
       (static_cast<int64_t>(blockIdx.x) * NW + wave) * P.block_scratch_floats;
   // without chunk records: (S, window) before every chunk of the current segment, then
@@ -1996,16 +2007,26 @@ void vjp_gradients_kernel(VjpParams P) {
     bool done_flush_rows = true;
     // step 0 of the band: row diag0 + 1 (query gradients), column 1 (value gradients, key
     // position 0)
-    const uint32_t symbol_stride = static_cast<uint32_t>(P.L.H) * D;
-    const uint32_t value_stride = static_cast<uint32_t>(P.L.Hv) * P.value_stride;
-    float* band_query_base = P.grad_query +
-        ((static_cast<int64_t>(u.start) + view.diag0 + 1) * P.L.H + u.head) * D;
-    float* band_key_base = P.grad_key + (static_cast<int64_t>(u.start) * P.L.H + u.head) * D;
-    float* band_value_base = P.grad_value +
-        ((static_cast<int64_t>(u.start) + 1) * P.L.Hv + hv) * P.value_stride + P.value_offset;
+    const uint32_t symbol_stride = P.symbols_by_head ? D : static_cast<uint32_t>(P.L.H) * D;
+    const uint32_t value_stride =
+        P.values_by_head ? P.value_stride : static_cast<uint32_t>(P.L.Hv) * P.value_stride;
+    float* band_query_base = P.symbols_by_head
+        ? P.grad_query + (u.word_base + view.diag0) * D
+        : P.grad_query + ((static_cast<int64_t>(u.start) + view.diag0 + 1) * P.L.H + u.head) * D;
+    float* band_key_base = P.symbols_by_head
+        ? P.grad_key + u.word_base * D
+        : P.grad_key + (static_cast<int64_t>(u.start) * P.L.H + u.head) * D;
+    // (sequence, value head, position 0) in a head-major tensor over the value heads
+    const int64_t value_run = VARLEN ? static_cast<int64_t>(hv) * P.L.N + u.start
+                                     : (static_cast<int64_t>(u.seq) * P.L.Hv + hv) * P.L.T;
+    float* band_value_base = P.values_by_head
+        ? P.grad_value + value_run * P.value_stride
+        : P.grad_value +
+              ((static_cast<int64_t>(u.start) + 1) * P.L.Hv + hv) * P.value_stride + P.value_offset;
     // One completed 16 x 16 tile: lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li.
-    // With at most 8 live columns the upper half of every 16 lanes takes rows e + 2 from the
-    // lower half, so that two instructions carry what would otherwise take four.
+    // With at most 8 live columns the upper half of every 16 lanes takes the odd rows from the
+    // lower half, so that two instructions carry what would otherwise take four and each of
+    // them covers pairs of neighbouring rows (one 64-byte segment in a head-major accumulator).
     // `base` (element (row 0, column 0) of the tile) and `row_stride` are wave-uniform, so
     // the address of a lane is a scalar pointer plus a 32-bit lane offset; FULL tiles (every
     // row exists) need no row test.
@@ -2015,13 +2036,13 @@ void vjp_gradients_kernel(VjpParams P) {
       // rows_left: valid rows counted from row 4 lg
       if (columns <= 8) {
         const int half = li >> 3;
-        const float first = dpp_row_shr8(values[0], values[2]);
-        const float second = dpp_row_shr8(values[1], values[3]);
+        const float first = dpp_row_shr8(values[0], values[1]);   // rows 4 lg, 4 lg + 1
+        const float second = dpp_row_shr8(values[2], values[3]);  // rows 4 lg + 2, 4 lg + 3
         if ((li & 7) < columns) {
-          const uint32_t offset = static_cast<uint32_t>(4 * lg + 2 * half) * row_stride + (li & 7);
-          if (FULL || 2 * half < rows_left) atomicAdd(base + offset, scale * first);
-          if (FULL || 2 * half + 1 < rows_left) {
-            atomicAdd(base + row_stride + offset, scale * second);
+          const uint32_t offset = static_cast<uint32_t>(4 * lg + half) * row_stride + (li & 7);
+          if (FULL || half < rows_left) atomicAdd(base + offset, scale * first);
+          if (FULL || 2 + half < rows_left) {
+            atomicAdd(base + 2 * row_stride + offset, scale * second);
           }
         }
       } else if (li < columns) {
@@ -2373,8 +2394,8 @@ void vjp_gradients_kernel(VjpParams P) {
                 keep = dropout_keeps(key, route_hash) ? inverse_keep : 0.0f;
               }
             }
-            const float adjoint =
-                (probability * adjoint_gain) * (keep * utility - expected) * inv_root;
+            // (without its constant factor adjoint_gain, which symbol_scale carries)
+            const float adjoint = (probability * inv_root) * (keep * utility - expected);
             tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16(probability * keep);
             // rows past the band's end run on repeated data and may hold anything,
             // NaN included: select, never multiply by zero
@@ -2681,12 +2702,28 @@ void vjp_gradients_kernel(VjpParams P) {
 }
 
 // Softsign Jacobian 1 / (1 + |x|)^2 applied once to the symbol-space sums.
+// Where the sums of a gradient tensor come from when they were accumulated head-major.
+struct HeadMajorSums {
+  const float* query;  // [sequence, head][position][D], row t stored at t - 1; NULL: in place
+  const float* key;    // [sequence, head][position][D]
+  const float* value;  // [sequence, value head][position][Dv], row a stored at a - 1
+  int H, Hv, D, Dv, T, N, varlen;
+};
+
+// head-major row of (token, head) in a tensor with `heads` heads
+__device__ __forceinline__ int64_t head_major_row(int64_t token, int head, int heads, int T,
+                                                  int N, int varlen) {
+  if (varlen) return static_cast<int64_t>(head) * N + token;
+  const int64_t batch = token / T;
+  return (batch * heads + head) * T + (token - batch * T);
+}
+
 template <int DTYPE>
 __global__ __launch_bounds__(256) void finalize_gradients_kernel(
     const void* __restrict__ query, const void* __restrict__ key,
     const void* __restrict__ value, float* __restrict__ grad_query,
     float* __restrict__ grad_key, float* __restrict__ grad_value, int64_t symbol_elements,
-    int64_t value_elements, const int32_t* __restrict__ offset_error) {
+    int64_t value_elements, const int32_t* __restrict__ offset_error, HeadMajorSums sums) {
   const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (offset_error != nullptr && *offset_error != 0) {
     // invalid cu_seqlens (packed layout): nothing was accumulated; every gradient is NaN
@@ -2699,18 +2736,42 @@ __global__ __launch_bounds__(256) void finalize_gradients_kernel(
     return;
   }
   if (index < symbol_elements) {
+    int64_t row = 0;
+    int d = 0;
+    if (sums.query != nullptr || sums.key != nullptr) {
+      const int64_t token_head = index / sums.D;
+      d = static_cast<int>(index - token_head * sums.D);
+      const int64_t token = token_head / sums.H;
+      row = head_major_row(token, static_cast<int>(token_head - token * sums.H), sums.H, sums.T,
+                           sums.N, sums.varlen);
+    }
     if (grad_query != nullptr) {
       const float den = 1.0f + fabsf(load_as_float<DTYPE>(query, index));
-      grad_query[index] *= 1.0f / (den * den);
+      // the slot below the first row of a run is the unused last slot of the run before it
+      const float sum = sums.query == nullptr ? grad_query[index]
+                        : (row > 0 ? sums.query[(row - 1) * sums.D + d] : 0.0f);
+      grad_query[index] = sum * (1.0f / (den * den));
     }
     if (grad_key != nullptr) {
       const float den = 1.0f + fabsf(load_as_float<DTYPE>(key, index));
-      grad_key[index] *= 1.0f / (den * den);
+      const float sum = sums.key == nullptr ? grad_key[index] : sums.key[row * sums.D + d];
+      grad_key[index] = sum * (1.0f / (den * den));
     }
   }
   if (index < value_elements && grad_value != nullptr) {
     const float den = 1.0f + fabsf(load_as_float<DTYPE>(value, index));
-    grad_value[index] *= 1.0f / (den * den);
+    float sum;
+    if (sums.value == nullptr) {
+      sum = grad_value[index];
+    } else {
+      const int64_t token_head = index / sums.Dv;
+      const int d = static_cast<int>(index - token_head * sums.Dv);
+      const int64_t token = token_head / sums.Hv;
+      const int64_t row = head_major_row(token, static_cast<int>(token_head - token * sums.Hv),
+                                         sums.Hv, sums.T, sums.N, sums.varlen);
+      sum = row > 0 ? sums.value[(row - 1) * sums.Dv + d] : 0.0f;
+    }
+    grad_value[index] = sum * (1.0f / (den * den));
   }
 }
 
@@ -2809,6 +2870,7 @@ ForwardWorkspace carve_forward(const ProblemView& v) {
 }
 
 constexpr int kValueSlice = 64;  // value dimensions one backward pass covers
+constexpr int kNarrowRow = 8;    // gradient rows up to this many floats are accumulated head-major
 
 // bytes of chunk records the backward workspace may hold (4 GiB unless the caller lowers it)
 constexpr size_t kDefaultRecordBudget = size_t(1) << 32;
@@ -2826,6 +2888,8 @@ int padded_value_width(int Dv) {
 struct VjpWorkspace {
   size_t header, seq_start, seq_len, block_prefix, step_prefix, stats, grad_rows,
       value_bits, block_scratch, total;
+  size_t sums_query, sums_key, sums_value;  // head-major accumulators (rows of <= 8 floats)
+  bool symbols_by_head, values_by_head;
   size_t checkpoints;
   int64_t checkpoint_capacity;  // chunk records that fit in the workspace (0: none kept)
   int record_floats;
@@ -2852,6 +2916,14 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   cursor += align_up(sizeof(uint16_t) * rows * grad_term_pitch(v.grad_terms, dvp));
   w.value_bits = cursor;
   cursor += align_up(sizeof(uint32_t) * static_cast<size_t>(v.value_rows) * value_words(slice_width));
+  // head-major accumulators for gradient rows of at most 8 floats (VjpParams::symbols_by_head)
+  w.symbols_by_head = v.L.D <= kNarrowRow;
+  w.values_by_head = v.L.Dv <= kNarrowRow;
+  const size_t symbol_sums = w.symbols_by_head ? sizeof(float) * rows * v.L.D : 0;
+  w.sums_query = cursor; cursor += align_up(symbol_sums);
+  w.sums_key = cursor; cursor += align_up(symbol_sums);
+  w.sums_value = cursor;
+  cursor += align_up(w.values_by_head ? sizeof(float) * static_cast<size_t>(v.value_rows) * v.L.Dv : 0);
   // Chunk records written by the row-statistics pass for the gradient pass, which
   // otherwise rebuilds the evidence with forward sweeps of its own and evaluates the
   // dropout hash a second time.
@@ -3073,6 +3145,12 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   const int full_width = L.Dv;
   const int64_t symbol_elements = view.symbol_rows * L.D;
   const int64_t value_elements = view.value_rows * full_width;
+  float* sum_query = grad_query != nullptr && w.symbols_by_head ? at<float>(workspace, w.sums_query)
+                                                                : grad_query;
+  float* sum_key = grad_key != nullptr && w.symbols_by_head ? at<float>(workspace, w.sums_key)
+                                                            : grad_key;
+  float* sum_value = grad_value != nullptr && w.values_by_head ? at<float>(workspace, w.sums_value)
+                                                               : grad_value;
   stage_begin(kStagePrepare, stream);
   for (int value_offset = 0; value_offset < full_width; value_offset += kValueSlice) {
     L.Dv = std::min(kValueSlice, full_width - value_offset);
@@ -3114,7 +3192,8 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
           blocks_for(prepare.ballot ? view.value_rows * L.Dv : view.value_rows, 256);
       prepare.stats_blocks = blocks_for(view.symbol_rows, 256);
       if (value_offset == 0) {  // the gradient buffers are cleared once, before the first slice
-        float* buffers[3] = {grad_query, grad_key, grad_value};
+        // what the gradient kernel adds into: the tensors, or the head-major accumulators
+        float* buffers[3] = {sum_query, sum_key, sum_value};
         const int64_t lengths[3] = {symbol_elements, symbol_elements, value_elements};
         int64_t largest = 0;
         for (int part = 0; part < 3; ++part) {
@@ -3167,9 +3246,11 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     }
     P.gradient_mask = gradient_mask;
     P.dvp = dvp;
-    P.grad_query = grad_query;
-    P.grad_key = grad_key;
-    P.grad_value = grad_value;
+    P.grad_query = sum_query;
+    P.grad_key = sum_key;
+    P.grad_value = sum_value;
+    P.symbols_by_head = w.symbols_by_head ? 1 : 0;
+    P.values_by_head = w.values_by_head ? 1 : 0;
     P.work_counter = counter;
     P.header = at<int32_t>(workspace, w.header);
     P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
@@ -3194,10 +3275,16 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
   }  // value slices
   const int64_t finalize_items = std::max(symbol_elements, value_elements);
   stage_begin(kStageFinalize, stream);
+  HeadMajorSums sums;
+  sums.query = sum_query != grad_query ? sum_query : nullptr;
+  sums.key = sum_key != grad_key ? sum_key : nullptr;
+  sums.value = sum_value != grad_value ? sum_value : nullptr;
+  sums.H = L.H; sums.Hv = L.Hv; sums.D = L.D; sums.Dv = full_width;
+  sums.T = L.T; sums.N = L.N; sums.varlen = L.varlen ? 1 : 0;
   hipLaunchKernelGGL(finalize_gradients_kernel<DTYPE>, dim3(blocks_for(finalize_items, 256)),
                      dim3(256), 0, stream, query, key, value, grad_query, grad_key, grad_value,
                      symbol_elements, value_elements,
-                     L.varlen ? at<const int32_t>(workspace, w.header) : nullptr);
+                     L.varlen ? at<const int32_t>(workspace, w.header) : nullptr, sums);
   stage_end(kStageFinalize, stream);
   const hipError_t launch = hipGetLastError();
   if (launch != hipSuccess) return fail_hip(launch, "surrogate vjp launch");
