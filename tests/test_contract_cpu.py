@@ -240,6 +240,40 @@ def test_c_abi_library_exports_every_declared_symbol():
     assert b"[1, 32]" in loaded.rosa_hip_last_error()
 
 
+def test_gradient_launch_plan_follows_the_shape():
+    """Host arithmetic of the gradient kernel's launch form (no device call): blocks of two
+    waves where the tiles are wide and bands outnumber the resident waves, the row queue
+    only while a block stays within its LDS share, and the process-wide override."""
+
+    def plan(dtype, lead, D, Hv, Dv, W):
+        query = torch.empty(*lead, D, dtype=dtype)
+        value = torch.empty(*lead[:-1], Hv, Dv, dtype=dtype)
+        return cabi.gradient_block_plan(query, value, W)
+
+    metric = plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128)
+    assert metric["waves"] == 1 and not metric["row_queue"]
+    config3 = plan(torch.bfloat16, (4, 4096, 32), 16, 32, 64, 32)
+    assert config3["waves"] == 2 and config3["row_queue"]
+    assert config3["lds_bytes"] <= 40 * 1024
+    # float32 inputs of the same shape stage three terms per element: the queue no longer
+    # fits the block's LDS share, the two waves stay
+    wide = plan(torch.float32, (4, 4096, 32), 16, 32, 64, 32)
+    assert wide["waves"] in (1, 2) and wide["lds_bytes"] <= 64 * 1024
+    if wide["waves"] == 2:
+        assert not wide["row_queue"] or wide["lds_bytes"] <= 40 * 1024
+    small = plan(torch.bfloat16, (1, 1024, 4), 16, 4, 64, 32)  # 64 bands: one wave each
+    assert small["waves"] == 1
+    try:
+        cabi.set_gradient_block_waves(2)
+        forced = plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128)
+        assert forced["waves"] == 2
+        cabi.set_gradient_block_waves(1)
+        assert plan(torch.bfloat16, (4, 4096, 32), 16, 32, 64, 32)["waves"] == 1
+    finally:
+        cabi.set_gradient_block_waves(None)
+    assert plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128) == metric
+
+
 def test_no_product_module_imports_the_oracle():
     package = os.path.join(ROOT, "rosa_soft_amd")
     for name in os.listdir(package):

@@ -253,6 +253,9 @@ PACKED_CASES = [
     ([1, 2, 127, 0, 128, 129], 2, 4, 2, 5, 160, 0.0, torch.float32),
     ([64, 65, 63], 4, 8, 2, 8, 16, 0.2, torch.bfloat16),
     ([300, 40, 0, 0, 513], 2, 2, 1, 33, 32, 0.1, torch.float16),
+    # single-token sequences between longer ones, odd starts: the head-major accumulators of
+    # narrow gradient rows (two neighbouring rows per atomic segment, rows stored one slot down)
+    ([1, 1, 67, 1, 3, 130], 3, 8, 1, 8, 8, 0.2, torch.float32),
 ]
 
 
@@ -583,3 +586,18 @@ def test_backward_without_chunk_records_recomputes_to_the_same_gradients(
     # both ways of getting the state give the same gradients up to summation order
     for got, expected in zip(without, with_records):
         assert_gradients_close(got, expected.cpu())
+
+
+def test_atomic_rate_measurement_is_plausible_and_checks_its_arguments(cabi):
+    """The measurement behind the gradient kernel's second bound: float atomics in the flush
+    pattern (16 rows of a tile per step) run at some tens of G row segments per second on
+    an MI355X whatever the number of live columns; bad arguments are refused with a status."""
+
+    full = cabi.measure_atomic_rate(512, 16)
+    half = cabi.measure_atomic_rate(512, 8)
+    assert 2e9 < full < 2e11, full
+    assert 0.5 < half / full < 2.0, (half, full)  # segments, not lanes, bound the rate
+    with pytest.raises(RuntimeError, match="row_floats"):
+        cabi.measure_atomic_rate(8, 8)
+    with pytest.raises(RuntimeError, match="columns"):
+        cabi.measure_atomic_rate(512, 17)
