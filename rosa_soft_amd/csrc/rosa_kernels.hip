@@ -1193,15 +1193,15 @@ __device__ __forceinline__ v4f mfma_bf16(v4u a, v4u b, v4f c) {
                                                  __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
 }
 
-// [leading | rest << 16] of a float: its upper 16 bits and the bfloat16 nearest to what
-// they leave.  Adjacent k indices of a matrix operand, so that a product with an
+// [leading | rest << 16] of a float: the bfloat16 nearest to it and the bfloat16 nearest to
+// what that leaves.  Adjacent k indices of a matrix operand, so that a product with an
 // operand that repeats its element for both gives x (to 2^-17) times that element.
 __device__ __forceinline__ uint32_t split_bf16(float x) {
   typedef float v2f __attribute__((ext_vector_type(2)));
   typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-  // leading term by truncation (its conversion below is exact), the rest rounded: the
-  // pair keeps x to 2^-16, with three simple instructions and one conversion
-  const float head = __uint_as_float(__float_as_uint(x) & 0xffff0000u);
+  // leading term rounded half up on the upper 16 bits (its conversion below is exact), the
+  // rest rounded by the conversion: |x - pair| <= 2^-9 * 2^-8 |x|, without a bias
+  const float head = __uint_as_float((__float_as_uint(x) + 0x8000u) & 0xffff0000u);
   const v2f parts = {head, x - head};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(parts, v2bf));
 }
@@ -1209,7 +1209,8 @@ __device__ __forceinline__ uint32_t split_bf16(float x) {
 // Three-term split of a float by truncation: x = leading + middle + rest to 2^-21 of |x|
 // (each term takes the upper 16 bits of what the terms before it leave; the subtractions
 // are exact).  Returns [leading | middle << 16]; `rest` receives the third term in the
-// upper half of its bits.
+// upper half of its bits.  (Rounding the third term instead changed no measured error: the
+// gate adjoints' own float32 recurrence is what limits dQ and dK.)
 __device__ __forceinline__ uint32_t split_bf16_exact(float x, uint32_t& rest) {
   const uint32_t leading = __float_as_uint(x) & 0xffff0000u;
   const float after_leading = x - __uint_as_float(leading);
