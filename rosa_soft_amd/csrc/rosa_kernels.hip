@@ -107,12 +107,14 @@ __device__ __forceinline__ float dpp_row_shr8(float keep, float src) {
                                                     0x118, 0xf, 0xf, false));
 }
 
-// The band kernels run one wavefront per block.  LDS instructions of one wave execute in
-// order, so data written by one lane is visible to another lane's later read without a
-// barrier; what is needed is that the compiler keeps the order, and nothing else: a full
-// __syncthreads() would also wait for every outstanding global store and atomic.
+// The band kernels run one wavefront per block (or waves that meet at barriers of their
+// own).  LDS instructions of one wave execute in order, so data written by one lane is
+// visible to another lane's later read without a barrier and without a wait; what is needed
+// is that the compiler keeps the order of the accesses, and nothing else: a
+// __syncthreads() would also wait for every outstanding global store and atomic, and an
+// s_waitcnt here would expose an LDS round trip at every phase of a chunk.
 __device__ __forceinline__ void wave_lds_fence() {
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  asm volatile("" ::: "memory");
 }
 
 // Meeting point of the waves of a block that exchange data through LDS only: the LDS
@@ -1333,6 +1335,76 @@ __device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad
   }
 }
 
+// utility_tile with the five column tiles taken through each stage together (sign words,
+// table entries, matrix products, stores): the LDS and matrix latencies of one tile are
+// covered by the others instead of adding up, at the price of twenty more live registers,
+// which the kernels have for some tile widths only.
+template <int NVW, int DVP, bool BY_COLUMN>
+__device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, int grad_pitch,
+                                                     int k_blocks, const uint32_t* value_columns,
+                                                     const uint32_t* sign_table, float* out,
+                                                     int pitch, float* discard, int lane) {
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  const uint16_t* a_row = grad_tile + li * grad_pitch + 8 * lg;
+  uint32_t words[5][NVW];
+#pragma unroll
+  for (int m = 0; m < 5; ++m) {
+#pragma unroll
+    for (int w = 0; w < NVW; ++w) words[m][w] = value_columns[(16 * m + li) * NVW + w];
+  }
+  v4f acc[5];
+#pragma unroll
+  for (int m = 0; m < 5; ++m) acc[m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  constexpr int kBlocksMax = grad_term_pitch(kMaxGradTerms, DVP) / 32;
+#pragma unroll
+  for (int q = 0; q < kBlocksMax; ++q) {
+    if (q > 0 && q >= k_blocks) break;  // wave-uniform; there is always a first block
+    const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
+    const int d0 = (32 * q + 8 * lg) & (DVP - 1);
+    v4u signs[5];
+#pragma unroll
+    for (int m = 0; m < 5; ++m) {
+      uint32_t word = words[m][0];
+      if constexpr (NVW > 1) word = d0 >= 32 ? words[m][1] : words[m][0];
+      const uint32_t byte = word >> (d0 & 31);
+      const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
+      const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
+      signs[m] = v4u{low.x, low.y, high.x, high.y};
+    }
+#pragma unroll
+    for (int m = 0; m < 5; ++m) {
+      acc[m] = BY_COLUMN ? mfma_bf16(signs[m], a, acc[m]) : mfma_bf16(a, signs[m], acc[m]);
+    }
+  }
+  // wait states of the matrix results, once for all five (see utility_tile)
+  asm volatile("s_nop 7\n\ts_nop 3"
+               : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]));
+#pragma unroll
+  for (int m = 0; m < 5; ++m) {
+    if constexpr (BY_COLUMN) {
+      const int r = li;
+      const int c = 16 * m + 4 * lg;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (m == 0 && c + e < r + 1) acc[m][e] = 0.0f;
+        if (m == 4 && c + e > r + kWave) acc[m][e] = 0.0f;
+      }
+      *reinterpret_cast<v4f*>(out + r * pitch + c) = acc[m];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int r = 4 * lg + e;
+        const int l = 64 - (16 * m + li) + r;
+        float* target = out + r * pitch + l;
+        if (m == 0) target = l < kWave ? target : discard + lane;
+        if (m == 4) target = l >= 0 ? target : discard + lane;
+        *target = acc[m][e];
+      }
+    }
+  }
+}
+
 template <int NVW, bool VARLEN>
 __device__ __forceinline__ bool make_view(const VjpParams& P, const Unit& u, BandView& view,
                                           int& value_head) {
@@ -1415,14 +1487,17 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
 __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, int lane) {
   const int li = lane & 15;
   const int lg = lane >> 4;
-  v4f sums = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  // a lane adds its 16 columns (four aligned 16-byte words of row li) and one product with a
+  // matrix of ones adds the four lanes of a row: float32 matrix instructions keep the
+  // vector pipe of the SIMD waiting, so there is one per tile, not one per word
+  float partial = 0.0f;
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) {
     const float4 part =
         *reinterpret_cast<const float4*>(tile_rows + li * pitch + 16 * ks + 4 * lg);
-    sums = mfma_16x16x4((part.x + part.y) + (part.z + part.w), 1.0f, sums);
+    partial += (part.x + part.y) + (part.z + part.w);
   }
-  return sums;
+  return mfma_16x16x4(partial, 1.0f, v4f{0.0f, 0.0f, 0.0f, 0.0f});
 }
 
 // Row-statistics pass: denominator and expected dropped utility of every row.
@@ -1560,9 +1635,17 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
-        utility_tile<NVW, DVP>(grads + local * grad_lds_pitch, grad_lds_pitch, P.grad_pitch / 32,
-                               value_columns + local * NVW, sign_table, utilities, kUtilityPitch,
-                               discard, lane);
+        // (the narrowest tile runs three waves per SIMD, the widest has no registers left)
+        if constexpr (DVP == 16 || DVP == 32 || DVP == 8) {
+          utility_tiles_staged<NVW, DVP, false>(grads + local * grad_lds_pitch, grad_lds_pitch,
+                                                P.grad_pitch / 32, value_columns + local * NVW,
+                                                sign_table, utilities, kUtilityPitch, discard,
+                                                lane);
+        } else {
+          utility_tile<NVW, DVP>(grads + local * grad_lds_pitch, grad_lds_pitch,
+                                 P.grad_pitch / 32, value_columns + local * NVW, sign_table,
+                                 utilities, kUtilityPitch, discard, lane);
+        }
         wave_lds_fence();
       }
       uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
@@ -2314,8 +2397,15 @@ void vjp_gradients_kernel(VjpParams P) {
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
-          utility_tile<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32, value_window + local * NVW,
-                                 sign_table, tile, kTilePitch, discard, lane);
+          if constexpr (DVP <= 32) {  // the widest tile has no registers for it (measured slower)
+            utility_tiles_staged<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32,
+                                                 value_window + local * NVW, sign_table, tile,
+                                                 kTilePitch, discard, lane);
+          } else {
+            utility_tile<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32,
+                                         value_window + local * NVW, sign_table, tile, kTilePitch,
+                                         discard, lane);
+          }
           wave_lds_fence();
         }
         issue_pending();
@@ -2436,12 +2526,32 @@ void vjp_gradients_kernel(VjpParams P) {
           }
         };
         if (want_v) {
-          v4u weights[kWindowTiles];
-          column_operands(weights);
           // the other factor: grad_output of the same rows, term by term, each element
           // repeated for the two terms of the weight (the third term of a float32
-          // grad_output is below the accuracy of the split weights and is left out)
+          // grad_output is below the accuracy of the split weights and is left out).
+          // Where registers allow, every LDS read of the section is issued before the first
+          // is used: one latency instead of one per operand.
           const int terms = P.grad_terms < 2 ? P.grad_terms : 2;
+          constexpr bool kReadsFirst = VT <= 2;
+          uint32_t elements[VT][2][4];
+          if constexpr (kReadsFirst) {
+#pragma unroll
+            for (int n = 0; n < VT; ++n) {
+              const int d = 16 * n + li;
+              const uint16_t* source = grad_tile + (4 * lg) * GP + (d < DVP ? d : DVP - 1);
+#pragma unroll
+              for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  // a second term that does not exist is read from the first and not used
+                  elements[n][t][j] = source[j * GP + (t < terms ? t : 0) * DVP];
+                }
+              }
+            }
+          }
+          v4u weights[kWindowTiles];
+          column_operands(weights);
+          if constexpr (kReadsFirst) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int n = 0; n < VT; ++n) {
             const int d = 16 * n + li;
@@ -2452,7 +2562,8 @@ void vjp_gradients_kernel(VjpParams P) {
               v4u grads;
 #pragma unroll
               for (int j = 0; j < 4; ++j) {
-                const uint32_t element = source[j * GP + t * DVP];
+                const uint32_t element =
+                    kReadsFirst ? elements[n][t][j] : uint32_t(source[j * GP + t * DVP]);
                 grads[j] = d < DVP ? element | (element << 16) : 0u;
               }
 #pragma unroll
@@ -2564,16 +2675,27 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
               for (int n = 0; n < DT; ++n) query_part[part][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             }
+            // every LDS read of the section is issued before the first product (one latency
+            // instead of one per step; the widest tile gains nothing from it)
+            uint4 k_words_of[kWindowTiles];
+            v4u adjoints_of[kWindowTiles];
+            v2u adjoint_rests_of[kWindowTiles];
 #pragma unroll
             for (int step = 0; step < kWindowTiles; ++step) {
-              const uint4 k_words =
-                  *reinterpret_cast<const uint4*>(key_tile + 4 * kWindowTiles * lg + 4 * step);
               // four neighbouring columns of row li: one aligned 16-byte word of the tile and
               // one aligned 8-byte word of the third terms
               const int c0 = 4 * kWindowTiles * lg + 4 * step;
-              const v4u adjoints = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
-              const v2u adjoint_rests =
+              k_words_of[step] = *reinterpret_cast<const uint4*>(key_tile + c0);
+              adjoints_of[step] = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
+              adjoint_rests_of[step] =
                   *reinterpret_cast<const v2u*>(rest_plane + li * kRestPitch + c0);
+            }
+            if constexpr (VT <= 2) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int step = 0; step < kWindowTiles; ++step) {
+              const uint4 k_words = k_words_of[step];
+              const v4u adjoints = adjoints_of[step];
+              const v2u adjoint_rests = adjoint_rests_of[step];
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
                 const int bit = 16 * n + li;
