@@ -8,12 +8,14 @@
 
 from __future__ import annotations
 
+import json
 import os
+import re
 import shlex
 import subprocess
 import sys
 import sysconfig
-from typing import List
+from typing import Dict, List
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
@@ -23,6 +25,8 @@ OFFLOAD_ARCH = "gfx950"
 HIP_SOURCE = os.path.join(HERE, "csrc", "rosa_kernels.hip")
 HIP_LIBRARY = os.path.join(HERE, "librosa_soft_hip.so")
 DISPATCH_SOURCE = os.path.join(HERE, "csrc", "rosa_dispatch.cpp")
+# registers, spills, scratch and LDS of every kernel, as the compiler reported them
+RESOURCE_REPORT = os.path.join(HERE, "kernel_resources.json")
 
 # -packed-fp32-ops is switched off on purpose: some packed-FP32 forms have
 # produced silently wrong results on this hardware generation.
@@ -38,20 +42,59 @@ def dispatcher_path() -> str:
     return os.path.join(HERE, "_C" + suffix)
 
 
-def _run(command: List[str]) -> None:
+RESOURCE_REMARK = re.compile(r"remark:\s+([A-Za-z /\[\]]+?):\s+(\S+) \[-Rpass-analysis=kernel-resource-usage\]")
+
+
+def _run(command: List[str]) -> str:
     print("+", " ".join(shlex.quote(part) for part in command), flush=True)
     completed = subprocess.run(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    noise = ("packed-fp32-ops", "is not a recognized feature")
-    lines = [line for line in completed.stdout.splitlines() if not any(n in line for n in noise)]
+    noise = ("packed-fp32-ops", "is not a recognized feature", "kernel-resource-usage")
+    lines, skip_excerpt = [], 0
+    for line in completed.stdout.splitlines():
+        if "kernel-resource-usage" in line and "Function Name" in line:
+            skip_excerpt = 2  # the remark of a function is followed by a source excerpt
+            continue
+        if skip_excerpt and re.match(r"\s+(\d+ )?\|", line):
+            skip_excerpt -= 1
+            continue
+        if not any(n in line for n in noise):
+            lines.append(line)
     if lines:
         print("\n".join(lines), flush=True)
     if completed.returncode != 0:
         raise RuntimeError(f"build step failed with exit code {completed.returncode}")
+    return completed.stdout
+
+
+def kernel_resources(compiler_output: str) -> Dict[str, Dict[str, int]]:
+    """Per kernel, what -Rpass-analysis=kernel-resource-usage reported: registers, spilled
+    registers, scratch bytes per lane, static LDS bytes."""
+
+    keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes",
+            "VGPRs Spill": "vgpr_spills", "SGPRs Spill": "sgpr_spills",
+            "LDS Size [bytes/block]": "lds_bytes", "Occupancy [waves/SIMD]": "waves_per_simd"}
+    report: Dict[str, Dict[str, int]] = {}
+    current = None
+    for name, value in RESOURCE_REMARK.findall(compiler_output):
+        name = name.strip()
+        if name == "Function Name":
+            current = report.setdefault(value, {})
+        elif current is not None and name in keys and value.isdigit():
+            current[keys[name]] = int(value)
+    return report
 
 
 def build_hip_library() -> str:
     hipcc = os.path.join(ROCM_HOME, "bin", "hipcc")
-    _run([hipcc, *HIPCC_FLAGS, HIP_SOURCE, "-o", HIP_LIBRARY])
+    output = _run([hipcc, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", HIP_SOURCE,
+                   "-o", HIP_LIBRARY])
+    report = kernel_resources(output)
+    with open(RESOURCE_REPORT, "w") as handle:
+        json.dump(report, handle, indent=0, sort_keys=True)
+    spilling = sorted(name for name, use in report.items()
+                      if use.get("vgpr_spills", 0) or use.get("scratch_bytes", 0))
+    print(f"{len(report)} kernels; spilling vector registers or using scratch: "
+          f"{spilling if spilling else 'none'}", flush=True)
     return HIP_LIBRARY
 
 

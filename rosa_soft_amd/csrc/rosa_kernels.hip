@@ -2675,27 +2675,33 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
               for (int n = 0; n < DT; ++n) query_part[part][n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             }
-            // every LDS read of the section is issued before the first product (one latency
-            // instead of one per step; the widest tile gains nothing from it)
-            uint4 k_words_of[kWindowTiles];
-            v4u adjoints_of[kWindowTiles];
-            v2u adjoint_rests_of[kWindowTiles];
-#pragma unroll
-            for (int step = 0; step < kWindowTiles; ++step) {
+            // Where registers allow, every LDS read of the section is issued before the first
+            // product (one latency instead of one per step); the widest tile reads step by step.
+            constexpr bool kReadsFirst = VT <= 2;
+            constexpr int kHeld = kReadsFirst ? kWindowTiles : 1;
+            uint4 k_words_of[kHeld];
+            v4u adjoints_of[kHeld];
+            v2u adjoint_rests_of[kHeld];
+            const auto read_step = [&](int step, int slot) {
               // four neighbouring columns of row li: one aligned 16-byte word of the tile and
               // one aligned 8-byte word of the third terms
               const int c0 = 4 * kWindowTiles * lg + 4 * step;
-              k_words_of[step] = *reinterpret_cast<const uint4*>(key_tile + c0);
-              adjoints_of[step] = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
-              adjoint_rests_of[step] =
+              k_words_of[slot] = *reinterpret_cast<const uint4*>(key_tile + c0);
+              adjoints_of[slot] = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
+              adjoint_rests_of[slot] =
                   *reinterpret_cast<const v2u*>(rest_plane + li * kRestPitch + c0);
+            };
+            if constexpr (kReadsFirst) {
+#pragma unroll
+              for (int step = 0; step < kWindowTiles; ++step) read_step(step, step);
+              __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (VT <= 2) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int step = 0; step < kWindowTiles; ++step) {
-              const uint4 k_words = k_words_of[step];
-              const v4u adjoints = adjoints_of[step];
-              const v2u adjoint_rests = adjoint_rests_of[step];
+              if constexpr (!kReadsFirst) read_step(step, 0);
+              const uint4 k_words = k_words_of[kReadsFirst ? step : 0];
+              const v4u adjoints = adjoints_of[kReadsFirst ? step : 0];
+              const v2u adjoint_rests = adjoint_rests_of[kReadsFirst ? step : 0];
 #pragma unroll
               for (int n = 0; n < DT; ++n) {
                 const int bit = 16 * n + li;

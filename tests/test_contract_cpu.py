@@ -274,6 +274,27 @@ def test_gradient_launch_plan_follows_the_shape():
     assert plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128) == metric
 
 
+def test_no_kernel_of_the_last_build_spills_or_uses_scratch():
+    """The build records what the compiler reported per kernel.  Spilled vector registers and
+    scratch memory are performance faults of the backward kernels (a reload waits behind
+    every atomic in flight): none of the instantiations may have any."""
+
+    from rosa_soft_amd import _build
+
+    if not os.path.exists(_build.RESOURCE_REPORT):
+        pytest.skip("no resource report: the library was not built by this tree's build step")
+    import json
+
+    with open(_build.RESOURCE_REPORT) as handle:
+        report = json.load(handle)
+    assert len(report) >= 100  # every instantiation of the backward kernels is listed
+    offenders = {name: use for name, use in report.items()
+                 if use.get("vgpr_spills", 0) or use.get("scratch_bytes", 0)}
+    assert not offenders, offenders
+    gradient = [use for name, use in report.items() if "vjp_gradients_kernel" in name]
+    assert gradient and all(use["vgprs"] + use.get("agprs", 0) <= 512 for use in gradient)
+
+
 def test_no_product_module_imports_the_oracle():
     package = os.path.join(ROOT, "rosa_soft_amd")
     for name in os.listdir(package):
