@@ -2217,12 +2217,13 @@ void vjp_gradients_kernel(VjpParams P) {
       }
       // one round trip brings in everything the segment needs
       wave_lds_fence();
-      constexpr bool kHeavy = VT > 2 || DT > 1;
+      // (all but the tightest variant: packed, Dv = 64, one wave per block has no registers
+      // for it and stages array by array, which took a quarter of the kernel at Dv = 64)
+      constexpr bool kHeavy = VT > 2 && VARLEN && NW == 1;
       if constexpr (!kHeavy) {
         // Every global load of the segment is issued before the first of them is used, so
         // the segment costs one memory latency (two when the grad_output rows need the
-        // registers of the other arrays), not one per staged array.  The widest tiles have
-        // no registers to spare at this point and stage array by array.
+        // registers of the other arrays), not one per staged array.
         const bool row_lane = lane < SEG;
         const int i = min(seg_first + lane, view.steps - 1);  // rows past the end repeat the last
         const int t = view.diag0 + 1 + i;
@@ -2293,16 +2294,21 @@ void vjp_gradients_kernel(VjpParams P) {
         // the grad_output rows come in groups that fit the registers free at this point
         constexpr int kGradGroup = kGradParts % 4 == 0 ? 4 : (kGradParts % 3 == 0 ? 3 : 1);
         static_assert(kGradParts % kGradGroup == 0, "whole groups");
+        // 16-byte pieces the segment really has (the terms of the input type), numbered row
+        // by row: a group of registers then never waits for pieces that do not exist
+        const int pieces = SEG * grad_chunks;
+        const float per_row = 1.0f / static_cast<float>(grad_chunks);
 #pragma unroll
         for (int group = 0; group < kGradParts; group += kGradGroup) {
+          if (group * kWave >= pieces) break;  // wave-uniform
           uint4 grad_in[kGradGroup];
 #pragma unroll
           for (int part = 0; part < kGradGroup; ++part) {
             const int index = (group + part) * kWave + lane;
-            const int r = index / kGradChunksMax;
-            const int piece = index - r * kGradChunksMax;
+            const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+            const int piece = index - r * grad_chunks;
             grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
-            if (piece < grad_chunks && seg_first + r < view.steps) {
+            if (index < pieces && seg_first + r < view.steps) {
               grad_in[part] = *reinterpret_cast<const uint4*>(
                   view.grad_rows +
                   static_cast<int64_t>(view.diag0 + 1 + seg_first + r) * P.grad_pitch + 8 * piece);
@@ -2315,9 +2321,9 @@ void vjp_gradients_kernel(VjpParams P) {
 #pragma unroll
           for (int part = 0; part < kGradGroup; ++part) {
             const int index = (group + part) * kWave + lane;
-            const int r = index / kGradChunksMax;
-            const int piece = index - r * kGradChunksMax;
-            if (piece < grad_chunks) {
+            const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+            const int piece = index - r * grad_chunks;
+            if (index < pieces) {
               *reinterpret_cast<uint4*>(grad_rows_lds + r * GP + 8 * piece) = grad_in[part];
             }
           }
