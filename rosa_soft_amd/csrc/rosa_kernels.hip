@@ -1269,76 +1269,16 @@ __device__ __forceinline__ void fill_sign_table(uint32_t* table, int lane) {
 // Utilities u(t, a) = sum_d grad_output[t, d] * sign(v[a, d]) of 16 rows against
 // their 80 window columns on the matrix cores, written in (row r, lane l)
 // coordinates: out[r * pitch + l] for the pair on diagonal lane l, whose window
-// column is c = 64 - l + r (BY_COLUMN: out[r * pitch + c], pitch a multiple of 4).  `grad_tile` holds the bfloat16 terms of the 16 grad_output
-// rows, `grad_pitch` elements each: k = term * DVP + d, `k_blocks` blocks of 32
-// (zero beyond the last term); the sum over the terms is the float32 product.
-// `value_columns` holds the sign words of the window columns (NVW per column).  Elements
-// of the first and last column tile that belong to no lane go to `discard` (one float
-// per lane).
-template <int NVW, int DVP, bool BY_COLUMN = false>
-__device__ __forceinline__ void utility_tile(const uint16_t* grad_tile, int grad_pitch,
-                                             int k_blocks, const uint32_t* value_columns,
-                                             const uint32_t* sign_table, float* out, int pitch,
-                                             float* discard, int lane) {
-  const int li = lane & 15;
-  const int lg = lane >> 4;
-  const uint16_t* a_row = grad_tile + li * grad_pitch + 8 * lg;
-#pragma unroll
-  for (int m = 0; m < 5; ++m) {
-    uint32_t words[NVW];
-#pragma unroll
-    for (int w = 0; w < NVW; ++w) words[w] = value_columns[(16 * m + li) * NVW + w];
-    v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    constexpr int kBlocksMax = grad_term_pitch(kMaxGradTerms, DVP) / 32;
-#pragma unroll
-    for (int q = 0; q < kBlocksMax; ++q) {
-      if (q > 0 && q >= k_blocks) break;  // wave-uniform; there is always a first block
-      const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
-      // this lane's k = 32 q + 8 lg .. + 7 are eight value dimensions of one term
-      const int d0 = (32 * q + 8 * lg) & (DVP - 1);
-      uint32_t word = words[0];
-      if constexpr (NVW > 1) word = d0 >= 32 ? words[1] : words[0];
-      const uint32_t byte = word >> (d0 & 31);
-      const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
-      const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
-      const v4u signs = {low.x, low.y, high.x, high.y};
-      // BY_COLUMN takes the transposed product: lane (li, lg) then holds columns
-      // 16 m + 4 lg .. + 3 of row li, four neighbours of one tile row
-      acc = BY_COLUMN ? mfma_bf16(signs, a, acc) : mfma_bf16(a, signs, acc);
-    }
-    // The product is read right behind a branch of the loop above, where the compiler has
-    // been seen to leave out the wait states a matrix result needs before vector or LDS
-    // instructions may read it (wrong utilities): they are spent here.
-    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(acc));
-    if constexpr (BY_COLUMN) {
-      // out[r][c]: one aligned 16-byte store; columns outside r + 1 .. r + 64 belong to no
-      // lane and stay zero
-      const int r = li;
-      const int c = 16 * m + 4 * lg;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (m == 0 && c + e < r + 1) acc[e] = 0.0f;
-        if (m == 4 && c + e > r + kWave) acc[e] = 0.0f;
-      }
-      *reinterpret_cast<v4f*>(out + r * pitch + c) = acc;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int r = 4 * lg + e;
-        const int l = 64 - (16 * m + li) + r;
-        float* target = out + r * pitch + l;
-        if (m == 0) target = l < kWave ? target : discard + lane;
-        if (m == 4) target = l >= 0 ? target : discard + lane;
-        *target = acc[e];
-      }
-    }
-  }
-}
-
-// utility_tile with the five column tiles taken through each stage together (sign words,
-// table entries, matrix products, stores): the LDS and matrix latencies of one tile are
-// covered by the others instead of adding up, at the price of twenty more live registers,
-// which the kernels have for some tile widths only.
+// column is c = 64 - l + r (BY_COLUMN: out[r * pitch + c], pitch a multiple of 4).
+// `grad_tile` holds the bfloat16 terms of the 16 grad_output rows, `grad_pitch` elements
+// each: k = term * DVP + d, `k_blocks` blocks of 32 (zero beyond the last term); the sum
+// over the terms is the float32 product.  `value_columns` holds the sign words of the
+// window columns (NVW per column).  Elements of the first and last column tile that
+// belong to no lane go to `discard` (one float per lane).
+// The five column tiles are taken through each stage together (sign words, table entries,
+// matrix products, stores): the LDS and matrix latencies of one tile are covered by the
+// others instead of adding up (one tile after the other took 13 % of the gradient kernel,
+// together 7 %), at the price of twenty more live registers.
 template <int NVW, int DVP, bool BY_COLUMN>
 __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, int grad_pitch,
                                                      int k_blocks, const uint32_t* value_columns,
@@ -1347,11 +1287,13 @@ __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, 
   const int li = lane & 15;
   const int lg = lane >> 4;
   const uint16_t* a_row = grad_tile + li * grad_pitch + 8 * lg;
-  uint32_t words[5][NVW];
+  // (two arrays, not one indexed by the word: a select between elements of one array
+  // becomes a dynamic index, and the array then lives in scratch memory)
+  uint32_t low_words[5], high_words[5];
 #pragma unroll
   for (int m = 0; m < 5; ++m) {
-#pragma unroll
-    for (int w = 0; w < NVW; ++w) words[m][w] = value_columns[(16 * m + li) * NVW + w];
+    low_words[m] = value_columns[(16 * m + li) * NVW];
+    high_words[m] = NVW > 1 ? value_columns[(16 * m + li) * NVW + NVW - 1] : 0u;
   }
   v4f acc[5];
 #pragma unroll
@@ -1365,8 +1307,8 @@ __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, 
     v4u signs[5];
 #pragma unroll
     for (int m = 0; m < 5; ++m) {
-      uint32_t word = words[m][0];
-      if constexpr (NVW > 1) word = d0 >= 32 ? words[m][1] : words[m][0];
+      uint32_t word = low_words[m];
+      if constexpr (NVW > 1) word = d0 >= 32 ? high_words[m] : low_words[m];
       const uint32_t byte = word >> (d0 & 31);
       const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
       const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
@@ -1377,7 +1319,9 @@ __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, 
       acc[m] = BY_COLUMN ? mfma_bf16(signs[m], a, acc[m]) : mfma_bf16(a, signs[m], acc[m]);
     }
   }
-  // wait states of the matrix results, once for all five (see utility_tile)
+  // The products are read right behind a branch of the loop above, where the compiler has
+  // been seen to leave out the wait states a matrix result needs before vector or LDS
+  // instructions may read it (wrong utilities): they are spent here, once for all five.
   asm volatile("s_nop 7\n\ts_nop 3"
                : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]));
 #pragma unroll
@@ -1635,17 +1579,9 @@ __global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
       float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
-        // (the narrowest tile runs three waves per SIMD, the widest has no registers left)
-        if constexpr (DVP == 16 || DVP == 32 || DVP == 8) {
-          utility_tiles_staged<NVW, DVP, false>(grads + local * grad_lds_pitch, grad_lds_pitch,
-                                                P.grad_pitch / 32, value_columns + local * NVW,
-                                                sign_table, utilities, kUtilityPitch, discard,
-                                                lane);
-        } else {
-          utility_tile<NVW, DVP>(grads + local * grad_lds_pitch, grad_lds_pitch,
-                                 P.grad_pitch / 32, value_columns + local * NVW, sign_table,
-                                 utilities, kUtilityPitch, discard, lane);
-        }
+        utility_tiles_staged<NVW, DVP, false>(grads + local * grad_lds_pitch, grad_lds_pitch,
+                                              P.grad_pitch / 32, value_columns + local * NVW,
+                                              sign_table, utilities, kUtilityPitch, discard, lane);
         wave_lds_fence();
       }
       uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
@@ -2403,15 +2339,9 @@ void vjp_gradients_kernel(VjpParams P) {
         // The one [row][lane] tile holds, in turn, the chunk's utilities, its route
         // weights d*p and its gate adjoints h; each pair's slot is replaced in place.
         if (want_qk) {
-          if constexpr (DVP <= 32) {  // the widest tile has no registers for it (measured slower)
-            utility_tiles_staged<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32,
-                                                 value_window + local * NVW, sign_table, tile,
-                                                 kTilePitch, discard, lane);
-          } else {
-            utility_tile<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32,
-                                         value_window + local * NVW, sign_table, tile, kTilePitch,
-                                         discard, lane);
-          }
+          utility_tiles_staged<NVW, DVP, true>(grad_tile, GP, P.grad_pitch / 32,
+                                               value_window + local * NVW, sign_table, tile,
+                                               kTilePitch, discard, lane);
           wave_lds_fence();
         }
         issue_pending();
