@@ -1451,7 +1451,8 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 // each from 16 lanes; every lane keeps its 16 dropout decisions of the chunk as bits and
 // stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
-__global__ __launch_bounds__(kWave) void vjp_row_stats_kernel(VjpParams P) {
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(DVP == 8 ? 3 : 1)))
+void vjp_row_stats_kernel(VjpParams P) {
   constexpr int kBlockRows = 32;     // rows staged in LDS at a time
   constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
   constexpr int kWeightPitch = 68;
