@@ -1451,7 +1451,7 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 // each from 16 lanes; every lane keeps its 16 dropout decisions of the chunk as bits and
 // stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(DVP == 8 ? 3 : 1)))
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(DVP <= 32 ? 3 : 1)))
 void vjp_row_stats_kernel(VjpParams P) {
   constexpr int kBlockRows = 32;     // rows staged in LDS at a time
   constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
@@ -1518,23 +1518,44 @@ void vjp_row_stats_kernel(VjpParams P) {
         symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
         stat = view.stats[t];
       }
+      // The grad_output rows come as 16-byte pieces, numbered row by row over the pieces the
+      // input type really has, in groups of at most two registers per lane: the first group
+      // travels with the other loads of the block, later ones (float32 rows of wider tiles)
+      // take a round trip of their own instead of the registers the chunk loop needs.
       constexpr int kGradParts = (kBlockRows * kGradChunksMax + kWave - 1) / kWave;
+      constexpr int kGradGroup = kGradParts < 2 ? kGradParts : 2;
       constexpr int kValueParts = ((kBlockRows + kWave) * NVW + kWave - 1) / kWave;
-      uint4 grad_in[kGradParts];
+      const int pieces = kBlockRows * grad_chunks;
+      const float per_row = 1.0f / static_cast<float>(grad_chunks);
+      uint4 grad_in[kGradGroup];
       uint32_t value_in[kValueParts];
-      if (needs_utility) {
+      const auto load_pieces = [&](int group) {
 #pragma unroll
-        for (int part = 0; part < kGradParts; ++part) {
-          const int index = part * kWave + lane;
-          const int r = index / kGradChunksMax;
-          const int piece = index - r * kGradChunksMax;
+        for (int part = 0; part < kGradGroup; ++part) {
+          const int index = (group + part) * kWave + lane;
+          const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+          const int piece = index - r * grad_chunks;
           grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
-          if (r < kBlockRows && piece < grad_chunks && first + r < view.steps) {
+          if (index < pieces && first + r < view.steps) {
             grad_in[part] = *reinterpret_cast<const uint4*>(
                 view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * P.grad_pitch +
                 8 * piece);
           }
         }
+      };
+      const auto store_pieces = [&](int group) {
+#pragma unroll
+        for (int part = 0; part < kGradGroup; ++part) {
+          const int index = (group + part) * kWave + lane;
+          const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+          const int piece = index - r * grad_chunks;
+          if (index < pieces) {
+            *reinterpret_cast<uint4*>(grads + r * grad_lds_pitch + 8 * piece) = grad_in[part];
+          }
+        }
+      };
+      if (needs_utility) {
+        load_pieces(0);
 #pragma unroll
         for (int part = 0; part < kValueParts; ++part) {
           const int index = part * kWave + lane;
@@ -1551,20 +1572,19 @@ void vjp_row_stats_kernel(VjpParams P) {
         row_words[1] = make_uint4(__float_as_uint(fmaf(stat.x, kLog2e, stat.w)), 0u, 0u, 0u);
       }
       if (needs_utility) {
-#pragma unroll
-        for (int part = 0; part < kGradParts; ++part) {
-          const int index = part * kWave + lane;
-          const int r = index / kGradChunksMax;
-          const int piece = index - r * kGradChunksMax;
-          if (r < kBlockRows && piece < grad_chunks) {
-            *reinterpret_cast<uint4*>(grads + r * grad_lds_pitch + 8 * piece) = grad_in[part];
-          }
-        }
+        store_pieces(0);
 #pragma unroll
         for (int part = 0; part < kValueParts; ++part) {
           if (part * kWave + lane < (kBlockRows + kWave) * NVW) {
             value_columns[part * kWave + lane] = value_in[part];
           }
+        }
+#pragma unroll
+        for (int group = kGradGroup; group < kGradParts; group += kGradGroup) {
+          if (group * kWave >= pieces) break;  // wave-uniform
+          load_pieces(group);
+          __builtin_amdgcn_sched_barrier(0);
+          store_pieces(group);
         }
       }
     }
