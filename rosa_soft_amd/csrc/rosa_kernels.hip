@@ -160,6 +160,16 @@ __device__ __forceinline__ uint32_t in_vector_register(uint32_t uniform) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+
+// popcount(x) + addend in the one instruction the hardware has for it.  (Written out because
+// the compiler turns an addend whose set bits lie above the count into an `or` and then no
+// longer finds the instruction's own addend.)
+__device__ __forceinline__ uint32_t popc_plus(uint32_t x, uint32_t addend) {
+  uint32_t result;
+  asm("v_bcnt_u32_b32 %0, %1, %2" : "=v"(result) : "v"(x), "v"(addend));
+  return result;
+}
 
 template <int DTYPE>
 __device__ __forceinline__ float load_as_float(const void* base, int64_t index) {
@@ -1093,6 +1103,13 @@ __device__ __forceinline__ RowSymbols staged_symbols(const uint32_t* row) {
 // of the plain product.
 constexpr int kCountBias = 0x3f800000;
 
+// popcount(x) + kCountBias: the bias is the inline constant 1.0 of the instruction
+__device__ __forceinline__ int biased_popc(uint32_t x) {
+  int result;
+  asm("v_bcnt_u32_b32 %0, %1, 1.0" : "=v"(result) : "v"(x));
+  return result;
+}
+
 __device__ __forceinline__ float decay_of_biased_count(int biased, float gate_log2) {
   const float slope = gate_log2 * 8388608.0f;
   return fast_exp2(fmaf(__int_as_float(biased), -slope, slope));
@@ -1112,22 +1129,21 @@ __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbol
   band.key_word = dpp_wave_shr1(symbols.key, band.key_word);
   StepOut out;
   out.a = a0 - lane;
-  const int mismatches = __popc(symbols.query ^ band.key_word);
-  const auto window_decay = [&]() {
-    return BIASED ? decay_of_biased_count(band.window, gate_log2)
-                  : fast_exp2(-gate_log2 * static_cast<float>(band.window));
-  };
-  const float gate = (BIASED || (STEADY && QUIET))
-      ? decay_of_biased_count(mismatches + kCountBias, gate_log2)
-      : fast_exp2(-gate_log2 * static_cast<float>(mismatches));
   if constexpr (STEADY && QUIET) {
     out.active = true;
-    out.gate = gate;
+    out.gate = decay_of_biased_count(biased_popc(symbols.query ^ band.key_word), gate_log2);
     out.overflow = 0.0f;
     band.evidence = fmaf(out.gate, band.evidence, out.gate);
     out.evidence = band.evidence;
     return out;
   }
+  const int mismatches = __popc(symbols.query ^ band.key_word);
+  const auto window_decay = [&]() {
+    return BIASED ? decay_of_biased_count(band.window, gate_log2)
+                  : fast_exp2(-gate_log2 * static_cast<float>(band.window));
+  };
+  const float gate = BIASED ? decay_of_biased_count(mismatches + kCountBias, gate_log2)
+                            : fast_exp2(-gate_log2 * static_cast<float>(mismatches));
   band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
   if constexpr (STEADY) {
     out.active = true;
@@ -1423,6 +1439,18 @@ __global__ __launch_bounds__(kWave) void vjp_row_max_kernel(VjpParams P) {
   }
 }
 
+// 2 * bits + (flag ? 1 : 0) as one add with carry (the compiler builds a select, a shift and
+// an or from the plain expression).
+__device__ __forceinline__ uint32_t doubled_plus_flag(uint32_t bits, bool flag) {
+  const uint64_t carry_in = __builtin_amdgcn_ballot_w64(flag);
+  uint64_t carry_out;
+  uint32_t result;
+  asm("v_addc_co_u32_e64 %0, %1, %2, %2, %3"
+      : "=v"(result), "=s"(carry_out)
+      : "v"(bits), "s"(carry_in));
+  return result;
+}
+
 // Sum of every row of a [16][pitch] LDS tile over its 64 columns: each lane adds four
 // neighbouring columns (one 16-byte read), and the matrix cores add the 16 partial sums
 // of a row (the partial sums times a matrix of ones).  `pitch` is a multiple of 4 floats.
@@ -1615,6 +1643,9 @@ void vjp_row_stats_kernel(VjpParams P) {
         // entering and the leaving mismatches are summed and applied after the chunk.
         constexpr bool QUIET = decltype(quiet_tag)::value;
         uint32_t entering = 0u, leaving = 0u;
+        // quiet chunks carry 1 + S: one fused multiply-add per row, and the root below
+        // needs no addition (the weight only sees S through sqrt(1 + S) anyway)
+        float one_plus_evidence = 1.0f + band.evidence;
         const uint32_t* row = rows + local * kRowWords;
         uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
         float next_shift = __uint_as_float(row[4]);
@@ -1636,33 +1667,44 @@ void vjp_row_stats_kernel(VjpParams P) {
             band.key_word = dpp_wave_shr1(symbols.key, band.key_word);
             band.old_key_word = dpp_wave_shr1(symbols.old_key, band.old_key_word);
             const uint32_t differing = symbols.query ^ band.key_word;
-            const float gate =
-                decay_of_biased_count(__popc(differing) + kCountBias, P.gate_log2);
-            band.evidence = fmaf(gate, band.evidence, gate);
-            entering += __popc(differing);
-            leaving += __popc(symbols.old_query ^ band.old_key_word);
-            s.evidence = band.evidence;
+            const float gate = decay_of_biased_count(biased_popc(differing), P.gate_log2);
+            one_plus_evidence = fmaf(gate, one_plus_evidence, 1.0f);
+            entering = popc_plus(differing, entering);
+            leaving = popc_plus(symbols.old_query ^ band.old_key_word, leaving);
             s.active = true;
           } else {
             s = forward_step<NVW, STEADY, false, true>(band, symbols, i, lane, W, P.gate_log2);
             peak_overflow = fmaxf(peak_overflow, s.overflow);
           }
-          const float one_plus = 1.0f + s.evidence;
-          const float root = one_plus * fast_rsq(one_plus);
+          // (outside quiet chunks the root is formed exactly as the gradient pass forms it:
+          // with long matches the logits are large, and a last-bit difference between the
+          // two passes' roots would show in the normalisation)
+          float root;
+          if constexpr (QUIET) {
+            root = fast_sqrt(one_plus_evidence);
+          } else {
+            const float one_plus = 1.0f + s.evidence;
+            root = one_plus * fast_rsq(one_plus);
+          }
           const bool live = STEADY || (s.active && r < rows_here);
           const float weight = live ? fast_exp2(fmaf(root, logit_gain, -shift)) : 0.0f;
-          float keep = 1.0f;
+          // (the factor 1 / (1 - p) of the kept pairs is applied to the row sums)
+          float dropped_utility = weight * utility;
           if constexpr (DROPOUT) {
             route_hash = dpp_wave_shr1(route_hash_of(i + 1), route_hash);
             set_row(key, t);
             const bool kept = dropout_keeps(key, route_hash);
-            keep = kept ? P.inverse_keep : 0.0f;
-            kept_bits |= kept ? (1u << r) : 0u;
+            dropped_utility = kept ? dropped_utility : 0.0f;
+            kept_bits = doubled_plus_flag(kept_bits, kept);  // rows end up in reverse order
           }
           weights[r * kWeightPitch + lane] = weight;
-          utilities[r * kUtilityPitch + lane] = weight * keep * utility;
+          utilities[r * kUtilityPitch + lane] = dropped_utility;
         }
-        if constexpr (QUIET) band.window += static_cast<int>(entering - leaving);
+        if constexpr (QUIET) {
+          band.window += static_cast<int>(entering - leaving);
+          band.evidence = one_plus_evidence - 1.0f;  // exact: 1 <= 1 + S
+        }
+        if constexpr (DROPOUT) kept_bits = __builtin_bitreverse32(kept_bits) >> 16;  // bit r: row r
       };
       if (chunk_first >= W + kWave && rows_here == kChunk) {
         // a window loses at most D mismatches per row
@@ -1689,7 +1731,9 @@ void vjp_row_stats_kernel(VjpParams P) {
                                     : e == 2 ? numerator_sums[2] : numerator_sums[3];
           float4* row_stats = view.stats + (view.diag0 + 1 + chunk_first + r);
           atomicAdd(&row_stats->y, weight_sum);
-          if (needs_utility) atomicAdd(&row_stats->z, numerator_sum);
+          if (needs_utility) {
+            atomicAdd(&row_stats->z, DROPOUT ? numerator_sum * P.inverse_keep : numerator_sum);
+          }
         }
       }
       if (view.checkpoints != nullptr) {
