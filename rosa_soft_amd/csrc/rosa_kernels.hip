@@ -1456,8 +1456,9 @@ __device__ __forceinline__ uint32_t doubled_plus_flag(uint32_t bits, bool flag) 
 // of a row (the partial sums times a matrix of ones).  `pitch` is a multiple of 4 floats.
 // Lane (li, lg) = (lane & 15, lane >> 4) returns with the sums of rows 4 lg + e in
 // element e, whatever li.
+template <int ROWS>
 __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, int lane) {
-  const int li = lane & 15;
+  const int li = lane & (ROWS - 1);  // a tile of eight rows repeats in the product
   const int lg = lane >> 4;
   // a lane adds its 16 columns (four aligned 16-byte words of row li) and one product with a
   // matrix of ones adds the four lanes of a row: float32 matrix instructions keep the
@@ -1481,7 +1482,9 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(DVP <= 32 ? 3 : 1)))
 void vjp_row_stats_kernel(VjpParams P) {
-  constexpr int kBlockRows = 32;     // rows staged in LDS at a time
+  // rows staged in LDS at a time: one chunk, loaded a chunk ahead.  With the half-height
+  // weight tile below a block's LDS stays under 10 KB, which lets four waves share a SIMD
+  constexpr int kBlockRows = kChunk;
   constexpr int kUtilityPitch = 68;  // rows 16-byte aligned, 16 lanes of a row read 64 banks
   constexpr int kWeightPitch = 68;
   __shared__ __attribute__((aligned(16))) uint32_t rows[kBlockRows * kRowWords];
@@ -1493,8 +1496,11 @@ void vjp_row_stats_kernel(VjpParams P) {
   __shared__ __attribute__((aligned(16))) uint32_t sign_table[kSignTableWords];
   __shared__ uint32_t value_columns[(kBlockRows + kWave) * NVW];
   __shared__ __attribute__((aligned(16))) float utilities[kChunk * kUtilityPitch];  // u, then e d u
-  __shared__ __attribute__((aligned(16))) float weights[kChunk * kWeightPitch];     // e
-  __shared__ float discard[kWave];
+  // e, eight rows at a time (their sums are taken after rows 7 and 15); while the utilities
+  // are formed it takes the elements of the edge tiles that belong to no lane
+  constexpr int kWeightRows = kChunk / 2;
+  __shared__ __attribute__((aligned(16))) float weights[kWeightRows * kWeightPitch];
+  float* const discard = weights;
   const Unit u = decode_unit<VARLEN>(P.L, blockIdx.x);
   if (!u.valid) return;
   BandView view;
@@ -1529,93 +1535,128 @@ void vjp_row_stats_kernel(VjpParams P) {
       static_cast<int>(ceilf(-__log2f(P.tail_threshold) / P.gate_log2)) + kChunk * P.L.D + 1;
   const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row actually present
   const int grad_lds_pitch = P.grad_pitch + 8;
+  // The global loads of a block (row words, row records, grad_output pieces, value sign
+  // words) set out one block ahead, into registers, right after the block before has been
+  // stored to LDS: a memory round trip per 32 rows was a fifth of a wave's time.  The
+  // grad_output rows come as 16-byte pieces, numbered row by row over the pieces the input
+  // type really has, in groups of at most two registers per lane: the first group travels
+  // ahead with the other loads, later ones (float32 rows of wider tiles) take a round trip of
+  // their own when the block starts instead of the registers the chunk loop needs.
+  constexpr int kGradParts = (kBlockRows * kGradChunksMax + kWave - 1) / kWave;
+  constexpr int kGradGroup = kGradParts < 2 ? kGradParts : 2;
+  constexpr int kValueParts = ((kBlockRows + kWave) * NVW + kWave - 1) / kWave;
+  const int pieces = kBlockRows * grad_chunks;
+  const float per_row = 1.0f / static_cast<float>(grad_chunks);
+  uint4 symbols_in;
+  float4 stat_in;
+  uint4 grad_in[kGradGroup];
+  uint32_t value_in[kValueParts];
+  const auto load_pieces = [&](int first, int group) {
+#pragma unroll
+    for (int part = 0; part < kGradGroup; ++part) {
+      const int index = (group + part) * kWave + lane;
+      const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+      const int piece = index - r * grad_chunks;
+      grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
+      if (index < pieces && first + r < view.steps) {
+        grad_in[part] = *reinterpret_cast<const uint4*>(
+            view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * P.grad_pitch +
+            8 * piece);
+      }
+    }
+  };
+  const auto store_pieces = [&](int group) {
+#pragma unroll
+    for (int part = 0; part < kGradGroup; ++part) {
+      const int index = (group + part) * kWave + lane;
+      const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
+      const int piece = index - r * grad_chunks;
+      if (index < pieces) {
+        *reinterpret_cast<uint4*>(grads + r * grad_lds_pitch + 8 * piece) = grad_in[part];
+      }
+    }
+  };
+  const auto issue_block_loads = [&](int first) {
+    const int i = min(first + lane, view.steps - 1);  // rows past the band's end repeat the last
+    const int t = view.diag0 + 1 + i;
+    symbols_in = make_uint4(0u, 0u, 0u, 0u);
+    stat_in = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (lane < kBlockRows) {
+      symbols_in.x = view.q[t];
+      symbols_in.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
+      symbols_in.z = view.k[i];
+      symbols_in.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
+      stat_in = view.stats[t];
+    }
+    if (needs_utility) {
+      load_pieces(first, 0);
+#pragma unroll
+      for (int part = 0; part < kValueParts; ++part) {
+        const int index = part * kWave + lane;
+        const int column = index / NVW;
+        const int a = first - 63 + column;
+        value_in[part] = (column < kBlockRows + kWave && a >= 1 && a <= view.len - 1)
+            ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
+      }
+    }
+  };
+  // What a chunk leaves in global memory (two row sums per row, its record) is held back
+  // until the next chunk has started: nothing young is then in flight when a block waits for
+  // its loads, which retire in order with every store and atomic issued before them.
+  float pending_weight_sum = 0.0f, pending_numerator_sum = 0.0f;
+  int pending_window = 0;
+  uint32_t pending_kept = 0u;
+  int pending_first = -1, pending_rows = 0;
+  const auto flush_outputs = [&]() {
+    if (pending_first < 0) return;
+    // lanes 0..3 of every 16-lane group write the four rows of their group
+    const int e = lane & 15;
+    const int r = 4 * (lane >> 4) + e;
+    if (e < 4 && r < pending_rows) {
+      float4* row_stats = view.stats + (view.diag0 + 1 + pending_first + r);
+      atomicAdd(&row_stats->y, pending_weight_sum);
+      if (needs_utility) atomicAdd(&row_stats->z, pending_numerator_sum);
+    }
+    if (view.checkpoints != nullptr) {
+      float* slot =
+          view.checkpoints + static_cast<int64_t>(pending_first / kChunk) * view.record_floats;
+      slot[kWave + lane] = __int_as_float(pending_window);
+      if constexpr (DROPOUT) {
+        // the gradient pass reads the decisions back instead of hashing again
+        reinterpret_cast<uint16_t*>(slot + kCheckpointFloats)[lane] =
+            static_cast<uint16_t>(pending_kept);
+      }
+    }
+    pending_first = -1;
+  };
+  issue_block_loads(0);
   for (int first = 0; first < view.steps; first += kBlockRows) {
     const int count = min(kBlockRows, view.steps - first);
     wave_lds_fence();
-    {
-      // every global load of the block is issued before the first of them is used
-      const bool row_lane = lane < kBlockRows;
-      const int i = min(first + lane, view.steps - 1);  // rows past the band's end repeat the last
-      const int t = view.diag0 + 1 + i;
-      uint4 symbols = make_uint4(0u, 0u, 0u, 0u);
-      float4 stat = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      if (row_lane) {
-        symbols.x = view.q[t];
-        symbols.y = (t - W - 1 >= 0) ? view.q[t - W - 1] : 0u;
-        symbols.z = view.k[i];
-        symbols.w = (i - W - 1 >= 0) ? view.k[i - W - 1] : 0u;
-        stat = view.stats[t];
-      }
-      // The grad_output rows come as 16-byte pieces, numbered row by row over the pieces the
-      // input type really has, in groups of at most two registers per lane: the first group
-      // travels with the other loads of the block, later ones (float32 rows of wider tiles)
-      // take a round trip of their own instead of the registers the chunk loop needs.
-      constexpr int kGradParts = (kBlockRows * kGradChunksMax + kWave - 1) / kWave;
-      constexpr int kGradGroup = kGradParts < 2 ? kGradParts : 2;
-      constexpr int kValueParts = ((kBlockRows + kWave) * NVW + kWave - 1) / kWave;
-      const int pieces = kBlockRows * grad_chunks;
-      const float per_row = 1.0f / static_cast<float>(grad_chunks);
-      uint4 grad_in[kGradGroup];
-      uint32_t value_in[kValueParts];
-      const auto load_pieces = [&](int group) {
+    if (lane < kBlockRows) {
+      uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
+      row_words[0] = symbols_in;
+      row_words[1] = make_uint4(__float_as_uint(fmaf(stat_in.x, kLog2e, stat_in.w)), 0u, 0u, 0u);
+    }
+    if (needs_utility) {
+      store_pieces(0);
 #pragma unroll
-        for (int part = 0; part < kGradGroup; ++part) {
-          const int index = (group + part) * kWave + lane;
-          const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
-          const int piece = index - r * grad_chunks;
-          grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
-          if (index < pieces && first + r < view.steps) {
-            grad_in[part] = *reinterpret_cast<const uint4*>(
-                view.grad_rows + static_cast<int64_t>(view.diag0 + 1 + first + r) * P.grad_pitch +
-                8 * piece);
-          }
-        }
-      };
-      const auto store_pieces = [&](int group) {
-#pragma unroll
-        for (int part = 0; part < kGradGroup; ++part) {
-          const int index = (group + part) * kWave + lane;
-          const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
-          const int piece = index - r * grad_chunks;
-          if (index < pieces) {
-            *reinterpret_cast<uint4*>(grads + r * grad_lds_pitch + 8 * piece) = grad_in[part];
-          }
-        }
-      };
-      if (needs_utility) {
-        load_pieces(0);
-#pragma unroll
-        for (int part = 0; part < kValueParts; ++part) {
-          const int index = part * kWave + lane;
-          const int column = index / NVW;
-          const int a = first - 63 + column;
-          value_in[part] = (column < kBlockRows + kWave && a >= 1 && a <= view.len - 1)
-              ? view.vbits[static_cast<int64_t>(a) * NVW + (index - column * NVW)] : 0u;
+      for (int part = 0; part < kValueParts; ++part) {
+        if (part * kWave + lane < (kBlockRows + kWave) * NVW) {
+          value_columns[part * kWave + lane] = value_in[part];
         }
       }
-      __builtin_amdgcn_sched_barrier(0);
-      if (row_lane) {
-        uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
-        row_words[0] = symbols;
-        row_words[1] = make_uint4(__float_as_uint(fmaf(stat.x, kLog2e, stat.w)), 0u, 0u, 0u);
-      }
-      if (needs_utility) {
-        store_pieces(0);
 #pragma unroll
-        for (int part = 0; part < kValueParts; ++part) {
-          if (part * kWave + lane < (kBlockRows + kWave) * NVW) {
-            value_columns[part * kWave + lane] = value_in[part];
-          }
-        }
-#pragma unroll
-        for (int group = kGradGroup; group < kGradParts; group += kGradGroup) {
-          if (group * kWave >= pieces) break;  // wave-uniform
-          load_pieces(group);
-          __builtin_amdgcn_sched_barrier(0);
-          store_pieces(group);
-        }
+      for (int group = kGradGroup; group < kGradParts; group += kGradGroup) {
+        if (group * kWave >= pieces) break;  // wave-uniform
+        load_pieces(first, group);
+        __builtin_amdgcn_sched_barrier(0);
+        store_pieces(group);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    if (first + kBlockRows < view.steps) issue_block_loads(first + kBlockRows);
+    __builtin_amdgcn_sched_barrier(0);
     for (int local = 0; local < count; local += kChunk) {
       const int rows_here = min(kChunk, count - local);
       const int chunk_first = first + local;
@@ -1624,6 +1665,7 @@ void vjp_row_stats_kernel(VjpParams P) {
             view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
         slot[lane] = band.evidence;
       }
+      flush_outputs();  // of the chunk before
       const int window_before = band.window - kCountBias;
       float peak_overflow = 0.0f;
       wave_lds_fence();
@@ -1634,6 +1676,7 @@ void vjp_row_stats_kernel(VjpParams P) {
         wave_lds_fence();
       }
       uint32_t kept_bits = 0u;  // bit r: this lane's pair of row r is kept
+      v4f first_weight_sums;    // of rows 0 .. 7
       // compiled twice: once every lane is past its window fill no masking is needed
       auto run_chunk = [&](auto steady_tag, auto quiet_tag) {
         constexpr bool STEADY = decltype(steady_tag)::value;
@@ -1647,6 +1690,92 @@ void vjp_row_stats_kernel(VjpParams P) {
         // needs no addition (the weight only sees S through sqrt(1 + S) anyway)
         float one_plus_evidence = 1.0f + band.evidence;
         const uint32_t* row = rows + local * kRowWords;
+        if constexpr (QUIET) {
+          // Quiet chunks, the common case, take their rows four at a time through each stage
+          // (slides and gates, evidence and weights, hash rounds, stores): every stage then
+          // offers the scheduler four independent dependency chains instead of one.
+          constexpr int kGroup = 4;
+          uint4 ahead_symbols[kGroup];
+          float ahead_shift[kGroup], ahead_utility[kGroup];
+          const auto fetch_group = [&](int g) {
+#pragma unroll
+            for (int j = 0; j < kGroup; ++j) {
+              ahead_symbols[j] = *reinterpret_cast<const uint4*>(row + (g + j) * kRowWords);
+              ahead_shift[j] = __uint_as_float(row[(g + j) * kRowWords + 4]);
+              ahead_utility[j] = utilities[(g + j) * kUtilityPitch + lane];
+            }
+          };
+          fetch_group(0);
+#pragma unroll
+          for (int g = 0; g < kChunk; g += kGroup) {
+            float gates[kGroup], shifts[kGroup], group_utilities[kGroup];
+            uint32_t hashes[kGroup];
+#pragma unroll
+            for (int j = 0; j < kGroup; ++j) {
+              const uint4 words = ahead_symbols[j];
+              shifts[j] = ahead_shift[j];
+              group_utilities[j] = ahead_utility[j];
+              band.key_word = dpp_wave_shr1(words.z, band.key_word);
+              band.old_key_word = dpp_wave_shr1(words.w, band.old_key_word);
+              const uint32_t differing = words.x ^ band.key_word;
+              gates[j] = decay_of_biased_count(biased_popc(differing), P.gate_log2);
+              entering = popc_plus(differing, entering);
+              leaving = popc_plus(words.y ^ band.old_key_word, leaving);
+              if constexpr (DROPOUT) {
+                route_hash = dpp_wave_shr1(route_hash_of(chunk_first + g + j + 1), route_hash);
+                hashes[j] = route_hash;
+              }
+            }
+            if (g + kGroup < kChunk) fetch_group(g + kGroup);
+            __builtin_amdgcn_sched_barrier(0);
+            float group_weights[kGroup];
+#pragma unroll
+            for (int j = 0; j < kGroup; ++j) {
+              one_plus_evidence = fmaf(gates[j], one_plus_evidence, 1.0f);
+              group_weights[j] =
+                  fast_exp2(fmaf(fast_sqrt(one_plus_evidence), logit_gain, -shifts[j]));
+            }
+            bool kept[kGroup];
+            if constexpr (DROPOUT) {
+              __builtin_amdgcn_sched_barrier(0);
+              uint32_t states[kGroup];
+#pragma unroll
+              for (int j = 0; j < kGroup; ++j) {
+                const int t = view.diag0 + 1 + chunk_first + g + j;
+                states[j] = hashes[j] ^ fold16(static_cast<uint32_t>(t) ^ 0xb5297a4du);
+              }
+              const uint32_t round_keys[4] = {key.head_key, key.batch_key, key.seed_low_key,
+                                              key.seed_high_key};
+#pragma unroll
+              for (int round = 0; round < 4; ++round) {
+#pragma unroll
+                for (int j = 0; j < kGroup; ++j) states[j] = open_round(states[j]) ^ round_keys[round];
+              }
+#pragma unroll
+              for (int j = 0; j < kGroup; ++j) kept[j] = fold16(open_round(states[j])) >= key.keep_from;
+              __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < kGroup; ++j) {
+              float dropped_utility = group_weights[j] * group_utilities[j];
+              if constexpr (DROPOUT) {
+                dropped_utility = kept[j] ? dropped_utility : 0.0f;
+                kept_bits = doubled_plus_flag(kept_bits, kept[j]);
+              }
+              weights[((g + j) & (kWeightRows - 1)) * kWeightPitch + lane] = group_weights[j];
+              utilities[(g + j) * kUtilityPitch + lane] = dropped_utility;
+            }
+            if (g + kGroup == kWeightRows) {
+              wave_lds_fence();
+              first_weight_sums = tile_row_sums<kWeightRows>(weights, kWeightPitch, lane);
+              wave_lds_fence();
+            }
+          }
+          band.window += static_cast<int>(entering - leaving);
+          band.evidence = one_plus_evidence - 1.0f;  // exact: 1 <= 1 + S
+          if constexpr (DROPOUT) kept_bits = __builtin_bitreverse32(kept_bits) >> 16;  // bit r: row r
+          return;
+        }
         uint4 next_symbols = *reinterpret_cast<const uint4*>(row);
         float next_shift = __uint_as_float(row[4]);
         float next_utility = utilities[lane];
@@ -1697,8 +1826,13 @@ void vjp_row_stats_kernel(VjpParams P) {
             dropped_utility = kept ? dropped_utility : 0.0f;
             kept_bits = doubled_plus_flag(kept_bits, kept);  // rows end up in reverse order
           }
-          weights[r * kWeightPitch + lane] = weight;
+          weights[(r & (kWeightRows - 1)) * kWeightPitch + lane] = weight;
           utilities[r * kUtilityPitch + lane] = dropped_utility;
+          if (r + 1 == kWeightRows) {
+            wave_lds_fence();
+            first_weight_sums = tile_row_sums<kWeightRows>(weights, kWeightPitch, lane);
+            wave_lds_fence();
+          }
         }
         if constexpr (QUIET) {
           band.window += static_cast<int>(entering - leaving);
@@ -1719,38 +1853,28 @@ void vjp_row_stats_kernel(VjpParams P) {
       }
       wave_lds_fence();
       {
-        const v4f weight_sums = tile_row_sums(weights, kWeightPitch, lane);
-        const v4f numerator_sums = tile_row_sums(utilities, kUtilityPitch, lane);
-        // lanes 0..3 of every 16-lane group write the four rows of their group
+        // the second half of the weight tile repeats as rows 8 .. 15 of the product, which is
+        // where the lanes of groups 2 and 3 expect the sums of the chunk's rows 8 .. 15
+        const v4f second_weight_sums = tile_row_sums<kWeightRows>(weights, kWeightPitch, lane);
+        const v4f weight_sums = lane < 32 ? first_weight_sums : second_weight_sums;
+        const v4f numerator_sums = tile_row_sums<kChunk>(utilities, kUtilityPitch, lane);
         const int e = lane & 15;
-        const int r = 4 * (lane >> 4) + e;
-        if (e < 4 && r < rows_here) {
-          const float weight_sum = e == 0 ? weight_sums[0] : e == 1 ? weight_sums[1]
-                                 : e == 2 ? weight_sums[2] : weight_sums[3];
-          const float numerator_sum = e == 0 ? numerator_sums[0] : e == 1 ? numerator_sums[1]
-                                    : e == 2 ? numerator_sums[2] : numerator_sums[3];
-          float4* row_stats = view.stats + (view.diag0 + 1 + chunk_first + r);
-          atomicAdd(&row_stats->y, weight_sum);
-          if (needs_utility) {
-            atomicAdd(&row_stats->z, DROPOUT ? numerator_sum * P.inverse_keep : numerator_sum);
-          }
-        }
+        pending_weight_sum = e == 0 ? weight_sums[0] : e == 1 ? weight_sums[1]
+                           : e == 2 ? weight_sums[2] : weight_sums[3];
+        pending_numerator_sum = e == 0 ? numerator_sums[0] : e == 1 ? numerator_sums[1]
+                              : e == 2 ? numerator_sums[2] : numerator_sums[3];
+        if constexpr (DROPOUT) pending_numerator_sum *= P.inverse_keep;
       }
-      if (view.checkpoints != nullptr) {
-        float* slot =
-            view.checkpoints + static_cast<int64_t>(chunk_first / kChunk) * view.record_floats;
-        // the sign bit of the window word tells the gradient pass that some overflow term
-        // of the chunk is large enough to matter
-        const bool noisy = __ballot(peak_overflow >= P.tail_threshold) != 0ull;
-        slot[kWave + lane] = __int_as_float(window_before | (noisy ? INT32_MIN : 0));
-        if constexpr (DROPOUT) {
-          // the gradient pass reads the decisions back instead of hashing again
-          reinterpret_cast<uint16_t*>(slot + kCheckpointFloats)[lane] =
-              static_cast<uint16_t>(kept_bits);
-        }
-      }
+      // the sign bit of the window word tells the gradient pass that some overflow term
+      // of the chunk is large enough to matter
+      const bool noisy = __ballot(peak_overflow >= P.tail_threshold) != 0ull;
+      pending_window = window_before | (noisy ? INT32_MIN : 0);
+      pending_kept = kept_bits;
+      pending_first = chunk_first;
+      pending_rows = rows_here;
     }
   }
+  flush_outputs();
 }
 
 // After the row-statistics pass a row's float4 (reference, denominator, dropped
@@ -3184,7 +3308,7 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
 
 // bytes of the staged grad_output rows of a block of the row-statistics kernel
 size_t row_stats_dynamic_lds(int grad_pitch) {
-  constexpr int kBlockRows = 32;
+  constexpr int kBlockRows = kChunk;  // as in the kernel
   return sizeof(uint16_t) * kBlockRows * static_cast<size_t>(grad_pitch + 8);
 }
 
