@@ -1473,6 +1473,15 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
   return mfma_16x16x4(partial, 1.0f, v4f{0.0f, 0.0f, 0.0f, 0.0f});
 }
 
+// Waves per SIMD the row-statistics kernel is compiled for: the most its registers allow
+// without a spill (the hash rounds of four rows at a time take about twelve); its LDS allows
+// four up to a padded value width of 32 with 16-bit inputs, three at 64.
+constexpr int row_stats_waves(int dvp, bool dropout) {
+  if (dvp <= 8) return 4;
+  if (dvp <= 32) return dropout ? 3 : 4;
+  return dropout ? 2 : 3;
+}
+
 // Row-statistics pass: denominator and expected dropped utility of every row.
 // Rows are processed 16 at a time without any branch in between.  A chunk leaves
 // its route weights and its dropped weighted utilities as two [row][lane] tiles
@@ -1480,7 +1489,8 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 // each from 16 lanes; every lane keeps its 16 dropout decisions of the chunk as bits and
 // stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(DVP <= 32 ? 3 : 1)))
+__global__ __launch_bounds__(kWave)
+__attribute__((amdgpu_waves_per_eu(row_stats_waves(DVP, DROPOUT))))
 void vjp_row_stats_kernel(VjpParams P) {
   // rows staged in LDS at a time: one chunk, loaded a chunk ahead.  With the half-height
   // weight tile below a block's LDS stays under 10 KB, which lets four waves share a SIMD
