@@ -1473,14 +1473,9 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
   return mfma_16x16x4(partial, 1.0f, v4f{0.0f, 0.0f, 0.0f, 0.0f});
 }
 
-// Waves per SIMD the row-statistics kernel is compiled for: the most its registers allow
-// without a spill (the hash rounds of four rows at a time take about twelve); its LDS allows
-// four up to a padded value width of 32 with 16-bit inputs, three at 64.
-constexpr int row_stats_waves(int dvp, bool dropout) {
-  if (dvp <= 8) return 4;
-  if (dvp <= 32) return dropout ? 3 : 4;
-  return dropout ? 2 : 3;
-}
+// Waves per SIMD the row-statistics kernel is compiled for (no variant spills at these): its
+// LDS allows four up to a padded value width of 32 with 16-bit inputs and three at 64.
+constexpr int row_stats_waves(int dvp) { return dvp <= 32 ? 4 : 3; }
 
 // Row-statistics pass: denominator and expected dropped utility of every row.
 // Rows are processed 16 at a time without any branch in between.  A chunk leaves
@@ -1490,7 +1485,7 @@ constexpr int row_stats_waves(int dvp, bool dropout) {
 // stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
-__attribute__((amdgpu_waves_per_eu(row_stats_waves(DVP, DROPOUT))))
+__attribute__((amdgpu_waves_per_eu(row_stats_waves(DVP))))
 void vjp_row_stats_kernel(VjpParams P) {
   // rows staged in LDS at a time: one chunk, loaded a chunk ahead.  With the half-height
   // weight tile below a block's LDS stays under 10 KB, which lets four waves share a SIMD
@@ -1562,9 +1557,13 @@ void vjp_row_stats_kernel(VjpParams P) {
   uint4 grad_in[kGradGroup];
   uint32_t value_in[kValueParts];
   const auto load_pieces = [&](int first, int group) {
+    // (the piece numbering is recomputed where it is used: kept across the chunk loop it
+    // would cost registers the wider variants do not have)
+    int piece_lane = lane;
+    asm volatile("" : "+v"(piece_lane));
 #pragma unroll
     for (int part = 0; part < kGradGroup; ++part) {
-      const int index = (group + part) * kWave + lane;
+      const int index = (group + part) * kWave + piece_lane;
       const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
       const int piece = index - r * grad_chunks;
       grad_in[part] = make_uint4(0u, 0u, 0u, 0u);
@@ -1576,9 +1575,11 @@ void vjp_row_stats_kernel(VjpParams P) {
     }
   };
   const auto store_pieces = [&](int group) {
+    int piece_lane = lane;
+    asm volatile("" : "+v"(piece_lane));
 #pragma unroll
     for (int part = 0; part < kGradGroup; ++part) {
-      const int index = (group + part) * kWave + lane;
+      const int index = (group + part) * kWave + piece_lane;
       const int r = static_cast<int>((static_cast<float>(index) + 0.5f) * per_row);
       const int piece = index - r * grad_chunks;
       if (index < pieces) {
