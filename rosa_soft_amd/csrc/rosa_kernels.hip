@@ -1947,18 +1947,26 @@ __device__ __forceinline__ float negated_symbol(uint32_t word, int bit) {
   return sign_from_bit31(word << (31 - bit));
 }
 
-// register budget of the gradient kernel: waves per SIMD it is compiled for
+// register budget of the gradient kernel: waves per SIMD it is compiled for.  Its time falls
+// almost in proportion to the waves that share a SIMD; one value tile and one symbol tile
+// fit three (168 registers) without a spill.
 constexpr int gradient_waves(int value_tiles, int symbol_tiles) {
-  if (value_tiles == 1 && symbol_tiles == 1) return 2;
+  if (value_tiles == 1 && symbol_tiles == 1) return 3;
   if (value_tiles == 4 && symbol_tiles == 2) return 1;   // 120 accumulator registers alone
   return 2;
 }
 
-// rows staged in LDS per segment of the gradient kernel (a multiple of kChunk)
-constexpr int gradient_segment(int dvp) { return dvp >= 16 ? 32 : 64; }
+// rows staged in LDS per segment of the gradient kernel (a multiple of kChunk): with 32 a
+// single-wave block of the narrowest tile needs 11.4 KB, which leaves room for three per SIMD
+constexpr int gradient_segment(int /*dvp*/) { return 32; }
 
-// resident waves of the persistent gradient kernel: two per SIMD of the 256 compute units
-constexpr int kMaxResidentBlocks = 2048;
+// resident waves of the persistent gradient kernel per wave it is compiled to hold on each
+// SIMD of the 256 compute units
+constexpr int kMaxResidentBlocks = 2048;  // at two waves per SIMD
+constexpr int resident_gradient_waves(int value_tiles, int symbol_tiles) {
+  return 1024 * (gradient_waves(value_tiles, symbol_tiles) < 2
+                     ? 2 : gradient_waves(value_tiles, symbol_tiles));
+}
 
 // Waves per block of the gradient kernel (rosa_hip_set_gradient_block_waves overrides).
 // Two waves halve the column atomics, which bound the wide tiles; the narrow tile is bound
@@ -2096,11 +2104,12 @@ void vjp_gradients_kernel(VjpParams P) {
   const int grad_chunks = P.grad_pitch / 8;   // 16-byte pieces per row
   constexpr int kGradChunksMax = grad_term_pitch(kMaxGradTerms, DVP) / 8;
 
-  // The wide tiles have no registers for the many addresses and offsets that derive from
-  // the lane number alone (the compiler hoists them out of all loops, spills them, and
-  // reloads them in front of every atomic): there the lane number is made opaque once per
-  // chunk, so that they are recomputed where they are used.
-  constexpr bool kRecomputeLaneValues = VT > 1 || DT > 1;
+  // The kernel has no registers for the many addresses and offsets that derive from the
+  // lane number alone (the compiler hoists them out of all loops: fifty registers of the
+  // narrowest tile, spills in the wide ones): the lane number is made opaque once per
+  // chunk, so that they are recomputed where they are used.  That costs the narrowest tile
+  // 3 % more instructions and gives it its third wave per SIMD.
+  constexpr bool kRecomputeLaneValues = true;
   // completed tiles wait in registers for the next chunk's replay to cover their atomics
   constexpr bool kFlushAtOnce = false;
   const int lane_id = threadIdx.x & (kWave - 1);
@@ -3214,7 +3223,8 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
                            static_cast<int64_t>(max_segments) * 2 * kWave;
   const int64_t units = static_cast<int64_t>(v.L.slots) * v.L.H;
   // resident waves of the gradient kernel (an even number: its blocks hold one or two waves)
-  w.resident_blocks = static_cast<int>(std::min<int64_t>((units + 1) & ~int64_t(1), kMaxResidentBlocks));
+  w.resident_blocks = static_cast<int>(std::min<int64_t>(
+      (units + 1) & ~int64_t(1), resident_gradient_waves((dvp + 15) / 16, v.L.D > 16 ? 2 : 1)));
   // keep the scratch pool below 2 GiB by running fewer resident blocks for huge windows
   const int64_t budget_floats = (int64_t(1) << 31) / 4;
   while (w.resident_blocks > 64 &&
