@@ -1295,7 +1295,7 @@ __device__ __forceinline__ void fill_sign_table(uint32_t* table, int lane) {
 // matrix products, stores): the LDS and matrix latencies of one tile are covered by the
 // others instead of adding up (one tile after the other took 13 % of the gradient kernel,
 // together 7 %), at the price of twenty more live registers.
-template <int NVW, int DVP, bool BY_COLUMN>
+template <int NVW, int DVP, bool BY_COLUMN, int BATCH = 5>
 __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, int grad_pitch,
                                                      int k_blocks, const uint32_t* value_columns,
                                                      const uint32_t* sign_table, float* out,
@@ -1303,63 +1303,80 @@ __device__ __forceinline__ void utility_tiles_staged(const uint16_t* grad_tile, 
   const int li = lane & 15;
   const int lg = lane >> 4;
   const uint16_t* a_row = grad_tile + li * grad_pitch + 8 * lg;
-  // (two arrays, not one indexed by the word: a select between elements of one array
-  // becomes a dynamic index, and the array then lives in scratch memory)
-  uint32_t low_words[5], high_words[5];
-#pragma unroll
-  for (int m = 0; m < 5; ++m) {
-    low_words[m] = value_columns[(16 * m + li) * NVW];
-    high_words[m] = NVW > 1 ? value_columns[(16 * m + li) * NVW + NVW - 1] : 0u;
-  }
-  v4f acc[5];
-#pragma unroll
-  for (int m = 0; m < 5; ++m) acc[m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   constexpr int kBlocksMax = grad_term_pitch(kMaxGradTerms, DVP) / 32;
+  // BATCH tiles at a time (all five where the registers are there)
 #pragma unroll
-  for (int q = 0; q < kBlocksMax; ++q) {
-    if (q > 0 && q >= k_blocks) break;  // wave-uniform; there is always a first block
-    const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
-    const int d0 = (32 * q + 8 * lg) & (DVP - 1);
-    v4u signs[5];
+  for (int m0 = 0; m0 < 5; m0 += BATCH) {
+    constexpr int kTilesMax = BATCH;
+    const int tiles = 5 - m0 < BATCH ? 5 - m0 : BATCH;  // folds: m0 is an unrolled constant
+    // (two arrays, not one indexed by the word: a select between elements of one array
+    // becomes a dynamic index, and the array then lives in scratch memory)
+    uint32_t low_words[kTilesMax], high_words[kTilesMax];
 #pragma unroll
-    for (int m = 0; m < 5; ++m) {
-      uint32_t word = low_words[m];
-      if constexpr (NVW > 1) word = d0 >= 32 ? high_words[m] : low_words[m];
-      const uint32_t byte = word >> (d0 & 31);
-      const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
-      const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
-      signs[m] = v4u{low.x, low.y, high.x, high.y};
+    for (int n = 0; n < kTilesMax; ++n) {
+      if (n >= tiles) break;
+      const int m = m0 + n;
+      low_words[n] = value_columns[(16 * m + li) * NVW];
+      high_words[n] = NVW > 1 ? value_columns[(16 * m + li) * NVW + NVW - 1] : 0u;
     }
+    v4f acc[kTilesMax];
 #pragma unroll
-    for (int m = 0; m < 5; ++m) {
-      acc[m] = BY_COLUMN ? mfma_bf16(signs[m], a, acc[m]) : mfma_bf16(a, signs[m], acc[m]);
-    }
-  }
-  // The products are read right behind a branch of the loop above, where the compiler has
-  // been seen to leave out the wait states a matrix result needs before vector or LDS
-  // instructions may read it (wrong utilities): they are spent here, once for all five.
-  asm volatile("s_nop 7\n\ts_nop 3"
-               : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]));
+    for (int n = 0; n < kTilesMax; ++n) acc[n] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-  for (int m = 0; m < 5; ++m) {
-    if constexpr (BY_COLUMN) {
-      const int r = li;
-      const int c = 16 * m + 4 * lg;
+    for (int q = 0; q < kBlocksMax; ++q) {
+      if (q > 0 && q >= k_blocks) break;  // wave-uniform; there is always a first block
+      const v4u a = *reinterpret_cast<const v4u*>(a_row + 32 * q);
+      const int d0 = (32 * q + 8 * lg) & (DVP - 1);
+      v4u signs[kTilesMax];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (m == 0 && c + e < r + 1) acc[m][e] = 0.0f;
-        if (m == 4 && c + e > r + kWave) acc[m][e] = 0.0f;
+      for (int n = 0; n < kTilesMax; ++n) {
+        if (n >= tiles) break;
+        uint32_t word = low_words[n];
+        if constexpr (NVW > 1) word = d0 >= 32 ? high_words[n] : low_words[n];
+        const uint32_t byte = word >> (d0 & 31);
+        const uint2 low = *reinterpret_cast<const uint2*>(sign_table + ((byte << 1) & 0x1e));
+        const uint2 high = *reinterpret_cast<const uint2*>(sign_table + ((byte >> 3) & 0x1e));
+        signs[n] = v4u{low.x, low.y, high.x, high.y};
       }
-      *reinterpret_cast<v4f*>(out + r * pitch + c) = acc[m];
+#pragma unroll
+      for (int n = 0; n < kTilesMax; ++n) {
+        if (n >= tiles) break;
+        acc[n] = BY_COLUMN ? mfma_bf16(signs[n], a, acc[n]) : mfma_bf16(a, signs[n], acc[n]);
+      }
+    }
+    // The products are read right behind a branch of the loop above, where the compiler has
+    // been seen to leave out the wait states a matrix result needs before vector or LDS
+    // instructions may read it (wrong utilities): they are spent here, once for the batch.
+    if constexpr (BATCH == 5) {
+      asm volatile("s_nop 7\n\ts_nop 3"
+                   : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]));
     } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int r = 4 * lg + e;
-        const int l = 64 - (16 * m + li) + r;
-        float* target = out + r * pitch + l;
-        if (m == 0) target = l < kWave ? target : discard + lane;
-        if (m == 4) target = l >= 0 ? target : discard + lane;
-        *target = acc[m][e];
+      for (int n = 0; n < kTilesMax; ++n) asm volatile("s_nop 7\n\ts_nop 3" : "+v"(acc[n]));
+    }
+#pragma unroll
+    for (int n = 0; n < kTilesMax; ++n) {
+      if (n >= tiles) break;
+      const int m = m0 + n;
+      if constexpr (BY_COLUMN) {
+        const int r = li;
+        const int c = 16 * m + 4 * lg;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (m == 0 && c + e < r + 1) acc[n][e] = 0.0f;
+          if (m == 4 && c + e > r + kWave) acc[n][e] = 0.0f;
+        }
+        *reinterpret_cast<v4f*>(out + r * pitch + c) = acc[n];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * lg + e;
+          const int l = 64 - (16 * m + li) + r;
+          float* target = out + r * pitch + l;
+          if (m == 0) target = l < kWave ? target : discard + lane;
+          if (m == 4) target = l >= 0 ? target : discard + lane;
+          *target = acc[n][e];
+        }
       }
     }
   }
@@ -1473,9 +1490,10 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
   return mfma_16x16x4(partial, 1.0f, v4f{0.0f, 0.0f, 0.0f, 0.0f});
 }
 
-// Waves per SIMD the row-statistics kernel is compiled for (no variant spills at these): its
-// LDS allows four up to a padded value width of 32 with 16-bit inputs and three at 64.
-constexpr int row_stats_waves(int dvp) { return dvp <= 32 ? 4 : 3; }
+// Waves per SIMD the row-statistics kernel is compiled for (no variant spills at these; the
+// widest tile with dropout is one register short of four).  Its LDS allows four with 16-bit
+// inputs at every width.
+constexpr int row_stats_waves(int dvp, bool dropout) { return dvp > 32 && dropout ? 3 : 4; }
 
 // Row-statistics pass: denominator and expected dropped utility of every row.
 // Rows are processed 16 at a time without any branch in between.  A chunk leaves
@@ -1485,7 +1503,7 @@ constexpr int row_stats_waves(int dvp) { return dvp <= 32 ? 4 : 3; }
 // stores them with the chunk's checkpoint for the gradient pass.
 template <int NVW, int DVP, bool VARLEN, bool DROPOUT>
 __global__ __launch_bounds__(kWave)
-__attribute__((amdgpu_waves_per_eu(row_stats_waves(DVP))))
+__attribute__((amdgpu_waves_per_eu(row_stats_waves(DVP, DROPOUT))))
 void vjp_row_stats_kernel(VjpParams P) {
   // rows staged in LDS at a time: one chunk, loaded a chunk ahead.  With the half-height
   // weight tile below a block's LDS stays under 10 KB, which lets four waves share a SIMD
@@ -1681,7 +1699,8 @@ void vjp_row_stats_kernel(VjpParams P) {
       float peak_overflow = 0.0f;
       wave_lds_fence();
       if (needs_utility) {
-        utility_tiles_staged<NVW, DVP, false>(grads + local * grad_lds_pitch, grad_lds_pitch,
+        // (the widest tile in two batches: its registers decide a fourth wave per SIMD)
+        utility_tiles_staged<NVW, DVP, false, (DVP > 32 ? 3 : 5)>(grads + local * grad_lds_pitch, grad_lds_pitch,
                                               P.grad_pitch / 32, value_columns + local * NVW,
                                               sign_table, utilities, kUtilityPitch, discard, lane);
         wave_lds_fence();
