@@ -1265,7 +1265,12 @@ __device__ __forceinline__ uint32_t pair_of(const uint16_t* first, const uint16_
 // negated symbol for both terms of a split operand; callers fold the sign into their scale.
 __device__ __forceinline__ uint32_t negated_symbol_pair(uint32_t word, int bit) {
   const int spread = __builtin_amdgcn_sbfe(static_cast<int>(word), bit, 1);  // 0 or all ones
-  return (static_cast<uint32_t>(spread) & 0x80008000u) | 0x3f803f80u;
+  // (a & b) | c is one instruction when no operand is a literal: the two constants are held
+  // in registers, one scalar and one vector (the instruction reads one scalar at most)
+  uint32_t sign_bits = 0x80008000u, ones = 0x3f803f80u;
+  asm("" : "+s"(sign_bits));
+  asm("" : "+v"(ones));
+  return (static_cast<uint32_t>(spread) & sign_bits) | ones;
 }
 
 // Four sign bits -> four bfloat16 values (+1.0 where the bit is set, -1.0 where it is
