@@ -3241,7 +3241,12 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   const int longest = v.L.varlen ? v.L.N : v.L.T;
   w.ring_rows = std::min(v.L.W, longest) + 1;
   const int segment_rows = gradient_segment(dvp);
-  const int max_segments = (longest + segment_rows - 1) / segment_rows + 1;
+  // one fallback checkpoint per segment of the longest possible band, for a wave that finds
+  // no records: never the case in a dense layout whose records fit (known here), decided on
+  // the device in a packed one
+  const bool may_run_without_records = v.L.varlen != 0 || w.checkpoint_capacity == 0;
+  const int max_segments =
+      may_run_without_records ? (longest + segment_rows - 1) / segment_rows + 1 : 0;
   w.block_scratch_floats = static_cast<int64_t>(w.ring_rows) * kWave +
                            2 * kCheckpointChunksMax * kWave +
                            static_cast<int64_t>(max_segments) * 2 * kWave;
