@@ -546,6 +546,18 @@ __device__ __forceinline__ RouteWinner scan_routes_wide(const Symbol* q, const S
 // `missing` = (W - run) << shift, so that the step is one saturating subtraction and the
 // key needs no shift: the winner is the *minimum* of missing | (low - a).  Chunks of 64
 // routes that lie entirely below the row block need no causal mask and are unrolled.
+//
+// On symbols of six or more random bits most steps match in no row of the wave (with 8 bits
+// 78 % of them): such a step leaves every run at zero and cannot improve a winner, so an
+// unmasked chunk runs in one of two forms.  The sparse form compares (one vector
+// instruction against the key symbol in a scalar register) and skips the step when no lane
+// matched; the update is done only on a step with a match, after the runs have been set to
+// zero if the step before it was skipped.  The dense form is the plain update of every
+// step.  Each chunk counts its steps with a match and the next chunk takes the form that
+// suits that count, so match-dense inputs (few symbol bits, repeated motifs) keep the dense
+// walk.
+constexpr int kDenseChunkHits = 52;  // steps with a match (of 64) from which the dense form pays
+
 template <typename Symbol>
 __device__ __forceinline__ RouteWinner scan_routes_narrow(const Symbol* q, const Symbol* k,
                                                           int t0, int length, int W, int shift,
@@ -557,20 +569,100 @@ __device__ __forceinline__ RouteWinner scan_routes_narrow(const Symbol* q, const
   const uint32_t cap = static_cast<uint32_t>(W) << shift;
   uint32_t best = cap | low;  // run 0
   uint32_t missing = cap;
+  // symbol of the row above the block (lane 0's predecessor row), wave-uniform
+  const uint32_t q_above = t0 >= 1 ? static_cast<uint32_t>(q[t0 - 1]) : 0u;
+  // key symbols of a chunk are fetched one chunk ahead: key position `column` (route
+  // column + 1) and the position before it, which decides whether the halo run is non-zero
+  uint32_t next_key = lane < length ? static_cast<uint32_t>(k[lane]) : 0u;
+  uint32_t next_before = (lane >= 1 && lane - 1 < length) ? static_cast<uint32_t>(k[lane - 1]) : 0u;
+  int hits = 0;  // steps with a match in the chunk before
   for (int a0 = 1; a0 <= a_last; a0 += kWave) {
     const int column = a0 - 1 + lane;
-    const int halo = halo_run(q, k, t0, column, W);
+    const uint32_t key_chunk = next_key;
+    const uint32_t key_before = next_before;
+    {
+      const int ahead = column + kWave;
+      const bool wanted = a0 + kWave <= a_last;
+      next_key = (wanted && ahead < length) ? static_cast<uint32_t>(k[ahead]) : 0u;
+      next_before = (wanted && ahead - 1 < length) ? static_cast<uint32_t>(k[ahead - 1]) : 0u;
+    }
+    // run of route `column` on the row above the block: non-zero only where the first
+    // symbols agree, which the registers decide; the rare longer compare reads memory
+    int halo = 0;
+    if (column >= 1 && column <= t0 - 1 && key_before == q_above) {
+      const int limit = min(W, column);
+      halo = 1;
+      while (halo < limit && q[t0 - 1 - halo] == k[column - 1 - halo]) ++halo;
+    }
     const uint32_t halo_missing = cap - (static_cast<uint32_t>(halo) << shift);
-    const uint32_t key_chunk = column < length ? k[column] : 0u;
     const uint32_t route_low = low - static_cast<uint32_t>(a0);
     if (a0 + kWave - 1 <= t0) {
+      if (hits < kDenseChunkHits) {
+        hits = 0;
+        int last_hit = -1;  // step that last updated the runs (they are valid when a chunk starts)
+        const Symbol* key_symbols = k + (a0 - 1);
+        constexpr int kBatch = 16;  // key symbols held in scalar registers at a time
+        uint32_t batch[kBatch], batch_ahead[kBatch];
+        const auto load_batch = [&](uint32_t (&into)[kBatch], int first) {
+          // wave-uniform addresses: scalar loads
 #pragma unroll
-      for (int j = 0; j < kWave; ++j) {
-        const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
-        const uint32_t above = dpp_wave_shr1(
-            static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
-        missing = q_symbol == k_symbol ? __builtin_elementwise_sub_sat(above, one) : cap;
-        best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+          for (int e = 0; e < kBatch; ++e) into[e] = key_symbols[first + e];
+        };
+        const auto arrive = [&](uint32_t (&held)[kBatch]) {
+#pragma unroll
+          for (int e = 0; e < kBatch; e += 8) {
+            asm volatile("" : "+s"(held[e]), "+s"(held[e + 1]), "+s"(held[e + 2]), "+s"(held[e + 3]),
+                              "+s"(held[e + 4]), "+s"(held[e + 5]), "+s"(held[e + 6]), "+s"(held[e + 7]));
+          }
+        };
+        if constexpr (sizeof(Symbol) == 4) load_batch(batch, 0);
+#pragma unroll
+        for (int j0 = 0; j0 < kWave; j0 += kBatch) {
+          if constexpr (sizeof(Symbol) == 4) {
+            // the batch is taken in here, and only then does the next one set out: a wait for
+            // scalar loads is a wait for all of them
+            arrive(batch);
+            if (j0 + kBatch < kWave) load_batch(batch_ahead, j0 + kBatch);
+          }
+#pragma unroll
+          for (int e = 0; e < kBatch; ++e) {
+            const int j = j0 + e;
+            uint32_t k_symbol;
+            if constexpr (sizeof(Symbol) == 4) {
+              k_symbol = batch[e];
+            } else {
+              k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+            }
+            const bool match = q_symbol == k_symbol;
+            if (__builtin_amdgcn_ballot_w64(match) != 0ull) {
+              if (last_hit != j - 1) missing = cap;  // skipped steps left every run at zero
+              const uint32_t above = dpp_wave_shr1(
+                  static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+              missing = match ? __builtin_elementwise_sub_sat(above, one) : cap;
+              best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+              last_hit = j;
+              ++hits;
+            }
+          }
+          if constexpr (sizeof(Symbol) == 4) {
+#pragma unroll
+            for (int e = 0; e < kBatch; ++e) batch[e] = batch_ahead[e];
+          }
+        }
+        if (last_hit != kWave - 1) missing = cap;
+      } else {
+        // (the steps with a match are counted on every eighth step)
+        hits = 0;
+#pragma unroll
+        for (int j = 0; j < kWave; ++j) {
+          const uint32_t k_symbol = __builtin_amdgcn_readlane(key_chunk, j);
+          const uint32_t above = dpp_wave_shr1(
+              static_cast<uint32_t>(__builtin_amdgcn_readlane(halo_missing, j)), missing);
+          const bool match = q_symbol == k_symbol;
+          if (j % 8 == 0) hits += __builtin_amdgcn_ballot_w64(match) != 0ull ? 8 : 0;
+          missing = match ? __builtin_elementwise_sub_sat(above, one) : cap;
+          best = min(best, missing | (route_low - static_cast<uint32_t>(j)));
+        }
       }
     } else {
       const int count = min(kWave, a_last - a0 + 1);
@@ -1039,7 +1131,9 @@ __device__ __forceinline__ void stage_rows(const BandView& view, int first, int 
       dst[1] = make_uint4(__float_as_uint(fmaf(row.x, kLog2e, row.w)), 0u, 0u, 0u);
     } else if constexpr (DETAIL == kRowFull) {
       const uint4 record = reinterpret_cast<const uint4*>(view.stats)[t];  // finalised
-      dst[1] = make_uint4(record.y, record.z, 0u, 0u);
+      // the replay order of the gradient pass (staged_symbols_replay_order)
+      dst[0] = make_uint4(symbols.x, symbols.z, record.y, record.z);
+      dst[1] = make_uint4(symbols.y, symbols.w, 0u, 0u);
     }
   }
 }
@@ -1165,21 +1259,33 @@ __device__ __forceinline__ StepOut forward_step(Band<NVW>& band, const RowSymbol
   return out;
 }
 
+// The gradient pass keeps what every row of its replay reads in the first four words:
+//   0 query word of row t          1 key word entering at lane 0
+//   2 exponent shift of the row    3 expected dropped utility
+//   4 query word of row t - W - 1  5 key word of column a0 - W - 1 entering at lane 0
+__device__ __forceinline__ RowSymbols staged_symbols_replay_order(const uint32_t* row) {
+  const uint2 front = *reinterpret_cast<const uint2*>(row);
+  const uint2 back = *reinterpret_cast<const uint2*>(row + 4);
+  return RowSymbols{front.x, back.x, front.y, back.y};
+}
+
 // Evidence-only sweep over `count` staged rows starting at step `first`.
-template <int NVW>
+template <int NVW, bool REPLAY_ORDER = false>
 __device__ __forceinline__ void sweep_rows(Band<NVW>& band, const uint32_t* rows, int first,
                                            int count, int lane, int W, float gate_log2) {
+  const auto symbols_of = [&](int r) {
+    return REPLAY_ORDER ? staged_symbols_replay_order(rows + r * kRowWords)
+                        : staged_symbols(rows + r * kRowWords);
+  };
   if (first >= W + kWave) {  // steady state: all 64 lanes are past their window fill
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, true>(band, staged_symbols(rows + r * kRowWords), first + r, lane, W,
-                              gate_log2);
+      forward_step<NVW, true>(band, symbols_of(r), first + r, lane, W, gate_log2);
     }
   } else {
 #pragma unroll 4
     for (int r = 0; r < count; ++r) {
-      forward_step<NVW, false>(band, staged_symbols(rows + r * kRowWords), first + r, lane, W,
-                               gate_log2);
+      forward_step<NVW, false>(band, symbols_of(r), first + r, lane, W, gate_log2);
     }
   }
 }
@@ -2417,8 +2523,8 @@ void vjp_gradients_kernel(VjpParams P) {
         const auto store_rows_and_keys = [&]() {
           if (row_lane) {
             uint4* row_words = reinterpret_cast<uint4*>(rows + lane * kRowWords);
-            row_words[0] = symbols;
-            row_words[1] = make_uint4(record.y, record.z, 0u, 0u);
+            row_words[0] = make_uint4(symbols.x, symbols.z, record.y, record.z);
+            row_words[1] = make_uint4(symbols.y, symbols.w, 0u, 0u);
             query_rows[lane] = seg_first + lane < view.steps ? symbols.x : 0u;
           }
 #pragma unroll
@@ -2520,8 +2626,8 @@ void vjp_gradients_kernel(VjpParams P) {
         ck_window[chunk * kWave + lane] = band.window;
         if (chunk + 1 < own_chunks) {
           const int local = chunk * kChunk;
-          sweep_rows<NVW>(band, rows + local * kRowWords, seg_first + local, kChunk, lane, W,
-                          P.gate_log2);
+          sweep_rows<NVW, true>(band, rows + local * kRowWords, seg_first + local, kChunk, lane,
+                                W, P.gate_log2);
         }
       }
       }  // segment_active
@@ -2600,42 +2706,45 @@ void vjp_gradients_kernel(VjpParams P) {
           constexpr bool STEADY = decltype(steady_tag)::value;
           constexpr bool CACHED = decltype(cached_tag)::value;  // keep decisions are read back
           constexpr bool QUIET = decltype(quiet_tag)::value;    // overflow terms are negligible
-          const uint32_t* row = rows + local * kRowWords;
+          // (the chunk's offset into the staged rows is held in a vector register: derived
+          // from a scalar it was formed again, two instructions, in front of every row's reads)
+          uint32_t row_offset = static_cast<uint32_t>(local) * kRowWords;
+          asm volatile("" : "+v"(row_offset));
+          const uint32_t* row = rows + row_offset;
           const float* slot = tile + 64 - lane;  // this lane's pair of row r: + r * (pitch + 1)
           // row words and utilities are fetched kRowsAhead rows before their use
           constexpr int kRowsAhead = kFetchAhead ? 2 : 1;
+          // replay order: everything a quiet chunk reads of a row is one 16-byte word
+          constexpr bool kOldWords = !(STEADY && QUIET);
           uint4 ahead_symbols[kRowsAhead];
           uint4 ahead_extra[kRowsAhead];
           float ahead_utility[kRowsAhead];
+          const auto fetch_row = [&](int from, int into) {
+            ahead_symbols[into] = *reinterpret_cast<const uint4*>(row + from * kRowWords);
+            if constexpr (kOldWords) {
+              ahead_extra[into] = *reinterpret_cast<const uint4*>(row + from * kRowWords + 4);
+            }
+            ahead_utility[into] = slot[from * (kTilePitch + 1)];
+          };
 #pragma unroll
-          for (int r = 0; r < kRowsAhead; ++r) {
-            ahead_symbols[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords);
-            ahead_extra[r] = *reinterpret_cast<const uint4*>(row + r * kRowWords + 4);
-            ahead_utility[r] = slot[r * (kTilePitch + 1)];
-          }
+          for (int r = 0; r < kRowsAhead; ++r) fetch_row(r, r);
 #pragma unroll
           for (int r = 0; r < kChunk; ++r) {
             const uint4 words = ahead_symbols[r % kRowsAhead];
-            const RowSymbols symbols{words.x, words.y, words.z, words.w};
-            const uint4 extra = ahead_extra[r % kRowsAhead];
+            uint4 extra = make_uint4(0u, 0u, 0u, 0u);
+            if constexpr (kOldWords) extra = ahead_extra[r % kRowsAhead];
+            const RowSymbols symbols{words.x, extra.x, words.y, extra.y};
             // the slot holds the pair's utility (anything finite when no symbol
             // gradient is wanted, in which case the adjoint is never used)
             const float utility = ahead_utility[r % kRowsAhead];
-            if (r + kRowsAhead < kChunk) {
-              const int ahead = r + kRowsAhead;
-              ahead_symbols[r % kRowsAhead] =
-                  *reinterpret_cast<const uint4*>(row + ahead * kRowWords);
-              ahead_extra[r % kRowsAhead] =
-                  *reinterpret_cast<const uint4*>(row + ahead * kRowWords + 4);
-              ahead_utility[r % kRowsAhead] = slot[ahead * (kTilePitch + 1)];
-            }
+            if (r + kRowsAhead < kChunk) fetch_row(r + kRowsAhead, r % kRowsAhead);
             // the loads stay here, ahead of their use (the scheduler would sink them)
             if constexpr (kFetchAhead) __builtin_amdgcn_sched_barrier(0);
             const bool row_ok = r < rows_here;
             const int i = min(first + r, last_step);
             const int t = view.diag0 + 1 + i;
-            const float shift = __uint_as_float(extra.x);
-            const float expected = __uint_as_float(extra.y);
+            const float shift = __uint_as_float(words.z);
+            const float expected = __uint_as_float(words.w);
             const StepOut s =
                 forward_step<NVW, STEADY, QUIET>(band, symbols, i, lane, W, P.gate_log2);
             const float one_plus = 1.0f + s.evidence;
