@@ -585,13 +585,75 @@ def run_runtime_workload(args) -> None:
     print(json.dumps(record))
 
 
+FUSED_WORKLOADS = {
+    # the projection behind the operator at the shape of config 3 (B4 T4096 H32 Dv64, bfloat16)
+    # with a square model width: out = residual + y @ W^T, y the operator's ternary output
+    "fused_output": dict(B=4, T=4096, H=32, D=16, Hv=32, Dv=64, W=32, N=2048),
+}
+
+BF16_MATRIX_PEAK = 2.5e15  # dense bfloat16 matrix peak of MI355X, FLOP/s
+
+
+def run_fused_workload(args) -> None:
+    """Hard forward in bit form + output projection fed with the bits, against the expanded
+    tensor + a library product (what the reference's caller does)."""
+
+    from rosa_soft_amd import cabi
+
+    config = FUSED_WORKLOADS[args.workload]
+    device = torch.device("cuda:0")
+    generator = torch.Generator(device=device).manual_seed(4321)
+    shape = lambda *dims: torch.randn(*dims, device=device, generator=generator).to(torch.bfloat16)
+    query = shape(config["B"], config["T"], config["H"], config["D"])
+    key = shape(config["B"], config["T"], config["H"], config["D"])
+    value = shape(config["B"], config["T"], config["Hv"], config["Dv"])
+    width = config["N"]
+    depth = config["H"] * config["Dv"]
+    weight = (shape(width, depth).float() / depth ** 0.5).to(torch.bfloat16)
+    residual = shape(config["B"], config["T"], width)
+    sign_words, routed = cabi.hard_forward_bits(query, key, value, config["W"])
+    begin_event = torch.cuda.Event(enable_timing=True)
+    end_event = torch.cuda.Event(enable_timing=True)
+
+    def timed(step) -> float:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        begin_event.record()
+        for _ in range(args.steps):
+            step()
+        end_event.record()
+        torch.cuda.synchronize()
+        return begin_event.elapsed_time(end_event) / args.steps
+
+    fused_ms = timed(lambda: cabi.project_routed_bits(sign_words, routed, config["Dv"], weight, residual))
+    library_ms = timed(lambda: torch.addmm(
+        residual.flatten(0, 1),
+        cabi.expand_output_bits(sign_words, routed, config["Dv"], torch.bfloat16).flatten(0, 1).flatten(1),
+        weight.t()))
+    tokens = config["B"] * config["T"]
+    flops = 2.0 * tokens * depth * width
+    record = {
+        "metric": "output projection from the bit form, tokens/sec",
+        "value": tokens / (fused_ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": fused_ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: " + ", ".join(f"{k}={v}" for k, v in config.items())},
+        "roofline": {"bound": "mfma", "achieved": flops / (fused_ms * 1e-3) / 1e12,
+                     "peak": BF16_MATRIX_PEAK / 1e12, "unit": "TFLOP/s",
+                     "frac": flops / (fused_ms * 1e-3) / BF16_MATRIX_PEAK, "traffic": None},
+        "expanded_tensor_plus_library_product_ms": library_ms,
+    }
+    print(json.dumps(record))
+
+
 def main() -> None:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=10)
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--workload", default="metric",
-                        choices=sorted(WORKLOADS) + sorted(RUNTIME_WORKLOADS))
+                        choices=sorted(WORKLOADS) + sorted(RUNTIME_WORKLOADS) + sorted(FUSED_WORKLOADS))
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-configs", action="store_true",
                         help="skip the block that times configurations 1 to 5 beside the metric shape")
@@ -621,6 +683,9 @@ def main() -> None:
 
     if args.workload in RUNTIME_WORKLOADS:
         run_runtime_workload(args)
+        return
+    if args.workload in FUSED_WORKLOADS:
+        run_fused_workload(args)
         return
 
     record = training_record(args)

@@ -152,6 +152,38 @@ int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query,
                                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Hard forward from symbol words that a producer has already written: the projections in
+ * front of the operator (self.query / self.key of examples/fit_soft_reference.py:374-392)
+ * can ballot the signs of their accumulators straight into the head-major word tensors
+ * that pack_sign_bits_pair_kernel writes (rosa_soft_kernels.cu:202-241), and this entry
+ * skips that packing pass.  `packed_query` / `packed_key` are inputs here (int32 [B,H,T] or
+ * [H,N], bit i = logit i > 0); `dtype` of the problem is that of `value` and `output`.
+ * The result leaves as `output` or, when `output` is NULL, as the bit form of
+ * rosa_hip_hard_forward_bits (`sign_words`, `routed`).  Same workspace as
+ * rosa_hip_hard_forward.
+ */
+int rosa_hip_hard_forward_words(const rosa_problem* problem, const int32_t* packed_query,
+                                const int32_t* packed_key, const void* value, void* output,
+                                uint32_t* sign_words, uint8_t* routed, int32_t* routes,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The projection behind the operator, fed with the bit form of its output:
+ *   out[t, n] = residual[t, n] + sum_{h, d} y[t, h, d] * weight[n, h * Dv + d],
+ *   y = routed ? (sign bit ? +1 : -1) : 0,
+ * i.e. `residual + self.output(routed.flatten(2))` of examples/fit_soft_reference.py:415-416
+ * without the ternary tensor in between: the matrix products (bfloat16 inputs, float32
+ * accumulation) expand their A operand from `sign_words` / `routed` in registers.
+ * `weight` is the [N][H * Dv] matrix of the linear layer, `residual` (optional) and `out`
+ * are [tokens][N]; all three bfloat16.  Dv must be 8, 16 or a multiple of 32, H * Dv a
+ * multiple of 32 and N a multiple of 64 (other shapes expand the bits and use a library
+ * product).  The reference has no such kernel.
+ */
+int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* routed,
+                                 int64_t tokens, int H, int Dv, const void* weight, int N,
+                                 const void* residual, void* out, void* stream);
+
+/*
  * rosa_hip_hard_forward for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  The workspace is a 16 MiB array that lives in the

@@ -34,6 +34,8 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_hard_forward_bits",
+    "rosa_hip_hard_forward_words",
+    "rosa_hip_project_routed_bits",
     "rosa_hip_hard_forward_static",
     "rosa_hip_pack_symbols",
     "rosa_hip_surrogate_vjp",
@@ -141,6 +143,14 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_hard_forward_bits.restype = ctypes.c_int
     library.rosa_hip_hard_forward_bits.argtypes = [
         problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_hard_forward_words.restype = ctypes.c_int
+    library.rosa_hip_hard_forward_words.argtypes = [
+        problem_p, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp,
+    ]
+    library.rosa_hip_project_routed_bits.restype = ctypes.c_int
+    library.rosa_hip_project_routed_bits.argtypes = [
+        vp, vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, vp, ctypes.c_int, vp, vp, vp,
     ]
     library.rosa_hip_hard_forward_static.restype = ctypes.c_int
     library.rosa_hip_hard_forward_static.argtypes = [problem_p, vp, vp, vp, vp, vp, vp, vp, vp]
@@ -331,6 +341,85 @@ def hard_forward_bits(
         )
     _check(status, "rosa_hip_hard_forward_bits")
     return sign_words, routed
+
+
+def hard_forward_words(
+    packed_q: Tensor,
+    packed_k: Tensor,
+    value: Tensor,
+    max_suffix_length: int,
+    symbol_bits: int,
+    cu_seqlens: Optional[Tensor] = None,
+    as_bits: bool = False,
+):
+    """Hard forward from symbol words a producer has already packed (no packing pass).
+
+    ``packed_q`` / ``packed_k`` are int32 ``[B, H, T]`` (``[H, N]`` packed), bit ``i`` set iff
+    logit ``i`` is positive; ``symbol_bits`` is their width ``D``.  Returns ``(output, routes)``
+    or, with ``as_bits``, ``(sign_words, routed, routes)`` in the layout of
+    ``hard_forward_bits``.
+    """
+
+    library = load()
+    assert packed_q.is_cuda and packed_q.is_contiguous() and packed_k.is_contiguous()
+    assert packed_q.dtype == torch.int32 and packed_k.dtype == torch.int32 and value.is_contiguous()
+    heads = packed_q.shape[-2]
+    # only the shapes of a query tensor are needed to describe the problem
+    if cu_seqlens is None:
+        shape = (packed_q.shape[0], packed_q.shape[2], heads, symbol_bits)
+    else:
+        shape = (packed_q.shape[1], heads, symbol_bits)
+    query_like = torch.empty(shape, dtype=value.dtype, device="meta")
+    problem = make_problem(query_like, value, max_suffix_length, cu_seqlens)
+    lead = shape[:-1]
+    with torch.cuda.device(value.device):
+        routes = torch.empty(packed_q.shape, dtype=torch.int32, device=value.device)
+        output = sign_words = routed = None
+        if as_bits:
+            words = (problem.Dv + 31) // 32
+            sign_words = torch.empty((*lead, words), dtype=torch.int32, device=value.device)
+            routed = torch.empty(lead, dtype=torch.uint8, device=value.device)
+        else:
+            output = torch.empty((*lead, problem.Dv), dtype=value.dtype, device=value.device)
+        size = library.rosa_hip_forward_workspace_bytes(ctypes.byref(problem))
+        workspace = torch.empty(max(size, 256), dtype=torch.uint8, device=value.device)
+        status = library.rosa_hip_hard_forward_words(
+            ctypes.byref(problem), _ptr(packed_q), _ptr(packed_k), _ptr(value), _ptr(output),
+            _ptr(sign_words), _ptr(routed), _ptr(routes), _ptr(workspace), workspace.numel(),
+            _stream(value),
+        )
+    _check(status, "rosa_hip_hard_forward_words")
+    return (sign_words, routed, routes) if as_bits else (output, routes)
+
+
+def project_routed_bits(sign_words: Tensor, routed: Tensor, value_dim: int, weight: Tensor,
+                        residual: Optional[Tensor] = None) -> Tensor:
+    """``residual + expand_output_bits(sign_words, routed).flatten(-2) @ weight.T`` in one kernel.
+
+    ``weight`` is the bfloat16 ``[N, H * Dv]`` matrix of a linear layer; the result (and the
+    optional ``residual``) is bfloat16 ``[..., N]`` over the leading axes of ``routed`` without
+    its head axis.
+    """
+
+    library = load()
+    assert sign_words.is_cuda and sign_words.is_contiguous() and routed.is_contiguous()
+    assert weight.dtype == torch.bfloat16 and weight.is_contiguous() and weight.dim() == 2
+    heads = routed.shape[-1]
+    tokens = routed.numel() // heads
+    width = weight.shape[0]
+    assert weight.shape[1] == heads * value_dim
+    lead = routed.shape[:-1]
+    if residual is not None:
+        assert residual.dtype == torch.bfloat16 and residual.is_contiguous()
+        assert tuple(residual.shape) == (*lead, width)
+    with torch.cuda.device(weight.device):
+        out = torch.empty((*lead, width), dtype=torch.bfloat16, device=weight.device)
+        status = library.rosa_hip_project_routed_bits(
+            _ptr(sign_words), _ptr(routed), tokens, heads, value_dim, _ptr(weight), width,
+            _ptr(residual), _ptr(out), _stream(weight),
+        )
+    _check(status, "rosa_hip_project_routed_bits")
+    return out
 
 
 def expand_output_bits(sign_words: Tensor, routed: Tensor, value_dim: int,

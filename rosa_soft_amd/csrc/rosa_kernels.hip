@@ -3405,14 +3405,17 @@ template <int DTYPE>
 int run_forward(const rosa_problem* p, const ProblemView& view, const void* query,
                 const void* key, const void* value, void* output, int32_t* packed_query,
                 int32_t* packed_key, int32_t* routes, int32_t* lengths, void* workspace,
-                hipStream_t stream, uint32_t* sign_words = nullptr, uint8_t* routed = nullptr) {
+                hipStream_t stream, uint32_t* sign_words = nullptr, uint8_t* routed = nullptr,
+                bool words_given = false) {
   Layout L = view.L;
   const ForwardWorkspace w = carve_forward(view);
   stage_begin(kStageForward, stream);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
                            stream);
   const int64_t elements = view.symbol_rows * L.D;
-  if (64 % L.D == 0) {
+  if (words_given) {
+    // a producer (the projection in front of the operator) has written the symbol words
+  } else if (64 % L.D == 0) {
     hipLaunchKernelGGL(pack_symbols_ballot_kernel<DTYPE>, dim3(blocks_for(elements, 256)),
                        dim3(256), 0, stream, query, key, packed_query, packed_key, elements, L.D,
                        L.H, L.T, L.N, L.varlen);
@@ -3850,14 +3853,158 @@ __global__ __launch_bounds__(256) void router_advance_kernel(RouterUpdate U) {
   U.history_lengths[slot] += router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot);
 }
 
+// ---------------------------------------------------------------------------
+// the projection that follows the operator, fed with the bit form of its output
+// ---------------------------------------------------------------------------
+//
+//   out[t, n] = residual[t, n] + sum_k y[t, k] * weight[n, k],   k = h * Dv + d,
+//   y[t, k] = routed[t, h] ? (bit d of sign_words[t, h] ? +1 : -1) : 0
+//
+// i.e. `residual + output(routed.flatten(2))` of the reference's caller
+// (examples/fit_soft_reference.py:374-417) without the ternary tensor in between: the A
+// operand of the matrix products is expanded from the bits in registers.  `weight` is the
+// [N][K] matrix of a linear layer (k contiguous), bfloat16; accumulation is float32.
+// A block of four waves computes 256 rows x 64 columns, each wave 64 x 64 (sixteen
+// 16 x 16 x 32 products per 32-wide k step).  Per step a block stages the weight tile
+// [64][32] and, per row, the 32 sign bits and 32 validity bits of the step in LDS; the loads
+// of the next step are in flight while the products of this one run.
+constexpr int kProjectRows = 256;
+constexpr int kProjectColumns = 64;
+constexpr int kProjectStep = 32;
+constexpr int kProjectWeightPitch = kProjectStep + 8;  // bfloat16 elements per staged weight row
+
+struct ProjectParams {
+  const uint32_t* sign_words;  // [tokens][H][nvw]
+  const uint8_t* routed;       // [tokens][H]
+  const uint16_t* weight;      // [N][K] bfloat16
+  const uint16_t* residual;    // [tokens][N] bfloat16 or NULL
+  uint16_t* out;               // [tokens][N] bfloat16
+  int64_t tokens;
+  int H, Dv, nvw, N, K;
+};
+
+// Eight sign bits and their validity -> eight bfloat16 values (two table entries of four):
+// entry (valid << 4 | nibble) holds +-1 per bit, or zeros where the head took the null route.
+constexpr int kTernaryTableWords = 64;
+
+__device__ __forceinline__ void fill_ternary_table(uint32_t* table, int index) {
+  if (index < kTernaryTableWords) {
+    const int entry = index >> 1;       // valid << 4 | nibble
+    const int nibble = entry & 15;
+    const bool valid = (entry >> 4) != 0;
+    const int low = (nibble >> (2 * (index & 1))) & 1;
+    const int high = (nibble >> (2 * (index & 1) + 1)) & 1;
+    table[index] = valid ? ((low ? 0x3f80u : 0xbf80u) | ((high ? 0x3f80u : 0xbf80u) << 16)) : 0u;
+  }
+}
+
+// sign bits and validity bits of k = 32 step .. 32 step + 31 of one token
+__device__ __forceinline__ uint2 ternary_step_bits(const ProjectParams& P, int64_t token, int step) {
+  const int k0 = step * kProjectStep;
+  uint32_t signs = 0u, valid = 0u;
+  if (token < P.tokens) {
+    if (P.Dv >= 32) {  // the step lies inside one head
+      const int head = k0 / P.Dv;
+      const int word = (k0 - head * P.Dv) >> 5;
+      signs = P.sign_words[(token * P.H + head) * P.nvw + word];
+      valid = P.routed[token * P.H + head] == 1 ? 0xffffffffu : 0u;
+    } else {           // 32 / Dv heads, one word each
+      const int heads = 32 / P.Dv;
+      const int head0 = k0 / P.Dv;
+      const uint32_t field = (1u << P.Dv) - 1u;
+      for (int j = 0; j < heads; ++j) {
+        const uint32_t word = P.sign_words[token * P.H + head0 + j] & field;
+        signs |= word << (j * P.Dv);
+        if (P.routed[token * P.H + head0 + j] == 1) valid |= field << (j * P.Dv);
+      }
+    }
+  }
+  return make_uint2(signs, valid);
+}
+
+__global__ __launch_bounds__(256) void project_routed_bits_kernel(ProjectParams P) {
+  __shared__ __attribute__((aligned(16))) uint16_t weight_tile[2][kProjectColumns * kProjectWeightPitch];
+  __shared__ __attribute__((aligned(8))) uint2 row_bits[2][kProjectRows];
+  __shared__ __attribute__((aligned(8))) uint32_t ternary_table[kTernaryTableWords];
+  const int thread = threadIdx.x;
+  const int lane = thread & 63;
+  const int wave = thread >> 6;
+  const int li = lane & 15;
+  const int lg = lane >> 4;
+  // neighbouring blocks share their weight columns (same blockIdx.y) and follow each other
+  // in row order, so the weight tiles of a column block stay in the cache of their XCD
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kProjectRows;
+  const int n0 = blockIdx.y * kProjectColumns;
+  fill_ternary_table(ternary_table, thread);
+
+  v4f acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  const int steps = P.K / kProjectStep;
+  // what a thread stages per step: 16 bytes of the weight tile and one row's bits
+  const int stage_n = thread >> 2;
+  const int stage_k = (thread & 3) * 8;
+  const uint16_t* weight_row = P.weight + static_cast<int64_t>(n0 + stage_n) * P.K + stage_k;
+  uint4 weight_in = *reinterpret_cast<const uint4*>(weight_row);
+  uint2 bits_in = ternary_step_bits(P, row0 + thread, 0);
+  for (int step = 0; step < steps; ++step) {
+    const int buffer = step & 1;
+    *reinterpret_cast<uint4*>(&weight_tile[buffer][stage_n * kProjectWeightPitch + stage_k]) = weight_in;
+    row_bits[buffer][thread] = bits_in;
+    __syncthreads();
+    if (step + 1 < steps) {  // the next step's loads are in flight during the products
+      weight_in = *reinterpret_cast<const uint4*>(weight_row + (step + 1) * kProjectStep);
+      bits_in = ternary_step_bits(P, row0 + thread, step + 1);
+    }
+    v4u b_operand[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      b_operand[j] = *reinterpret_cast<const v4u*>(
+          &weight_tile[buffer][(16 * j + li) * kProjectWeightPitch + 8 * lg]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint2 bits = row_bits[buffer][wave * 64 + 16 * i + li];
+      const uint32_t byte = (bits.x >> (8 * lg)) & 0xffu;
+      const uint32_t valid = (bits.y >> (8 * lg)) & 1u;  // a head is valid as a whole
+      const uint2 low = *reinterpret_cast<const uint2*>(
+          ternary_table + 2 * ((valid << 4) | (byte & 15u)));
+      const uint2 high = *reinterpret_cast<const uint2*>(
+          ternary_table + 2 * ((valid << 4) | (byte >> 4)));
+      const v4u a_operand = {low.x, low.y, high.x, high.y};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(a_operand, b_operand[j], acc[i][j]);
+    }
+  }
+  // lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li of every 16 x 16 tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int64_t token = row0 + wave * 64 + 16 * i + 4 * lg + e;
+      if (token >= P.tokens) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t index = token * P.N + n0 + 16 * j + li;
+        float value = acc[i][j][e];
+        if (P.residual != nullptr) value += __uint_as_float(static_cast<uint32_t>(P.residual[index]) << 16);
+        P.out[index] = static_cast<uint16_t>(bf16_nearest(value));
+      }
+    }
+  }
+}
+
 int forward_entry(const rosa_problem* problem, const void* query, const void* key,
                   const void* value, void* output, int32_t* packed_query, int32_t* packed_key,
                   int32_t* routes, int32_t* lengths, void* workspace, size_t workspace_bytes,
-                  void* stream, uint32_t* sign_words, uint8_t* routed) {
+                  void* stream, uint32_t* sign_words, uint8_t* routed, bool words_given = false) {
   ProblemView view;
   const int bad = check_problem(problem, &view);
   if (bad != 0) return bad;
-  if (!query || !key || !value || !packed_query || !packed_key || !workspace)
+  if ((!words_given && (!query || !key)) || !value || !packed_query || !packed_key || !workspace)
     return fail(2, "hard_forward: NULL tensor or workspace pointer");
   if (workspace_bytes < carve_forward(view).total) return fail(3, "hard_forward: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -3865,15 +4012,15 @@ int forward_entry(const rosa_problem* problem, const void* query, const void* ke
     case ROSA_DTYPE_F32:
       return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
                                          packed_key, routes, lengths, workspace, s, sign_words,
-                                         routed);
+                                         routed, words_given);
     case ROSA_DTYPE_F16:
       return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
                                          packed_key, routes, lengths, workspace, s, sign_words,
-                                         routed);
+                                         routed, words_given);
     default:
       return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
                                           packed_key, routes, lengths, workspace, s, sign_words,
-                                          routed);
+                                          routed, words_given);
   }
 }
 
@@ -3969,6 +4116,49 @@ int rosa_hip_hard_forward_bits(const rosa_problem* problem, const void* query, c
   if (!sign_words || !routed) return fail(2, "hard_forward_bits: NULL output pointer");
   return forward_entry(problem, query, key, value, nullptr, packed_query, packed_key, nullptr,
                        nullptr, workspace, workspace_bytes, stream, sign_words, routed);
+}
+
+int rosa_hip_hard_forward_words(const rosa_problem* problem, const int32_t* packed_query,
+                                const int32_t* packed_key, const void* value, void* output,
+                                uint32_t* sign_words, uint8_t* routed, int32_t* routes,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  if (!output && !(sign_words && routed))
+    return fail(2, "hard_forward_words: give the output tensor or both parts of its bit form");
+  if (output) { sign_words = nullptr; routed = nullptr; }
+  return forward_entry(problem, nullptr, nullptr, value, output, const_cast<int32_t*>(packed_query),
+                       const_cast<int32_t*>(packed_key), routes, nullptr, workspace,
+                       workspace_bytes, stream, sign_words, routed, true);
+}
+
+int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* routed,
+                                 int64_t tokens, int H, int Dv, const void* weight, int N,
+                                 const void* residual, void* out, void* stream) {
+  if (tokens < 0 || H < 1 || Dv < 1 || N < 1) return fail(1, "project_routed_bits: bad sizes");
+  if (tokens == 0) return 0;
+  if (!sign_words || !routed || !weight || !out) return fail(2, "project_routed_bits: NULL pointer");
+  const int64_t K = static_cast<int64_t>(H) * Dv;
+  if (Dv % 8 != 0 || !(32 % Dv == 0 || Dv % 32 == 0) || K % kProjectStep != 0 || K > INT32_MAX)
+    return fail(1, "project_routed_bits: the value width must be 8, 16 or a multiple of 32, and "
+                   "H * Dv a multiple of 32");
+  if (N % kProjectColumns != 0)
+    return fail(1, "project_routed_bits: the output width must be a multiple of 64");
+  const int64_t row_blocks = (tokens + kProjectRows - 1) / kProjectRows;
+  if (row_blocks > INT32_MAX || N / kProjectColumns > 65535)
+    return fail(1, "project_routed_bits: too many blocks");
+  ProjectParams P;
+  P.sign_words = sign_words;
+  P.routed = routed;
+  P.weight = static_cast<const uint16_t*>(weight);
+  P.residual = static_cast<const uint16_t*>(residual);
+  P.out = static_cast<uint16_t*>(out);
+  P.tokens = tokens;
+  P.H = H; P.Dv = Dv; P.nvw = value_words(Dv); P.N = N; P.K = static_cast<int>(K);
+  hipLaunchKernelGGL(project_routed_bits_kernel,
+                     dim3(static_cast<unsigned>(row_blocks), static_cast<unsigned>(N / kProjectColumns)),
+                     dim3(256), 0, static_cast<hipStream_t>(stream), P);
+  const hipError_t launch = hipGetLastError();
+  if (launch != hipSuccess) return fail_hip(launch, "project_routed_bits launch");
+  return 0;
 }
 
 int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query, const void* key,
