@@ -853,7 +853,8 @@ struct VjpParams {
   int symbols_by_head;          // grad_query / grad_key point to head-major accumulators
   int values_by_head;           // grad_value points to a head-major accumulator
   int32_t* work_counter;
-  const int32_t* header;        // [0] offsets flag, [1] work counter, [3] chunk records fit
+  const int32_t* header;        // [0] offsets flag, [1] work counter, [3] chunk records fit,
+                                // [4] the row-statistics pass met a long match
   float* checkpoints;           // one record per (band, 16-row chunk), or NULL
   int record_floats;            // kCheckpointFloats (+ kKeepBitFloats with dropout)
   int value_stride;             // value width of the tensors (L.Dv is the slice being processed)
@@ -976,7 +977,10 @@ template <bool VARLEN>
 __device__ __forceinline__ void init_row_stats(int64_t index, const Layout& L,
                                                float4* __restrict__ stats, float scale,
                                                int analytic, int32_t* __restrict__ work_counter) {
-  if (index == 0) *work_counter = 0;
+  if (index == 0) {
+    work_counter[0] = 0;
+    work_counter[3] = 0;  // header word 4: a long match was met
+  }
   const int64_t rows = static_cast<int64_t>(L.N) * L.H;
   if (index >= rows) return;
   // head-major index -> local row t
@@ -1606,6 +1610,8 @@ __device__ __forceinline__ v4f tile_row_sums(const float* tile_rows, int pitch, 
 // inputs at every width.
 constexpr int row_stats_waves(int dvp, bool dropout) { return dvp > 32 && dropout ? 3 : 4; }
 
+constexpr float kLongMatchEvidence = 6.0f;
+
 // Row-statistics pass: denominator and expected dropped utility of every row.
 // Rows are processed 16 at a time without any branch in between.  A chunk leaves
 // its route weights and its dropped weighted utilities as two [row][lane] tiles
@@ -2009,6 +2015,12 @@ void vjp_row_stats_kernel(VjpParams P) {
       // the sign bit of the window word tells the gradient pass that some overflow term
       // of the chunk is large enough to matter
       const bool noisy = __ballot(peak_overflow >= P.tail_threshold) != 0ull;
+      // The gradient pass carries its gate adjoints in two bfloat16 terms unless matches get
+      // long: their adjoints are much larger than the gradient sums they cancel in.  Evidence
+      // of kLongMatchEvidence at a chunk's end takes an exact match of at least that many rows
+      // (random symbols of eight bits never reach it).  Header word 4; every writer writes 1.
+      const bool long_match = __ballot(band.evidence >= kLongMatchEvidence) != 0ull;
+      if ((noisy || long_match) && lane == 0) P.work_counter[3] = 1;
       pending_window = window_before | (noisy ? INT32_MIN : 0);
       pending_kept = kept_bits;
       pending_first = chunk_first;
@@ -2192,11 +2204,20 @@ GradientBlockPlan plan_gradient_blocks(int dvp, int D, int value_words_per_colum
   return plan;
 }
 
-template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT, int NW>
+// TERMS: bfloat16 terms that carry a gate adjoint into the symbol contractions.  Two terms
+// hold it to 2^-18 of its size, which is enough where the terms of a gradient sum are of the
+// size of the sum.  Long matches make them much larger than the sum (a row's adjoints
+// cancel), so a launch in which the row-statistics pass has met a long match (evidence of
+// kLongMatchEvidence at the end of a chunk, or an overflow term that matters: header word 4)
+// runs the three-term form, 2^-21 by truncation; both forms are launched and the one that
+// does not apply returns at once.
+template <int NVW, int DVP, int DT, bool VARLEN, bool DROPOUT, int NW, int TERMS>
 __global__ __launch_bounds__(kWave * NW)
 __attribute__((amdgpu_waves_per_eu(gradient_waves((DVP + 15) / 16, DT))))
 void vjp_gradients_kernel(VjpParams P) {
   static_assert(NW == 1 || NW == 2, "blocks of one or two waves");
+  static_assert(TERMS == 2 || TERMS == 3, "two or three terms per gate adjoint");
+  if ((P.header[4] != 0) != (TERMS == 3)) return;
   constexpr int VT = (DVP + 15) / 16;   // value-dimension MFMA tiles
   constexpr bool kFetchAhead = true;  // row words and operands are fetched ahead of their use
   constexpr int SEG = gradient_segment(DVP);  // rows staged in LDS at a time
@@ -2864,9 +2885,13 @@ void vjp_gradients_kernel(VjpParams P) {
               const float b = fmaf(gate_below, adjoint_carry, keep_adjoint[r]);
               adjoint_carry = b;
               gate_below = keep_gate[r];
-              uint32_t rest;
-              tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(b * keep_evidence[r], rest);
-              rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
+              if constexpr (TERMS == 2) {
+                tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16(b * keep_evidence[r]);
+              } else {
+                uint32_t rest;
+                tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(b * keep_evidence[r], rest);
+                rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
+              }
             }
           } else {
 #pragma unroll
@@ -2897,9 +2922,13 @@ void vjp_gradients_kernel(VjpParams P) {
             const float h = fmaf(b, keep_evidence[r], -ring_sum);
             if (ring_live == 0) ring_sum = 0.0f;
             const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
-            uint32_t rest;
-            tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(active ? h : 0.0f, rest);
-            rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
+            if constexpr (TERMS == 2) {
+              tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16(active ? h : 0.0f);
+            } else {
+              uint32_t rest;
+              tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16_exact(active ? h : 0.0f, rest);
+              rest_plane[r * (kRestPitch + 1) + 64 - lane] = static_cast<uint16_t>(rest >> 16);
+            }
           }
           }
           wave_lds_fence();
@@ -2910,6 +2939,7 @@ void vjp_gradients_kernel(VjpParams P) {
             column_operands(adjoints);
 #pragma unroll
             for (int m = 0; m < kWindowTiles; ++m) {
+              if constexpr (TERMS == 2) break;
               const uint16_t* column = rest_plane + 16 * m + li;
               const int r = 4 * lg;
               adjoint_rests[m] = v2u{
@@ -2933,12 +2963,14 @@ void vjp_gradients_kernel(VjpParams P) {
               for (int m = 0; m < kWindowTiles; ++m) {
                 key_acc[m][n] = mfma_bf16(adjoints[m], symbols, key_acc[m][n]);
               }
-              mfma_shape_change();
+              if constexpr (TERMS == 3) {
+                mfma_shape_change();
 #pragma unroll
-              for (int m = 0; m < kWindowTiles; ++m) {
-                key_acc[m][n] = mfma_bf16_k16(adjoint_rests[m], symbols_once, key_acc[m][n]);
+                for (int m = 0; m < kWindowTiles; ++m) {
+                  key_acc[m][n] = mfma_bf16_k16(adjoint_rests[m], symbols_once, key_acc[m][n]);
+                }
+                mfma_shape_change();
               }
-              mfma_shape_change();
             }
           }
           // row sums: rows are complete for this band after the chunk
@@ -2966,8 +2998,10 @@ void vjp_gradients_kernel(VjpParams P) {
               const int c0 = 4 * kWindowTiles * lg + 4 * step;
               k_words_of[slot] = *reinterpret_cast<const uint4*>(key_tile + c0);
               adjoints_of[slot] = *reinterpret_cast<const v4u*>(tile_bits + li * kTilePitch + c0);
-              adjoint_rests_of[slot] =
-                  *reinterpret_cast<const v2u*>(rest_plane + li * kRestPitch + c0);
+              if constexpr (TERMS == 3) {
+                adjoint_rests_of[slot] =
+                    *reinterpret_cast<const v2u*>(rest_plane + li * kRestPitch + c0);
+              }
             };
             if constexpr (kReadsFirst) {
 #pragma unroll
@@ -2988,7 +3022,9 @@ void vjp_gradients_kernel(VjpParams P) {
                 const v2u symbols_once = {__builtin_amdgcn_perm(symbols[1], symbols[0], 0x07060100u),
                                           __builtin_amdgcn_perm(symbols[3], symbols[2], 0x07060100u)};
                 query_part[step & 1][n] = mfma_bf16(adjoints, symbols, query_part[step & 1][n]);
-                query_part[2][n] = mfma_bf16_k16(adjoint_rests, symbols_once, query_part[2][n]);
+                if constexpr (TERMS == 3) {
+                  query_part[2][n] = mfma_bf16_k16(adjoint_rests, symbols_once, query_part[2][n]);
+                }
               }
             }
 #pragma unroll
@@ -3507,11 +3543,16 @@ int launch_vjp_passes(const VjpParams& P, const VjpWorkspace& w, bool analytic,
   Q.row_queue = plan.row_queue ? 1 : 0;
   const unsigned blocks = static_cast<unsigned>(std::max(1, w.resident_blocks / plan.waves));
   stage_begin(kStageGradients, stream);
+  // both forms of the kernel (see its TERMS): the one that does not apply returns at once
   if (plan.waves == 2) {
-    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 2>), dim3(blocks),
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 2, 2>), dim3(blocks),
+                       dim3(kWave * 2), plan.lds_bytes, stream, Q);
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 2, 3>), dim3(blocks),
                        dim3(kWave * 2), plan.lds_bytes, stream, Q);
   } else {
-    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 1>), dim3(blocks),
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 1, 2>), dim3(blocks),
+                       dim3(kWave), plan.lds_bytes, stream, Q);
+    hipLaunchKernelGGL((vjp_gradients_kernel<NVW, DVP, DT, VARLEN, DROPOUT, 1, 3>), dim3(blocks),
                        dim3(kWave), plan.lds_bytes, stream, Q);
   }
   stage_end(kStageGradients, stream);
