@@ -297,12 +297,18 @@ __host__ __device__ inline int64_t band_steps_before(int len, int band) {
 }
 
 // The row-statistics pass leaves a record per 16-row chunk of a band for the gradient
-// pass: (S, window) of every diagonal before the chunk's first row and, with dropout,
-// the keep decisions of the chunk (bit r of lane l's 16-bit word = row r, diagonal l).
+// pass, 64 lanes each: S of every diagonal before the chunk's first row (float), the window
+// count there as 16 bits (saturated at kRecordWindowMax; bit 15 is set, in every lane, when
+// some overflow term of the chunk is large enough to matter) and, with dropout, the keep
+// decisions of the chunk (bit r of lane l's 16-bit word = row r, diagonal l): 0.375 bytes
+// per pair, 0.5 with dropout.  A saturated count is exact where it matters: the launch keeps
+// records only when every count that can still produce a relevant overflow term within a
+// chunk lies below the saturation value.
 // Chunk c of the band with global step offset `steps_before` and global band number
 // `bands_before` owns slot steps_before / 16 + bands_before + c (distinct for all
 // chunks of all bands, because a band of n steps has fewer than n / 16 + 2 chunks).
-constexpr int kCheckpointFloats = 128;  // [S | window][64 lanes]
+constexpr int kRecordWindowMax = 0x7fff;
+constexpr int kCheckpointFloats = 96;   // S [64 lanes], then the 16-bit window words
 constexpr int kKeepBitFloats = 32;      // 64 lanes x 16 bits
 __host__ __device__ inline int64_t checkpoint_slots(int64_t steps, int64_t bands) {
   return steps / 16 + bands + 1;
@@ -861,6 +867,7 @@ struct VjpParams {
   int value_offset;             // first value dimension of the slice
   float* block_scratch;         // per resident block: ring + segment checkpoints
   int64_t block_scratch_floats;
+  int segment_group;            // segments per group of the fallback checkpoints (see carve_vjp)
   int ring_rows;                // W + 1 clipped to the longest possible diagonal
   int total_units;
   int wave_lds_floats;          // LDS floats each wave of a gradient block owns
@@ -1766,7 +1773,7 @@ void vjp_row_stats_kernel(VjpParams P) {
     if (view.checkpoints != nullptr) {
       float* slot =
           view.checkpoints + static_cast<int64_t>(pending_first / kChunk) * view.record_floats;
-      slot[kWave + lane] = __int_as_float(pending_window);
+      reinterpret_cast<uint16_t*>(slot + kWave)[lane] = static_cast<uint16_t>(pending_window);
       if constexpr (DROPOUT) {
         // the gradient pass reads the decisions back instead of hashing again
         reinterpret_cast<uint16_t*>(slot + kCheckpointFloats)[lane] =
@@ -2012,7 +2019,7 @@ void vjp_row_stats_kernel(VjpParams P) {
                               : e == 2 ? numerator_sums[2] : numerator_sums[3];
         if constexpr (DROPOUT) pending_numerator_sum *= P.inverse_keep;
       }
-      // the sign bit of the window word tells the gradient pass that some overflow term
+      // bit 15 of the window word tells the gradient pass that some overflow term
       // of the chunk is large enough to matter
       const bool noisy = __ballot(peak_overflow >= P.tail_threshold) != 0ull;
       // The gradient pass carries its gate adjoints in two bfloat16 terms unless matches get
@@ -2021,7 +2028,7 @@ void vjp_row_stats_kernel(VjpParams P) {
       // (random symbols of eight bits never reach it).  Header word 4; every writer writes 1.
       const bool long_match = __ballot(band.evidence >= kLongMatchEvidence) != 0ull;
       if ((noisy || long_match) && lane == 0) P.work_counter[3] = 1;
-      pending_window = window_before | (noisy ? INT32_MIN : 0);
+      pending_window = min(window_before, kRecordWindowMax) | (noisy ? 0x8000 : 0);
       pending_kept = kept_bits;
       pending_first = chunk_first;
       pending_rows = rows_here;
@@ -2287,7 +2294,11 @@ void vjp_gradients_kernel(VjpParams P) {
   // before every segment of the band
   float* ck_evidence = ring + static_cast<int64_t>(P.ring_rows) * kWave;   // [SEG_CHUNKS][64]
   int* ck_window = reinterpret_cast<int*>(ck_evidence + SEG_CHUNKS * kWave);
-  float* seg_ck = ck_evidence + 2 * kCheckpointChunksMax * kWave;  // [(S, window)][64] per segment
+  // without records, two levels of (S, window) checkpoints: before every group of
+  // `segment_group` segments of the band (one forward sweep over the band), and before every
+  // segment of the group the reverse walk is in (one more sweep over that group)
+  float* group_ck = ck_evidence + 2 * kCheckpointChunksMax * kWave;  // [group][(S, window)][64]
+  const int G = P.segment_group;
 
   // zero the tile once: its margins are never written again
   for (int index = lane; index < kChunk * kTilePitch; index += kWave) tile[index] = 0.0f;
@@ -2346,22 +2357,32 @@ void vjp_gradients_kernel(VjpParams P) {
     // Without stored checkpoints, a band-level forward sweep leaves (S, window) before the
     // first row of every segment and a segment-level one before every chunk.
     const bool stored = have_band && view.checkpoints != nullptr;
-    if (have_band && !stored && segments > 1) {
-      band.evidence = 0.0f;
-      band.window = 0;
-      load_sliding<NVW>(band, view, 0, lane, W);
-      for (int segment = 0; segment < segments - 1; ++segment) {
-        seg_ck[(2 * segment) * kWave + lane] = band.evidence;
-        seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+    const int groups = (segments + G - 1) / G;
+    float* seg_ck = group_ck + static_cast<int64_t>(2 * groups) * kWave;  // [segment of the group]
+    // sweep over segments [from, to) starting from `band`, leaving the state before each of
+    // them where `keep` says; the state after the last one is not needed
+    const auto sweep_segments = [&](int from, int to, auto keep) {
+      load_sliding<NVW>(band, view, from * SEG, lane, W);
+      for (int segment = from; segment < to; ++segment) {
+        keep(segment);
+        if (segment + 1 == to) break;
         const int first = segment * SEG;
         wave_lds_fence();
         stage_rows<NVW, kRowSymbols>(view, first, SEG, lane, rows, W);
         wave_lds_fence();
         sweep_rows<NVW>(band, rows, first, SEG, lane, W, P.gate_log2);
       }
-      const int segment = segments - 1;
-      seg_ck[(2 * segment) * kWave + lane] = band.evidence;
-      seg_ck[(2 * segment + 1) * kWave + lane] = __int_as_float(band.window);
+    };
+    if (have_band && !stored && segments > 1) {
+      band.evidence = 0.0f;
+      band.window = 0;
+      // (the sweep ends with the last group's first segment: nothing later is kept)
+      sweep_segments(0, (groups - 1) * G + 1, [&](int segment) {
+        if (segment % G == 0) {
+          group_ck[(2 * (segment / G)) * kWave + lane] = band.evidence;
+          group_ck[(2 * (segment / G) + 1) * kWave + lane] = __int_as_float(band.window);
+        }
+      });
     }
 
     // reverse state carried across chunks and segments
@@ -2484,7 +2505,7 @@ void vjp_gradients_kernel(VjpParams P) {
       const float* slot =
           view.checkpoints + static_cast<int64_t>(chunk_index) * view.record_floats;
       record_evidence = slot[lane];
-      record_window = __float_as_int(slot[kWave + lane]);
+      record_window = reinterpret_cast<const uint16_t*>(slot + kWave)[lane];
       if constexpr (DROPOUT) {
         record_kept = reinterpret_cast<const uint16_t*>(slot + kCheckpointFloats)[lane];
       }
@@ -2500,8 +2521,18 @@ void vjp_gradients_kernel(VjpParams P) {
       if (segment_active) {
       if (!stored) {
         if (segments > 1) {
-          band.evidence = seg_ck[(2 * segment) * kWave + lane];
-          band.window = __float_as_int(seg_ck[(2 * segment + 1) * kWave + lane]);
+          if (segment == segments - 1 || segment % G == G - 1) {
+            // the walk enters a group: the state before each of its segments up to this one
+            const int group = segment / G;
+            band.evidence = group_ck[(2 * group) * kWave + lane];
+            band.window = __float_as_int(group_ck[(2 * group + 1) * kWave + lane]);
+            sweep_segments(group * G, segment + 1, [&](int inner) {
+              seg_ck[(2 * (inner % G)) * kWave + lane] = band.evidence;
+              seg_ck[(2 * (inner % G) + 1) * kWave + lane] = __int_as_float(band.window);
+            });
+          }
+          band.evidence = seg_ck[(2 * (segment % G)) * kWave + lane];
+          band.window = __float_as_int(seg_ck[(2 * (segment % G) + 1) * kWave + lane]);
         } else {
           band.evidence = 0.0f;
           band.window = 0;
@@ -2687,9 +2718,10 @@ void vjp_gradients_kernel(VjpParams P) {
                        : "=&v"(band.evidence), "=&v"(window_word)
                        : "v"(evidence_in), "v"(window_in));
         }
-        band.window = window_word & INT32_MAX;
         // stored records say whether any overflow term of the chunk matters
-        const bool chunk_quiet = stored && __builtin_amdgcn_readfirstlane(window_word) >= 0;
+        const bool chunk_quiet =
+            stored && (__builtin_amdgcn_readfirstlane(window_word) & 0x8000) == 0;
+        band.window = stored ? (window_word & kRecordWindowMax) : window_word;
         // sliding registers of the chunk's first step: column first - lane
         band.key_word = key_window[local + 63 - lane];
         band.old_key_word = old_key_window[local + 63 - lane];
@@ -3315,9 +3347,14 @@ ForwardWorkspace carve_forward(const ProblemView& v) {
 constexpr int kValueSlice = 64;  // value dimensions one backward pass covers
 constexpr int kNarrowRow = 8;    // gradient rows up to this many floats are accumulated head-major
 
-// bytes of chunk records the backward workspace may hold (4 GiB unless the caller lowers it)
+// bytes of chunk records the backward workspace may hold unless the caller sets a limit:
+// at most 4 GiB, and in a packed layout, whose sequence lengths the host does not know, at
+// most 1.5 KiB per token and head (what sequences of about 6 000 tokens need with dropout;
+// longer ones make the device fall back to rebuilding the evidence in the gradient pass)
 constexpr size_t kDefaultRecordBudget = size_t(1) << 32;
-size_t g_record_budget_bytes = kDefaultRecordBudget;
+constexpr size_t kPackedRecordBytesPerRow = 1536;
+constexpr size_t kNoRecordBudget = static_cast<size_t>(-1);
+size_t g_record_budget_bytes = kNoRecordBudget;  // set by rosa_hip_set_record_budget
 
 int value_words(int Dv) { return (Dv + 31) / 32; }
 
@@ -3338,6 +3375,7 @@ struct VjpWorkspace {
   int record_floats;
   int resident_blocks;
   int64_t block_scratch_floats;
+  int segment_group;
   int ring_rows;
 };
 
@@ -3373,8 +3411,12 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.checkpoints = cursor;
   w.record_floats = kCheckpointFloats + (dropout ? kKeepBitFloats : 0);
   {
-    const int64_t budget =
-        static_cast<int64_t>(g_record_budget_bytes / (sizeof(float) * w.record_floats));
+    size_t budget_bytes = g_record_budget_bytes;
+    if (budget_bytes == kNoRecordBudget) {
+      budget_bytes = kDefaultRecordBudget;
+      if (v.L.varlen) budget_bytes = std::min(budget_bytes, kPackedRecordBytesPerRow * rows);
+    }
+    const int64_t budget = static_cast<int64_t>(budget_bytes / (sizeof(float) * w.record_floats));
     const int64_t steps = v.L.varlen
         ? static_cast<int64_t>(v.L.H) * band_steps_total(v.L.N)
         : static_cast<int64_t>(v.L.B) * v.L.H * band_steps_total(v.L.T);
@@ -3389,12 +3431,21 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   // one fallback checkpoint per segment of the longest possible band, for a wave that finds
   // no records: never the case in a dense layout whose records fit (known here), decided on
   // the device in a packed one
-  const bool may_run_without_records = v.L.varlen != 0 || w.checkpoint_capacity == 0;
+  // (nor in one whose window counts the records can always hold: see the launch)
+  const bool may_run_without_records =
+      v.L.varlen != 0 || w.checkpoint_capacity == 0 ||
+      (static_cast<int64_t>(w.ring_rows) * v.L.D > kRecordWindowMax);
   const int max_segments =
       may_run_without_records ? (longest + segment_rows - 1) / segment_rows + 1 : 0;
+  // two levels: a checkpoint per group of G segments and one per segment of a group, with G
+  // near the square root of the segment count
+  w.segment_group = 4;
+  while (w.segment_group * w.segment_group < max_segments) ++w.segment_group;
+  const int max_groups = max_segments > 0 ? (max_segments + w.segment_group - 1) / w.segment_group : 0;
   w.block_scratch_floats = static_cast<int64_t>(w.ring_rows) * kWave +
                            2 * kCheckpointChunksMax * kWave +
-                           static_cast<int64_t>(max_segments) * 2 * kWave;
+                           static_cast<int64_t>(max_segments > 0 ? max_groups + w.segment_group : 0) *
+                               2 * kWave;
   const int64_t units = static_cast<int64_t>(v.L.slots) * v.L.H;
   // resident waves of the gradient kernel (an even number: its blocks hold one or two waves)
   w.resident_blocks = static_cast<int>(std::min<int64_t>(
@@ -3710,12 +3761,21 @@ int run_vjp(const rosa_problem* p, const ProblemView& view, const void* query, c
     P.values_by_head = w.values_by_head ? 1 : 0;
     P.work_counter = counter;
     P.header = at<int32_t>(workspace, w.header);
-    P.checkpoints = w.checkpoint_capacity > 0 ? at<float>(workspace, w.checkpoints) : nullptr;
+    // The records hold saturated window counts: they are kept when no count can saturate, or
+    // when every count that can still produce a relevant overflow term within a chunk lies
+    // below the saturation value (otherwise, with a long window and a tiny mismatch_scale,
+    // the gradient pass rebuilds the evidence itself).
+    const bool windows_fit =
+        static_cast<int64_t>(w.ring_rows) * L.D <= kRecordWindowMax ||
+        -std::log2(P.tail_threshold) / P.gate_log2 + kChunk * L.D + 2 <= kRecordWindowMax;
+    P.checkpoints = (w.checkpoint_capacity > 0 && windows_fit) ? at<float>(workspace, w.checkpoints)
+                                                              : nullptr;
     P.record_floats = w.record_floats;
     P.value_stride = full_width;
     P.value_offset = value_offset;
     P.block_scratch = at<float>(workspace, w.block_scratch);
     P.block_scratch_floats = w.block_scratch_floats;
+    P.segment_group = w.segment_group;
     P.ring_rows = w.ring_rows;
     P.total_units = L.slots * L.H;
     const bool dropout = dropout_p > 0.0f;
@@ -4361,7 +4421,7 @@ void rosa_hip_set_gradient_block_waves(int waves) {
 }
 
 void rosa_hip_set_record_budget(size_t bytes) {
-  g_record_budget_bytes = bytes == static_cast<size_t>(-1) ? kDefaultRecordBudget : bytes;
+  g_record_budget_bytes = bytes;  // (size_t)-1: the default
 }
 
 int rosa_hip_stage_timing(int enable) {

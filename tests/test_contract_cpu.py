@@ -240,6 +240,34 @@ def test_c_abi_library_exports_every_declared_symbol():
     assert b"[1, 32]" in loaded.rosa_hip_last_error()
 
 
+def test_backward_workspace_sizes_at_training_shapes():
+    """Host arithmetic of the backward workspace (no device call): the chunk records cost half
+    a byte per pair with dropout, a packed layout is capped per token and head, and forbidding
+    the records makes the workspace of a training shape much smaller."""
+
+    from rosa_soft_amd import cabi
+
+    loaded = cabi.load()
+    size = lambda problem, dropout: loaded.rosa_hip_vjp_workspace_bytes(
+        ctypes.byref(problem), 7, 1.0, int(dropout))
+    metric = cabi.RosaProblem(dtype=0, B=2, T=4096, N=8192, S=0, H=64, D=8, Hv=16, Dv=8, W=128)
+    pairs = 2 * 64 * 4096 * 4095 // 2
+    cabi.set_record_budget(None)
+    try:
+        with_dropout, without_dropout = size(metric, True), size(metric, False)
+        assert 0.5 * pairs < with_dropout < 0.5 * pairs + 200 * 2 ** 20
+        assert 0.375 * pairs < without_dropout < 0.375 * pairs + 200 * 2 ** 20
+        cabi.set_record_budget(0)
+        assert size(metric, True) < 300 * 2 ** 20
+        cabi.set_record_budget(None)
+        # configuration 5: 32 768 packed tokens, 64 heads (cu_seqlens is not read by the query)
+        packed = cabi.RosaProblem(dtype=2, B=0, T=0, N=32768, S=8, H=64, D=32, Hv=8, Dv=32, W=64)
+        packed.cu_seqlens = 1  # any non-null address: the size query never dereferences it
+        assert size(packed, True) < 1536 * 32768 * 64 + 400 * 2 ** 20
+    finally:
+        cabi.set_record_budget(None)
+
+
 def test_gradient_launch_plan_follows_the_shape():
     """Host arithmetic of the gradient kernel's launch form (no device call): blocks of two
     waves where the tiles are wide and bands outnumber the resident waves, the row queue

@@ -367,7 +367,7 @@ def test_packed_record_budget_on_both_sides_of_the_device_decision(cabi, c_oracl
         bands = (length - 2) // 64 + 1
         return bands * (length - 1) - 32 * bands * (bands - 1)
 
-    record_bytes = 4 * (128 + 32)  # (S, window) of 64 diagonals + 16 keep bits per lane
+    record_bytes = 4 * (96 + 32)  # S and a 16-bit window count of 64 diagonals + 16 keep bits per lane
     slots = lambda parts: (H * sum(band_steps(n) for n in parts)) // 16 \
         + H * sum((n + 63) // 64 for n in parts) + 1
     needed, worst = slots(lengths) * record_bytes, slots([total]) * record_bytes
