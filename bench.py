@@ -48,6 +48,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 FP32_MATRIX_PEAK_TFLOPS = 157.3
+# vector ALU: 256 CUs x 4 SIMDs x 16 lanes per clock at the 2.4 GHz peak engine clock
+VALU_PEAK_LANE_OPS = 256 * 4 * 16 * 2.4e9
 
 # name: dense  -> dict(B, T, H, D, Hv, Dv, W, p, ms, dtype, pattern)
 #       packed -> dict(lengths, H, D, Hv, Dv, W, p, ms, dtype)
@@ -281,6 +283,39 @@ def roofline_fractions(measured: dict) -> dict:
     return out
 
 
+def algorithmic_lane_ops(config) -> dict:
+    """Vector lane operations per (row, route) pair that the diagonal recurrence itself needs,
+    one per arithmetic instruction of a lane, whatever its issue rate (32-bit integer
+    multiplies and sqrt/exp2/rsq take four issue slots each on CDNA4, which the count ignores).
+
+    Row statistics: gate (xor, popcount, table) 3, suffix score 1, window term 2, logit
+    (sqrt, fma, exp2) 3, normaliser and expectation sums 2, utility 1 = 12; the dropout hash adds
+    five rounds of (xor, multiply, shift, xor, multiply), the closing fold and the compare, 28.
+    Gradients: the same replay without the sums 9, probability 1, keep bit and utility 2,
+    route adjoint (rsq, two products) 3, weight as two bfloat16 terms 4, reverse carry 1,
+    window sum 2, gate adjoint 1, its two bfloat16 terms 4 = 27.
+    """
+
+    hashed = 28 if config["p"] > 0 else 0
+    return {"vjp_row_stats": 12 + hashed, "vjp_gradients": 27}
+
+
+def valu_fractions(measured: dict) -> dict:
+    """The vector-ALU roof of the two backward kernels: algorithmic lane operations per pair
+    (`algorithmic_lane_ops`) x pairs over the kernel's time, against the VALU peak."""
+
+    pairs = pair_count(measured["config"])
+    out = {}
+    for stage, per_pair in algorithmic_lane_ops(measured["config"]).items():
+        ms = measured["stage_ms"].get(stage)
+        if ms:
+            rate = per_pair * pairs / (ms * 1e-3)
+            out[stage] = dict(lane_ops_per_pair=per_pair, achieved=rate / 1e12,
+                              peak=VALU_PEAK_LANE_OPS / 1e12, unit="T lane-op/s",
+                              frac=rate / VALU_PEAK_LANE_OPS)
+    return out
+
+
 def atomic_row_segments(config, plan: dict) -> int:
     """64-byte row segments the float atomics of one gradient-kernel launch touch.
 
@@ -326,6 +361,8 @@ def config_summary(measured: dict) -> dict:
         vjp_gradients_ms=round(measured["stage_ms"].get("vjp_gradients", float("nan")), 4),
         vjp_row_stats_ms=round(measured["stage_ms"].get("vjp_row_stats", float("nan")), 4),
         vjp_gradients_frac=round(fractions.get("vjp_gradients", {}).get("frac", float("nan")), 4),
+        vjp_gradients_valu_frac=round(
+            valu_fractions(measured).get("vjp_gradients", {}).get("frac", float("nan")), 4),
         whole_backward_frac=round(fractions.get("whole_backward", {}).get("frac", float("nan")), 4),
         waves_per_block=measured["gradient_block_plan"]["waves"],
         atomic_row_segments=atomic_row_segments(config, measured["gradient_block_plan"]),
@@ -333,6 +370,16 @@ def config_summary(measured: dict) -> dict:
 
 
 PROFILE_FIGURE = re.compile(r"^bench: (\w+) = ([-+0-9.eE]+)\s*$", re.MULTILINE)
+PROFILE_SOURCE = re.compile(r"^bench-source: ([0-9a-f]{16})\s*$", re.MULTILINE)
+
+
+def kernel_source_digest() -> str:
+    """Digest of the HIP source and flags the library is built from; the counter summaries
+    under profiles/ carry the digest of what they measured."""
+
+    from rosa_soft_amd import _build
+
+    return _build.source_digest()
 
 
 def profile_figures(workload: str) -> dict:
@@ -341,16 +388,22 @@ def profile_figures(workload: str) -> dict:
     The rocprofv3 summaries under profiles/ end in lines `bench: name = value`; those are
     what a counter run measured for this workload (HBM bytes per launch of the gradient
     kernel, busy fractions of the VALU and matrix pipes, issued matrix instructions).
-    A workload without summaries yields an empty dict, never a guess.
+    A workload without summaries yields an empty dict, never a guess; `stale` is set when a
+    summary was taken from another version of the kernel source than the one in the tree.
     """
 
     figures = {}
+    stale = False
     for suffix in ("backward_hbm_traffic", "backward_issue_counters"):
         path = os.path.join(ROOT, "profiles", f"{workload}_{suffix}.md")
         if os.path.exists(path):
             with open(path) as handle:
-                for name, value in PROFILE_FIGURE.findall(handle.read()):
-                    figures[name] = float(value)
+                text = handle.read()
+            for name, value in PROFILE_FIGURE.findall(text):
+                figures[name] = float(value)
+            stale = stale or PROFILE_SOURCE.findall(text) != [kernel_source_digest()]
+    if figures:
+        figures["stale"] = stale
     return figures
 
 
@@ -395,8 +448,15 @@ def training_record(args) -> dict:
                 "read from the rocprofv3 summaries under profiles/ (null when this workload "
                 "has none)",
     }
+    valu = valu_fractions(measured)
+    roofline["valu"] = dict(valu.get("vjp_gradients", {}), row_stats_kernel=valu.get("vjp_row_stats"),
+                            note="algorithmic vector lane operations per pair (stated in "
+                                 "algorithmic_lane_ops) x pairs / kernel time, against 256 CUs x 4 "
+                                 "SIMDs x 16 lanes x 2.4 GHz; the roof that binds at D = Dv = 8")
     if figures:
-        roofline["issue"] = {k: v for k, v in figures.items() if k != "traffic_bytes_per_launch"}
+        roofline["issue"] = {k: v for k, v in figures.items()
+                             if k not in ("traffic_bytes_per_launch", "stale")}
+        roofline["profile_figures_stale"] = figures["stale"]
     # the other bound of the gradient kernel: its global float atomics, priced against the
     # rate measured on this GPU in this run
     from rosa_soft_amd import cabi

@@ -67,7 +67,9 @@ size_t rosa_hip_vjp_workspace_bytes(const rosa_problem* problem, int gradient_ma
  * 4 GiB, (size_t)-1 restores it, 0 forbids the records.  A backward whose records do not
  * fit recomputes instead (forward sweeps and a second hash evaluation in the gradient
  * pass): same results, less memory, more time.  Process-wide; call it before sizing the
- * workspace.  The reference has no counterpart (its backward keeps no state between
+ * workspace, and not while another thread sizes a workspace or runs a backward: the value
+ * is read atomically, but a size query and the launch it was made for must see the same
+ * one.  The reference has no counterpart (its backward keeps no state between
  * kernels); the knob exists for callers that must bound the workspace.
  */
 void rosa_hip_set_record_budget(size_t bytes);
@@ -77,9 +79,23 @@ void rosa_hip_set_record_budget(size_t bytes);
  * shape (the default).  With two waves the blocks own pairs of neighbouring diagonal bands
  * and add their column sums in LDS before the global atomics.  The reference has no
  * counterpart (one block per row there); the knob exists for measurements and so that
- * tests can run both forms on small problems.
+ * tests can run both forms on small problems.  Process-wide, with the same rule as the
+ * record budget: do not change it between a size query and its launch, nor while another
+ * thread does either.
  */
 void rosa_hip_set_gradient_block_waves(int waves);
+
+/*
+ * Rows of a piece of a diagonal band in the backward's gradient kernel: 0 for the library's
+ * choice by shape (the default: bands are cut only when there are fewer than two of them per
+ * resident wave, into pieces of at least four windows), -1 for never, or a number of rows
+ * (rounded up to whole 32-row segments, at least 64).  Pieces of one band are walked by
+ * different waves, each starting max_suffix_length - 1 rows below its last row.  No
+ * counterpart in the reference; the knob exists for measurements and so that tests can
+ * force cuts on small problems.  Like the other setters it must not race with size queries
+ * or launches of other threads.
+ */
+void rosa_hip_set_gradient_piece_rows(int rows);
 
 /*
  * How the backward's gradient kernel will be launched for `problem` (no counterpart in the
@@ -192,6 +208,9 @@ int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* rout
  * workspace fits, i.e. about tokens * H <= 4 190 000, and returns 3 with a message
  * beyond that.  All calls on one GPU share that GPU's array: calls that overlap in time
  * on one GPU (different streams or threads) race and must be ordered by the caller.
+ * The first call on a device looks up the array's address (hipGetSymbolAddress), which is
+ * not a stream operation: make that call before recording the stream into a graph; every
+ * later call on the device is kernel launches only.
  * Outputs and their meaning are those of rosa_hip_hard_forward.
  */
 int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query,

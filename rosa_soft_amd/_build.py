@@ -8,6 +8,7 @@
 
 from __future__ import annotations
 
+import hashlib
 import json
 import os
 import re
@@ -23,6 +24,14 @@ ROCM_HOME = os.environ.get("ROCM_HOME", "/opt/rocm")
 OFFLOAD_ARCH = "gfx950"
 
 HIP_SOURCE = os.path.join(HERE, "csrc", "rosa_kernels.hip")
+# the band kernels of the backward, compiled once per tile family (sign words per value
+# column, padded value width, symbol tiles) so that the families build side by side
+INSTANCES_SOURCE = os.path.join(HERE, "csrc", "rosa_vjp_instances.hip")
+TILE_FAMILIES = [(1, 8, 1), (1, 8, 2), (1, 16, 1), (1, 16, 2), (1, 32, 1), (1, 32, 2),
+                 (2, 64, 1), (2, 64, 2)]
+HIP_HEADERS = [os.path.join(HERE, "csrc", name)
+               for name in ("rosa_device_common.hpp", "rosa_vjp_bands.hpp")]
+OBJECT_DIR = os.path.join(HERE, "build_objects")
 HIP_LIBRARY = os.path.join(HERE, "librosa_soft_hip.so")
 DISPATCH_SOURCE = os.path.join(HERE, "csrc", "rosa_dispatch.cpp")
 # registers, spills, scratch and LDS of every kernel, as the compiler reported them
@@ -31,7 +40,7 @@ RESOURCE_REPORT = os.path.join(HERE, "kernel_resources.json")
 # -packed-fp32-ops is switched off on purpose: some packed-FP32 forms have
 # produced silently wrong results on this hardware generation.
 HIPCC_FLAGS = [
-    f"--offload-arch={OFFLOAD_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+    f"--offload-arch={OFFLOAD_ARCH}", "-O3", "-std=c++17", "-fPIC",
     "-munsafe-fp-atomics", "-Wno-pass-failed",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
@@ -47,8 +56,16 @@ RESOURCE_REMARK = re.compile(r"remark:\s+([A-Za-z /\[\]]+?):\s+(\S+) \[-Rpass-an
 
 def _run(command: List[str]) -> str:
     print("+", " ".join(shlex.quote(part) for part in command), flush=True)
-    completed = subprocess.run(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    return _report(subprocess.run(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                                  text=True))
+
+
+def _report(completed) -> str:
+    """Print what a finished build step said, without the compiler's known noise."""
+
     noise = ("packed-fp32-ops", "is not a recognized feature", "kernel-resource-usage")
+    if completed.returncode == 0:
+        noise += ("In file included from",)  # the include trail of a remark
     lines, skip_excerpt = [], 0
     for line in completed.stdout.splitlines():
         if "kernel-resource-usage" in line and "Function Name" in line:
@@ -84,16 +101,59 @@ def kernel_resources(compiler_output: str) -> Dict[str, Dict[str, int]]:
     return report
 
 
+# entry of the resource report that names what was compiled (see source_digest)
+BUILD_RECORD = "__build__"
+
+
+def source_digest() -> str:
+    """First 16 hex digits of the SHA-256 of the HIP source and the compiler flags: what a
+    resource report or a counter summary must name to speak for the library in the tree."""
+
+    digest = hashlib.sha256()
+    for path in (HIP_SOURCE, INSTANCES_SOURCE, *HIP_HEADERS):
+        with open(path, "rb") as handle:
+            digest.update(handle.read())
+    digest.update(" ".join(HIPCC_FLAGS).encode())
+    return digest.hexdigest()[:16]
+
+
 def build_hip_library() -> str:
+    """Compile the main translation unit and the eight tile families side by side, then link.
+
+    One compiler process per translation unit; the families take one to two minutes each,
+    which is also the build's wall time on eight cores."""
+
+    from concurrent.futures import ThreadPoolExecutor
+
     hipcc = os.path.join(ROCM_HOME, "bin", "hipcc")
-    output = _run([hipcc, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", HIP_SOURCE,
-                   "-o", HIP_LIBRARY])
+    digest = source_digest()  # of what the compilers are about to read
+    os.makedirs(OBJECT_DIR, exist_ok=True)
+    jobs = [([hipcc, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", HIP_SOURCE],
+             os.path.join(OBJECT_DIR, "rosa_kernels.o"))]
+    for nvw, dvp, symbol_tiles in TILE_FAMILIES:
+        jobs.append(([hipcc, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage",
+                      f"-DROSA_FAMILY_NVW={nvw}", f"-DROSA_FAMILY_DVP={dvp}",
+                      f"-DROSA_FAMILY_DT={symbol_tiles}", "-c", INSTANCES_SOURCE],
+                     os.path.join(OBJECT_DIR, f"rosa_vjp_{nvw}_{dvp}_{symbol_tiles}.o")))
+
+    def compile_one(job):
+        command = [*job[0], "-o", job[1]]
+        print("+", " ".join(shlex.quote(part) for part in command), flush=True)
+        return subprocess.run(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+
+    workers = max(1, min(len(jobs), os.cpu_count() or 1, 16))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        finished = list(pool.map(compile_one, jobs))
+    output = "".join(_report(completed) for completed in finished)
+    _run([hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC",
+          *(job[1] for job in jobs), "-o", HIP_LIBRARY])
     report = kernel_resources(output)
+    report[BUILD_RECORD] = {"source_digest": digest}
     with open(RESOURCE_REPORT, "w") as handle:
         json.dump(report, handle, indent=0, sort_keys=True)
     spilling = sorted(name for name, use in report.items()
                       if use.get("vgpr_spills", 0) or use.get("scratch_bytes", 0))
-    print(f"{len(report)} kernels; spilling vector registers or using scratch: "
+    print(f"{len(report) - 1} kernels; spilling vector registers or using scratch: "
           f"{spilling if spilling else 'none'}", flush=True)
     return HIP_LIBRARY
 

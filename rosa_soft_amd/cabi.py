@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_vjp_workspace_bytes",
     "rosa_hip_set_record_budget",
     "rosa_hip_set_gradient_block_waves",
+    "rosa_hip_set_gradient_piece_rows",
     "rosa_hip_measure_atomic_rate",
     "rosa_hip_gradient_block_plan",
     "rosa_hip_hard_forward",
@@ -121,6 +122,8 @@ def load() -> ctypes.CDLL:
     ]
     library.rosa_hip_set_gradient_block_waves.restype = None
     library.rosa_hip_set_gradient_block_waves.argtypes = [ctypes.c_int]
+    library.rosa_hip_set_gradient_piece_rows.restype = None
+    library.rosa_hip_set_gradient_piece_rows.argtypes = [ctypes.c_int]
     library.rosa_hip_gradient_block_plan.restype = ctypes.c_int
     library.rosa_hip_gradient_block_plan.argtypes = [
         problem_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
@@ -576,6 +579,13 @@ def set_gradient_block_waves(waves: Optional[int]) -> None:
     """Waves per block of the gradient kernel: 1, 2, or ``None`` for the library's choice."""
 
     load().rosa_hip_set_gradient_block_waves(0 if waves is None else int(waves))
+
+
+def set_gradient_piece_rows(rows: Optional[int]) -> None:
+    """Rows of a piece of a band in the gradient kernel: a number, -1 for never, or ``None``
+    for the library's choice by shape."""
+
+    load().rosa_hip_set_gradient_piece_rows(0 if rows is None else int(rows))
 
 
 def gradient_block_plan(query: Tensor, value: Tensor, max_suffix_length: int,

@@ -37,13 +37,14 @@ from . import cabi
 __all__ = ["RosaRuntime"]
 
 
-def _integer_parameter(name: str, value: int) -> int:
-    if isinstance(value, bool):
+def _as_int(name: str, value: Any) -> int:
+    """A Python int from anything that indexes exactly (numpy and torch integer scalars
+    included); booleans and everything else are a TypeError naming the argument."""
+
+    indexes = not isinstance(value, bool) and hasattr(type(value), "__index__")
+    if not indexes:
         raise TypeError(f"{name} must be an integer")
-    try:
-        return operator.index(value)
-    except TypeError as error:
-        raise TypeError(f"{name} must be an integer") from error
+    return int(operator.index(value))
 
 
 def _pack_sign_bits(logits: Tensor, device: torch.device) -> Tensor:
@@ -60,7 +61,9 @@ def _pack_sign_bits(logits: Tensor, device: torch.device) -> Tensor:
         raise ValueError(f"RosaRuntime supports 1..8 bits, got {bits}")
     logits = logits.to(device)
     if logits.dtype not in (torch.float32, torch.float16, torch.bfloat16):
-        logits = logits.to(torch.float32)  # float64: the sign survives the narrowing
+        # wider than the kernel reads (float64): only the sign matters, and a narrowing cast
+        # would flush positives below the float32 range to zero, so hand over +-1 instead
+        logits = torch.where(logits > 0, 1.0, -1.0).to(torch.float32)
     return cabi.pack_symbols(logits, torch.uint8)
 
 
@@ -70,27 +73,31 @@ def _unpack_sign_bits(packed: Tensor, bits: int, dtype: torch.dtype) -> Tensor:
     return binary.mul(2).sub(1)
 
 
-def _normalize_sequence_ids(sequence_ids, slot_count: int) -> Optional[Tuple[int, ...]]:
+_ID_DTYPES = frozenset({torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64})
+
+
+def _slot_ids(sequence_ids, slot_count: int) -> Optional[Tuple[int, ...]]:
+    """The caller's slot labels as a tuple of distinct ints, one per slot, or None when no
+    labels were given (checks and messages of rosa_soft/runtime.py:149-176)."""
+
     if sequence_ids is None:
         return None
     if isinstance(sequence_ids, Tensor):
         if sequence_ids.ndim != 1:
             raise ValueError("sequence_ids must be a 1D tensor")
-        if sequence_ids.dtype not in (
-            torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64,
-        ):
+        if sequence_ids.dtype not in _ID_DTYPES:
             raise TypeError("sequence_ids must contain integers")
-        raw_ids = sequence_ids.detach().to(device="cpu").tolist()
+        items = sequence_ids.detach().cpu().tolist()
+    elif isinstance(sequence_ids, Sequence) and not isinstance(sequence_ids, (str, bytes)):
+        items = sequence_ids
     else:
-        if isinstance(sequence_ids, (str, bytes)) or not isinstance(sequence_ids, Sequence):
-            raise TypeError("sequence_ids must be an integer sequence")
-        raw_ids = list(sequence_ids)
-    normalized = tuple(_integer_parameter("sequence_ids", item) for item in raw_ids)
-    if len(normalized) != slot_count:
+        raise TypeError("sequence_ids must be an integer sequence")
+    ids = tuple(_as_int("sequence_ids", item) for item in items)
+    if len(ids) != slot_count:
         raise ValueError(f"sequence_ids must contain one ID per slot ({slot_count})")
-    if len(set(normalized)) != len(normalized):
+    if len(frozenset(ids)) < len(ids):
         raise ValueError("sequence_ids must be unique")
-    return normalized
+    return ids
 
 
 def _flatten_packed(query: Tensor, key: Tensor, payload: Tensor, cu_seqlens: Optional[Tensor]):
@@ -179,11 +186,11 @@ class RosaRuntime:
     ) -> None:
         if num_payload_heads is None:
             num_payload_heads = num_heads
-        self._num_heads = _integer_parameter("num_heads", num_heads)
-        self._num_payload_heads = _integer_parameter("num_payload_heads", num_payload_heads)
-        self._qk_bits = _integer_parameter("qk_bits", qk_bits)
-        self._payload_bits = _integer_parameter("payload_bits", payload_bits)
-        self._max_suffix_length = _integer_parameter("max_suffix_length", max_suffix_length)
+        self._num_heads = _as_int("num_heads", num_heads)
+        self._num_payload_heads = _as_int("num_payload_heads", num_payload_heads)
+        self._qk_bits = _as_int("qk_bits", qk_bits)
+        self._payload_bits = _as_int("payload_bits", payload_bits)
+        self._max_suffix_length = _as_int("max_suffix_length", max_suffix_length)
         for name, width in (("qk_bits", self._qk_bits), ("payload_bits", self._payload_bits)):
             if not 1 <= width <= 8:
                 raise ValueError(
@@ -377,7 +384,7 @@ class RosaRuntime:
         if payload.size(1) != self.num_payload_heads:
             raise ValueError("packed payload head count must equal num_payload_heads")
         slot_count = len(offsets) - 1
-        normalized_ids = _normalize_sequence_ids(sequence_ids, slot_count)
+        normalized_ids = _slot_ids(sequence_ids, slot_count)
         if stream is not None and caller_device.type != "cuda":
             raise ValueError("stream requires CUDA inputs")
         if stream is not None and stream.device != caller_device:

@@ -309,12 +309,19 @@ def test_no_kernel_of_the_last_build_spills_or_uses_scratch():
 
     from rosa_soft_amd import _build
 
-    if not os.path.exists(_build.RESOURCE_REPORT):
-        pytest.skip("no resource report: the library was not built by this tree's build step")
+    if not os.path.exists(_build.HIP_LIBRARY):
+        pytest.skip("the HIP library is not built")
     import json
 
+    # a library without the report of its own build (built by hand, or from another version
+    # of the source) would let register regressions through unseen: that is a failure
+    assert os.path.exists(_build.RESOURCE_REPORT), "library present but no resource report"
     with open(_build.RESOURCE_REPORT) as handle:
         report = json.load(handle)
+    built_from = report.pop(_build.BUILD_RECORD, {}).get("source_digest")
+    assert built_from == _build.source_digest(), (
+        "the resource report (and the library beside it) was built from another version of "
+        "the HIP source or other flags: rebuild")
     assert len(report) >= 100  # every instantiation of the backward kernels is listed
     offenders = {name: use for name, use in report.items()
                  if use.get("vgpr_spills", 0) or use.get("scratch_bytes", 0)}
@@ -329,7 +336,10 @@ def test_no_kernel_of_the_last_build_spills_or_uses_scratch():
     for name, use in report.items():
         registers = use["vgprs"] + use.get("agprs", 0)
         if "vjp_gradients_kernelILi1ELi8ELi1E" in name or "vjp_gradients_kernelILi1ELi16ELi1E" in name:
-            assert registers <= budget[3], (name, registers)
+            # (the form that walks pieces of bands, last template argument true, is compiled
+            # for two waves: it only runs when the bands are too few to fill three)
+            pieces = name.endswith("ELb1EEEvNS_9VjpParamsE")
+            assert registers <= budget[2 if pieces else 3], (name, registers)
         if "vjp_row_stats_kernel" in name:
             wide_with_dropout = "ILi2ELi64E" in name and name.split("ILi2ELi64E")[1].startswith(("Lb0ELb1E", "Lb1ELb1E"))
             assert registers <= budget[3 if wide_with_dropout else 4], (name, registers)

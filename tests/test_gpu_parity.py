@@ -590,6 +590,76 @@ def test_backward_without_chunk_records_recomputes_to_the_same_gradients(
         assert_gradients_close(got, expected.cpu())
 
 
+# --------------------------------------------------------------------------- pieces of bands
+
+PIECE_CASES = [
+    # B, T, H, D, Hv, Dv, W, p, dtype, pattern, piece_rows, mask, lengths
+    # a match of the whole sequence: every piece starts inside it, the halo (W - 1 rows,
+    # rounded up to chunks) is longer than the pieces
+    (1, 400, 1, 8, 1, 8, 128, 0.0, torch.float32, "all_match", 64, 7, None),
+    (1, 530, 2, 2, 2, 32, 256, 0.0, torch.float16, "all_match", 128, 7, None),
+    (1, 450, 2, 4, 1, 6, 40, 0.0, torch.float32, "shifted", 64, 7, None),
+    (1, 450, 2, 4, 1, 6, 40, 0.25, torch.float32, "shifted", 96, 7, None),
+    (1, 333, 2, 7, 1, 20, 9, 0.0, torch.float16, "periodic", 64, 7, None),
+    (1, 333, 1, 3, 1, 8, 600, 0.1, torch.float32, "periodic", 64, 7, None),
+    (2, 700, 3, 20, 3, 33, 64, 0.1, torch.bfloat16, "random", 192, 7, None),
+    # one gradient at a time: without symbol gradients the pieces take no halo
+    (1, 300, 2, 5, 1, 6, 33, 0.2, torch.float32, "shifted", 64, 4, None),
+    (1, 300, 2, 5, 1, 6, 33, 0.2, torch.float32, "shifted", 64, 1, None),
+    (1, 300, 2, 5, 1, 6, 33, 0.2, torch.float32, "shifted", 64, 2, None),
+    # packed sequences: pieces past the end of a short sequence's bands are empty work items
+    (1, 0, 2, 3, 2, 5, 16, 0.1, torch.float32, "random", 64, 7, [70, 0, 1, 300, 129]),
+    (1, 0, 2, 8, 1, 8, 150, 0.0, torch.float32, "all_match", 64, 7, [257, 64, 390]),
+]
+
+
+@pytest.mark.parametrize("records", [True, False], ids=["records", "no_records"])
+@pytest.mark.parametrize("B,T,H,D,Hv,Dv,W,p,dtype,pattern,piece_rows,mask,lengths", PIECE_CASES)
+def test_bands_cut_into_pieces_match_oracle(cabi, c_oracle, records, B, T, H, D, Hv, Dv, W, p,
+                                            dtype, pattern, piece_rows, mask, lengths):
+    """The gradient kernel cuts long bands into pieces when a shape has few of them; forced
+    here at test sizes.  A piece restarts the reverse recurrences W - 1 rows below its last
+    row and leaves its first 64 columns' partial sums to the piece above: long matches that
+    cross every cut are the cases that would show a wrong halo or a lost partial sum."""
+
+    seed = 31337 if p > 0 else None
+    if lengths is None:
+        query, key, value, grad_output = make_case(B, T, H, D, Hv, Dv, dtype, seed=T + W,
+                                                   pattern=pattern)
+        offsets = None
+    else:
+        total = sum(lengths)
+        query, key, value, grad_output = (
+            t[0] for t in make_case(1, total, H, D, Hv, Dv, dtype, seed=total, pattern=pattern))
+        offsets = [0] + [int(x) for x in np.cumsum(lengths)]
+    cabi.set_gradient_piece_rows(piece_rows)
+    cabi.set_record_budget(None if records else 0)
+    try:
+        _, _, _, _, grads = run_device(cabi, query, key, value, grad_output, W, 1.0, p, 3.0, seed,
+                                       mask, offsets)
+        cabi.set_gradient_piece_rows(-1)
+        _, _, _, _, whole = run_device(cabi, query, key, value, grad_output, W, 1.0, p, 3.0, seed,
+                                       mask, offsets)
+    finally:
+        cabi.set_gradient_piece_rows(None)
+        cabi.set_record_budget(None)
+    if lengths is None:
+        want = c_oracle.surrogate_vjp(query, key, value, grad_output, max_suffix_length=W,
+                                      dropout_p=p, seed=seed)
+    else:
+        want = c_oracle.varlen_surrogate_vjp(query, key, value, offsets, grad_output,
+                                             max_suffix_length=W, dropout_p=p, seed=seed)
+    longest_logit = 2.4142 * ((1.0 + min(W, max(T, max(lengths or [0])))) ** 0.5 - 1.0)
+    slack = max(1.0, longest_logit / 40.0)
+    for bit, name, got, unsplit, expected in zip((1, 2, 4), ("grad_query", "grad_key", "grad_value"),
+                                                 grads, whole, want):
+        if not mask & bit:
+            assert got is None
+            continue
+        assert_gradients_close(got, expected, name, slack)
+        assert_gradients_close(got, unsplit.cpu(), name + " against whole bands", slack)
+
+
 def test_atomic_rate_measurement_is_plausible_and_checks_its_arguments(cabi):
     """The measurement behind the gradient kernel's second bound: float atomics in the flush
     pattern (16 rows of a tile per step) run at some tens of G row segments per second on

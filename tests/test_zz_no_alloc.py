@@ -87,3 +87,41 @@ def test_sizes_beyond_the_static_scratch_are_rejected(cabi):
     problem = cabi.make_problem(query[:, :100], value[:, :100], 4)
     assert library.rosa_hip_hard_forward_static(
         ctypes.byref(problem), None, None, None, None, None, None, None, None) != 0
+
+
+def test_static_forward_records_into_a_hip_graph_after_a_first_call_outside(cabi):
+    """The callers this entry point exists for record it into a HIP graph.  Its first call on
+    a device looks up the address of the scratch array, which is not a stream operation and
+    must therefore happen before the recording; after that the call is launches only.  Every
+    replay is checked against eager work done between the replays, on inputs rewritten in
+    place, and neither torch's allocator nor the device's free memory moves."""
+
+    generator = torch.Generator(device=DEVICE).manual_seed(77)
+    q = torch.randn(2, 300, 4, 6, device=DEVICE, generator=generator)
+    k = torch.randn(2, 300, 4, 6, device=DEVICE, generator=generator)
+    v = torch.randn(2, 300, 2, 10, device=DEVICE, generator=generator)
+    want = cabi.hard_forward(q, k, v, 32)
+    outputs = tuple(torch.full_like(t, 77) for t in want)
+    cabi.hard_forward_static(q, k, v, 32, outputs=outputs)  # the first call: outside
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cabi.hard_forward_static(q, k, v, 32, outputs=outputs)
+    torch.cuda.synchronize()
+    free_bytes = torch.cuda.mem_get_info(DEVICE)[0]
+    for _ in range(3):
+        q.copy_(torch.randn(q.shape, device=DEVICE, generator=generator))
+        k.copy_(q.roll(1, dims=1))
+        want = cabi.hard_forward(q, k, v, 32)
+        for tensor in outputs:
+            tensor.fill_(77)
+        torch.cuda.synchronize()
+        allocated = torch.cuda.memory_allocated(DEVICE)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated(DEVICE) == allocated
+        for got, expected in zip(outputs, want):
+            assert torch.equal(got, expected)
+        assert int((outputs[3] > 0).sum()) > 0
+    # (torch's cache may have grown for the eager calls' workspaces; the replays take nothing)
+    assert torch.cuda.mem_get_info(DEVICE)[0] >= free_bytes - (64 << 20)
