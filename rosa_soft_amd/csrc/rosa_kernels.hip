@@ -1127,7 +1127,8 @@ VjpWorkspace carve_vjp(const ProblemView& v, bool dropout) {
   w.segment_group = 4;
   while (w.segment_group * w.segment_group < max_segments) ++w.segment_group;
   const int max_groups = max_segments > 0 ? (max_segments + w.segment_group - 1) / w.segment_group : 0;
-  w.block_scratch_floats = static_cast<int64_t>(w.ring_rows) * kWave +
+  // (the ring holds a float and a bfloat16 per row and lane)
+  w.block_scratch_floats = static_cast<int64_t>(w.ring_rows) * (kWave + kWave / 2) +
                            2 * kCheckpointChunksMax * kWave +
                            static_cast<int64_t>(max_segments > 0 ? max_groups + w.segment_group : 0) *
                                2 * kWave;

@@ -1237,7 +1237,11 @@ void vjp_gradients_kernel(VjpParams P) {
       (static_cast<int64_t>(blockIdx.x) * NW + wave) * P.block_scratch_floats;
   // without chunk records: (S, window) before every chunk of the current segment, then
   // before every segment of the band
-  float* ck_evidence = ring + static_cast<int64_t>(P.ring_rows) * kWave;   // [SEG_CHUNKS][64]
+  // (three-term form) what the float32 ring terms do not hold of (b + rest) * overflow, as
+  // bfloat16: the second float of the windowed sum
+  [[maybe_unused]] uint16_t* ring_low =
+      reinterpret_cast<uint16_t*>(ring + static_cast<int64_t>(P.ring_rows) * kWave);
+  float* ck_evidence = ring + static_cast<int64_t>(P.ring_rows) * (kWave + kWave / 2);  // [SEG_CHUNKS][64]
   int* ck_window = reinterpret_cast<int*>(ck_evidence + SEG_CHUNKS * kWave);
   // without records, two levels of (S, window) checkpoints: before every group of
   // `segment_group` segments of the band (one forward sweep over the band), and before every
@@ -1357,6 +1361,10 @@ void vjp_gradients_kernel(VjpParams P) {
     [[maybe_unused]] float carry_rest = 0.0f;
     float gate_below = 0.0f;      // gate of the row below
     float ring_sum = 0.0f;        // sum of b * overflow over the next W + 1 rows
+    // what ring_sum has lost and the sum of the terms' low parts (three-term form): h is the
+    // difference of b (S + o) and this sum, both hundreds of adjoints large along an exact
+    // match longer than the window, so both are carried as two floats
+    [[maybe_unused]] float ring_sum_low = 0.0f;
     int ring_live = 0;            // rows for which the ring still holds non-zero terms
     int ring_fresh = 0;           // ring reads that must be treated as zero
     const int last_step = my_steps - 1;
@@ -1916,6 +1924,11 @@ void vjp_gradients_kernel(VjpParams P) {
             gate_below = keep_gate[r];
             const float overflow = keep_overflow[r];
             const float term = overflow >= P.tail_threshold ? b * overflow : 0.0f;
+            [[maybe_unused]] float term_low = 0.0f;
+            if constexpr (TERMS == 3) {
+              term_low = overflow >= P.tail_threshold
+                  ? fmaf(carry_rest, overflow, fmaf(b, overflow, -term)) : 0.0f;
+            }
             const bool any_term = __ballot(term != 0.0f) != 0ull;
             if (any_term) {
               if (ring_live == 0) ring_fresh = P.ring_rows;
@@ -1924,19 +1937,39 @@ void vjp_gradients_kernel(VjpParams P) {
             if (ring_live > 0) {
               const int slot = i % P.ring_rows;
               float leaving = 0.0f;
+              [[maybe_unused]] float leaving_low = 0.0f;
               if (ring_fresh > 0) {
                 --ring_fresh;
               } else {
                 leaving = ring[slot * kWave + lane];
+                if constexpr (TERMS == 3) {
+                  leaving_low = __uint_as_float(uint32_t(ring_low[slot * kWave + lane]) << 16);
+                }
               }
               ring[slot * kWave + lane] = term;
-              ring_sum += term - leaving;
+              if constexpr (TERMS == 2) {
+                ring_sum += term - leaving;
+              } else {
+                // the low part enters the sum as it is stored, so that it leaves as it entered
+                const uint32_t low_bits = __float_as_uint(term_low) & 0xffff0000u;
+                ring_low[slot * kWave + lane] = static_cast<uint16_t>(low_bits >> 16);
+                const float added = __fadd_rn(ring_sum, term);
+                const float added_rest = __fsub_rn(term, __fsub_rn(added, ring_sum));
+                const float left = __fsub_rn(added, leaving);
+                const float left_rest = __fsub_rn(__fsub_rn(added, left), leaving);
+                ring_sum = left;
+                ring_sum_low += (__uint_as_float(low_bits) - leaving_low) + (added_rest + left_rest);
+              }
               --ring_live;
             }
             const float h = TERMS == 2
                 ? fmaf(b, keep_evidence[r], -ring_sum)
-                : fmaf(b, keep_evidence[r], fmaf(carry_rest, keep_evidence[r], -ring_sum));
-            if (ring_live == 0) ring_sum = 0.0f;
+                : fmaf(b, keep_evidence[r], -ring_sum) +
+                      fmaf(carry_rest, keep_evidence[r], -ring_sum_low);
+            if (ring_live == 0) {
+              ring_sum = 0.0f;
+              if constexpr (TERMS == 3) ring_sum_low = 0.0f;
+            }
             const bool active = steady || ((i + 1 - lane) >= 1 && r < rows_here);
             if constexpr (TERMS == 2) {
               tile_bits[r * (kTilePitch + 1) + 64 - lane] = split_bf16(active ? h : 0.0f);

@@ -140,14 +140,21 @@ SHORT = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 191, 200, 257, 320, 400]
 # a running float32 sum of hundreds of route adjoints of both signs.  The three-term form of
 # the gradient kernel (the one such inputs select) carries what those additions lose in a
 # second float.
+# With a window shorter than the match the gate adjoint is the difference of that sum
+# and its windowed sum: both are carried as two floats there.
 ONCE_OVER_THE_BAR = [
-    (38, 14),
+    (38, 14),   # window beyond the sequence: 320 rows, float16, dropout
+    (68, 7),    # 1024 rows, window 128, scale 2, dropout 0.5
+    (69, 14),   # 257 rows, window 33, scale 2
+    (77, 30),   # 320 rows, window 7, scale 2, float32
 ]
+LONG = [511, 777, 1024, 1500, 2049]
 
 
 @pytest.mark.parametrize("stream,index", ONCE_OVER_THE_BAR)
 def test_long_match_cases_that_once_exceeded_the_bar(cabi, c_oracle, stream, index):
-    c, run = case_at(stream, index, SHORT)
+    # (streams with a seed divisible by four drew their lengths from the long list)
+    c, run = case_at(stream, index, SHORT if stream % 4 else LONG)
     assert c["pattern"] == "periodic"
     try:
         cabi.set_gradient_block_waves(2 if (index + stream) % 2 else None)
