@@ -1807,8 +1807,12 @@ void vjp_gradients_kernel(VjpParams P) {
           }
         };
         const bool steady = first >= W + kWave && rows_here == kChunk;
+        // A quiet chunk takes no overflow term and tracks no window, so its unmasked form
+        // only needs every lane to have a pair in every row: from the band's row 64 on, not
+        // only once the windows are full.
+        const bool unmasked_quiet = chunk_quiet && first >= kWave && rows_here == kChunk;
         const bool cached = DROPOUT && stored;
-        if (steady && chunk_quiet) {
+        if (unmasked_quiet) {
           if (cached) replay(std::true_type{}, std::true_type{}, std::true_type{});
           else replay(std::true_type{}, std::false_type{}, std::true_type{});
         } else if (steady) {
@@ -1887,7 +1891,7 @@ void vjp_gradients_kernel(VjpParams P) {
         if (want_qk) {
           wave_lds_fence();
           // reverse walk of the chunk: gate adjoints replace the weights
-          const bool quiet = steady && chunk_quiet && ring_live == 0;
+          const bool quiet = unmasked_quiet && ring_live == 0;
           if (quiet) {
             // no overflow term of the chunk can move a gradient and the ring is empty:
             // h = b (S + o), nothing to mask

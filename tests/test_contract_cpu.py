@@ -255,8 +255,10 @@ def test_backward_workspace_sizes_at_training_shapes():
     cabi.set_record_budget(None)
     try:
         with_dropout, without_dropout = size(metric, True), size(metric, False)
-        assert 0.5 * pairs < with_dropout < 0.5 * pairs + 200 * 2 ** 20
-        assert 0.375 * pairs < without_dropout < 0.375 * pairs + 200 * 2 ** 20
+        # (beside the records: staged grad_output rows, value words, row statistics and, per
+        # resident wave of the gradient kernel, a ring of W + 1 rows of six bytes per lane)
+        assert 0.5 * pairs < with_dropout < 0.5 * pairs + 250 * 2 ** 20
+        assert 0.375 * pairs < without_dropout < 0.375 * pairs + 250 * 2 ** 20
         cabi.set_record_budget(0)
         assert size(metric, True) < 300 * 2 ** 20
         cabi.set_record_budget(None)
