@@ -77,7 +77,7 @@ def case_at(stream_seed, index, lengths):
     return c, draw_run(rng, c)
 
 
-def check_case(cabi, c_oracle, rng, index, c, run=None):
+def check_case(cabi, c_oracle, rng, index, c, run=None, widen=1.0):
     seed, parts = draw_run(rng, c) if run is None else run
     controls = dict(max_suffix_length=c["W"], scale=c["scale"], dropout_p=c["p"],
                     mismatch_scale=c["ms"], seed=seed)
@@ -109,7 +109,7 @@ def check_case(cabi, c_oracle, rng, index, c, run=None):
     # the same widening with the logit's magnitude L = scale * U(min(W, longest)) as in
     # test_surrogate_vjp_matches_oracle: none while scale * L <= 40
     longest_logit = c["scale"] * 2.4142 * ((1.0 + min(c["W"], max(longest, 1))) ** 0.5 - 1.0)
-    slack = max(1.0, c["scale"] * longest_logit / 40.0)
+    slack = widen * max(1.0, c["scale"] * longest_logit / 40.0)
     for bit, got, expected, name in zip((1, 2, 4), grads, want, "qkv"):
         if c["mask"] & bit:
             assert_gradients_close(got, expected, f"{label} d{name}", slack=slack)
@@ -159,5 +159,21 @@ def test_long_match_cases_that_once_exceeded_the_bar(cabi, c_oracle, stream, ind
     try:
         cabi.set_gradient_block_waves(2 if (index + stream) % 2 else None)
         check_case(cabi, c_oracle, None, index, c, run)
+    finally:
+        cabi.set_gradient_block_waves(None)
+
+
+def test_value_gradient_tail_case_of_the_two_term_weights(cabi, c_oracle):
+    """The one excess that 184 further stream seeds (about 17 000 cases) leave: 64 rows, window
+    1, dropout 0.5, value gradient only.  With a window of one every route of a row weighs the
+    same, the column sums of the value gradient cancel almost completely, and what is left of
+    the 2^-17 of the two-term route weights meets the 1e-5 max|want| floor of the bar: 1.23
+    times the bar on one element.  Pinned at 1.5 times the bar, so that it cannot grow."""
+
+    c, run = case_at(134, 105, SHORT)
+    assert c["W"] == 1 and c["mask"] == 4 and c["T"] == 64
+    try:
+        cabi.set_gradient_block_waves(2 if (105 + 134) % 2 else None)
+        check_case(cabi, c_oracle, None, 105, c, run, widen=1.5)
     finally:
         cabi.set_gradient_block_waves(None)
