@@ -334,9 +334,13 @@ def atomic_row_segments(config, plan: dict) -> int:
     value_segments = 0.5 if Dv <= 8 else sum(
         -(-4 * min(64, Dv - first) // 64) for first in range(0, Dv, 64))
     rows = columns = 0
+    piece_rows = plan.get("piece_rows", 0)
     for length in lengths:
         steps = [length - 1 - 64 * band for band in range((length + 63) // 64)]
         steps = [n for n in steps if n > 0]
+        if piece_rows > 0:
+            # every piece but the first of a band flushes four more column tiles (64 columns)
+            columns += sum(64 * ((n - 1) // piece_rows) for n in steps)
         if plan["waves"] == 2:
             leads = steps[0::2]
             columns += sum(leads)
@@ -365,6 +369,7 @@ def config_summary(measured: dict) -> dict:
             valu_fractions(measured).get("vjp_gradients", {}).get("frac", float("nan")), 4),
         whole_backward_frac=round(fractions.get("whole_backward", {}).get("frac", float("nan")), 4),
         waves_per_block=measured["gradient_block_plan"]["waves"],
+        band_pieces=measured["gradient_block_plan"].get("pieces", 1),
         atomic_row_segments=atomic_row_segments(config, measured["gradient_block_plan"]),
     )
 

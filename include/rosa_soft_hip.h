@@ -107,6 +107,14 @@ int rosa_hip_gradient_block_plan(const rosa_problem* problem, int* waves, int* r
                                  size_t* lds_bytes);
 
 /*
+ * Whether and how the gradient kernel will cut the diagonal bands of `problem` into pieces
+ * (no counterpart in the reference; see rosa_hip_set_gradient_piece_rows): `piece_rows` is
+ * the length of a piece in rows, 0 for whole bands, `pieces` the work items per band.  Host
+ * arithmetic only; returns 0 or a problem-check status.
+ */
+int rosa_hip_gradient_piece_plan(const rosa_problem* problem, int* piece_rows, int* pieces);
+
+/*
  * Measurement aid, no counterpart in the reference: the rate at which this GPU performs
  * global float atomic adds in the access pattern of the backward's gradient flush
  * (16 x 16 tiles at random rows of `buffer`, rows `row_floats` floats apart, `columns` <= 16

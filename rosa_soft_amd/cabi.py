@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_set_gradient_piece_rows",
     "rosa_hip_measure_atomic_rate",
     "rosa_hip_gradient_block_plan",
+    "rosa_hip_gradient_piece_plan",
     "rosa_hip_hard_forward",
     "rosa_hip_hard_routes",
     "rosa_hip_hard_forward_bits",
@@ -128,6 +129,10 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_gradient_block_plan.argtypes = [
         problem_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
         ctypes.POINTER(ctypes.c_size_t),
+    ]
+    library.rosa_hip_gradient_piece_plan.restype = ctypes.c_int
+    library.rosa_hip_gradient_piece_plan.argtypes = [
+        problem_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
     ]
     library.rosa_hip_measure_atomic_rate.restype = ctypes.c_int
     library.rosa_hip_measure_atomic_rate.argtypes = [
@@ -590,14 +595,20 @@ def set_gradient_piece_rows(rows: Optional[int]) -> None:
 
 def gradient_block_plan(query: Tensor, value: Tensor, max_suffix_length: int,
                         cu_seqlens: Optional[Tensor] = None) -> dict:
-    """Launch form of the gradient kernel for a problem: waves per block, row queue, LDS bytes."""
+    """Launch form of the gradient kernel for a problem: waves per block, row queue, LDS bytes,
+    and the rows of a piece of a band (0: whole bands) with the work items per band."""
 
     problem = make_problem(query, value, max_suffix_length, cu_seqlens)
     waves, queue, lds = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
     status = load().rosa_hip_gradient_block_plan(
         ctypes.byref(problem), ctypes.byref(waves), ctypes.byref(queue), ctypes.byref(lds))
     _check(status, "rosa_hip_gradient_block_plan")
-    return dict(waves=waves.value, row_queue=bool(queue.value), lds_bytes=lds.value)
+    piece_rows, pieces = ctypes.c_int(0), ctypes.c_int(1)
+    status = load().rosa_hip_gradient_piece_plan(
+        ctypes.byref(problem), ctypes.byref(piece_rows), ctypes.byref(pieces))
+    _check(status, "rosa_hip_gradient_piece_plan")
+    return dict(waves=waves.value, row_queue=bool(queue.value), lds_bytes=lds.value,
+                piece_rows=piece_rows.value, pieces=pieces.value)
 
 
 def measure_atomic_rate(row_floats: int, columns: int = 16, device: str = "cuda:0") -> float:

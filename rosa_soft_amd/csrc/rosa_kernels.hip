@@ -2186,6 +2186,27 @@ int rosa_hip_gradient_block_plan(const rosa_problem* problem, int* waves, int* r
   return 0;
 }
 
+int rosa_hip_gradient_piece_plan(const rosa_problem* problem, int* piece_rows, int* pieces) {
+  ProblemView view;
+  const int status = check_problem(problem, &view);
+  if (status != 0) return status;
+  const int slice_width = std::min(view.L.Dv, kValueSlice);
+  const int dvp = padded_value_width(slice_width);
+  const int symbol_tiles = view.L.D > 16 ? 2 : 1;
+  const int64_t units = static_cast<int64_t>(view.L.slots) * view.L.H;
+  const GradientBlockPlan blocks = plan_gradient_blocks(
+      dvp, view.L.D, value_words(slice_width), grad_term_pitch(view.grad_terms, dvp), units);
+  PiecePlan plan{0, 1};
+  if (blocks.waves == 1) {
+    plan = plan_band_pieces(units, view.L.varlen ? view.L.N : view.L.T, view.L.W,
+                            resident_gradient_waves((dvp + 15) / 16, symbol_tiles),
+                            gradient_segment(dvp));
+  }
+  if (piece_rows != nullptr) *piece_rows = plan.piece_rows;
+  if (pieces != nullptr) *pieces = plan.max_pieces;
+  return 0;
+}
+
 int rosa_hip_measure_atomic_rate(void* buffer, size_t buffer_bytes, int row_floats, int columns,
                                  double* segments_per_second, void* stream) {
   if (buffer == nullptr || segments_per_second == nullptr) return fail(1, "NULL argument");

@@ -282,6 +282,24 @@ def test_gradient_launch_plan_follows_the_shape():
 
     metric = plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128)
     assert metric["waves"] == 1 and not metric["row_queue"]
+    # 8 192 bands on 3 072 resident waves: whole bands
+    assert metric["piece_rows"] == 0 and metric["pieces"] == 1
+    # configuration 4: 2 048 bands of up to 8 191 rows on 2 048 resident waves are cut into two
+    # pieces of whole 32-row segments, each at least four windows long
+    long_bands = plan(torch.float16, (1, 8192, 16), 2, 16, 32, 256)
+    assert long_bands["waves"] == 1 and long_bands["pieces"] == 2
+    assert long_bands["piece_rows"] == 4096 and long_bands["piece_rows"] >= 4 * 256
+    try:
+        cabi.set_gradient_piece_rows(-1)
+        assert plan(torch.float16, (1, 8192, 16), 2, 16, 32, 256)["pieces"] == 1
+        cabi.set_gradient_piece_rows(100)  # rounded up to whole segments
+        forced = plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128)
+        assert forced["piece_rows"] == 128 and forced["pieces"] == 32
+        cabi.set_gradient_block_waves(2)   # two-wave blocks walk whole bands
+        assert plan(torch.float32, (2, 4096, 64), 8, 16, 8, 128)["pieces"] == 1
+    finally:
+        cabi.set_gradient_piece_rows(None)
+        cabi.set_gradient_block_waves(None)
     config3 = plan(torch.bfloat16, (4, 4096, 32), 16, 32, 64, 32)
     assert config3["waves"] == 2 and config3["row_queue"]
     assert config3["lds_bytes"] <= 40 * 1024
