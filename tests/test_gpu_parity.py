@@ -603,6 +603,10 @@ PIECE_CASES = [
     (1, 333, 2, 7, 1, 20, 9, 0.0, torch.float16, "periodic", 64, 7, None),
     (1, 333, 1, 3, 1, 8, 600, 0.1, torch.float32, "periodic", 64, 7, None),
     (2, 700, 3, 20, 3, 33, 64, 0.1, torch.bfloat16, "random", 192, 7, None),
+    # value width above 64: two slices, each a run of both passes with its own pieces
+    (1, 260, 2, 9, 1, 70, 24, 0.2, torch.float32, "shifted", 64, 7, None),
+    # window beyond the sequence: the halo of every piece reaches the band's end
+    (1, 200, 1, 8, 1, 8, 1000, 0.0, torch.float32, "periodic", 64, 7, None),
     # one gradient at a time: without symbol gradients the pieces take no halo
     (1, 300, 2, 5, 1, 6, 33, 0.2, torch.float32, "shifted", 64, 4, None),
     (1, 300, 2, 5, 1, 6, 33, 0.2, torch.float32, "shifted", 64, 1, None),
