@@ -150,3 +150,52 @@ def test_packed_config5_full_size(cabi, c_oracle):
         value[start:end, 2:3].unsqueeze(0), config["W"],
     )
     assert torch.equal(routes[17:18, start:end].cpu(), want_routes[0])
+
+
+def test_one_long_sequence_three_ways(cabi):
+    """One sequence of 32 768 tokens (four heads): few, long bands, the shape for which the
+    gradient kernel cuts bands into pieces.  No oracle finishes this size; the three ways the
+    kernel can get its state must agree with each other instead: chunk records with pieces
+    (the default here), chunk records with whole bands, and no records at all (forward sweeps
+    from two levels of checkpoints).  Accumulation order differs, so the comparison is to the
+    bar of the parity tests, widened by two for two device results."""
+
+    T, H, D, Hv, Dv, W = 32768, 4, 8, 2, 8, 64
+    generator = torch.Generator(device=DEVICE).manual_seed(2024)
+    query = torch.randn(1, T, H, D, device=DEVICE, generator=generator)
+    key = torch.randn(1, T, H, D, device=DEVICE, generator=generator)
+    key[:, 5000:5400] = query[:, 4000:4400]  # a long exact match in the middle
+    value = torch.randn(1, T, Hv, Dv, device=DEVICE, generator=generator)
+    grad_output = torch.randn(1, T, H, Dv, device=DEVICE, generator=generator)
+    seed = torch.tensor(77, dtype=torch.int64, device=DEVICE)
+    out, packed_q, packed_k, routes = cabi.hard_forward(query, key, value, W)
+    plan = cabi.gradient_block_plan(query, value, W)
+    assert plan["pieces"] > 1
+
+    def backward():
+        grads = cabi.surrogate_vjp(query, key, value, grad_output, packed_q, packed_k, seed, W,
+                                   1.0, 0.1, 3.0, 7)
+        torch.cuda.synchronize()
+        return grads
+
+    try:
+        pieces = backward()
+        cabi.set_gradient_piece_rows(-1)
+        whole = backward()
+        cabi.set_gradient_piece_rows(None)
+        cabi.set_record_budget(0)
+        swept = backward()
+    finally:
+        cabi.set_gradient_piece_rows(None)
+        cabi.set_record_budget(None)
+    assert int((routes > 0).sum()) > T  # matches were found
+    for name, a, b, c in zip(("grad_query", "grad_key", "grad_value"), pieces, whole, swept):
+        assert torch.isfinite(a).all() and float(a.abs().max()) > 0, name
+        for other, label in ((b, "whole bands"), (c, "no records")):
+            tolerance = 2e-4 * a.abs() + 2e-5 * a.abs().max()
+            excess = float(((a - other).abs() - tolerance).max())
+            assert excess <= 0.0, f"{name} against {label}: exceeds tolerance by {excess:.3e}"
+    # structural zeros: first query row, last key row, first value row
+    assert torch.count_nonzero(pieces[0][:, 0]) == 0
+    assert torch.count_nonzero(pieces[1][:, -1]) == 0
+    assert torch.count_nonzero(pieces[2][:, 0]) == 0
