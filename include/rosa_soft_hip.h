@@ -197,11 +197,12 @@ int rosa_hip_hard_forward_words(const rosa_problem* problem, const int32_t* pack
  *   y = routed ? (sign bit ? +1 : -1) : 0,
  * i.e. `residual + self.output(routed.flatten(2))` of examples/fit_soft_reference.py:415-416
  * without the ternary tensor in between: the matrix products (bfloat16 inputs, float32
- * accumulation) expand their A operand from `sign_words` / `routed` in registers.
+ * accumulation) expand the operand that holds y from `sign_words` / `routed` in registers.
  * `weight` is the [N][H * Dv] matrix of the linear layer, `residual` (optional) and `out`
  * are [tokens][N]; all three bfloat16.  Dv must be 8, 16 or a multiple of 32, H * Dv a
  * multiple of 32 and N a multiple of 64 (other shapes expand the bits and use a library
- * product).  The reference has no such kernel.
+ * product).  `weight` and `sign_words` must be 16-byte aligned, `out` and `residual`
+ * 8-byte, `routed` 4-byte (error 1 otherwise).  The reference has no such kernel.
  */
 int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* routed,
                                  int64_t tokens, int H, int Dv, const void* weight, int N,

@@ -1670,17 +1670,22 @@ __global__ __launch_bounds__(256) void router_advance_kernel(RouterUpdate U) {
 //   y[t, k] = routed[t, h] ? (bit d of sign_words[t, h] ? +1 : -1) : 0
 //
 // i.e. `residual + output(routed.flatten(2))` of the reference's caller
-// (examples/fit_soft_reference.py:374-417) without the ternary tensor in between: the A
-// operand of the matrix products is expanded from the bits in registers.  `weight` is the
+// (examples/fit_soft_reference.py:374-417) without the ternary tensor in between: the
+// operand of the matrix products that holds y is expanded from the bits in registers (the
+// weights are the products' row operand, so that a lane ends up with four neighbouring
+// output columns of one token).  `weight` is the
 // [N][K] matrix of a linear layer (k contiguous), bfloat16; accumulation is float32.
 // A block of four waves computes 256 rows x 64 columns, each wave 64 x 64 (sixteen
-// 16 x 16 x 32 products per 32-wide k step).  Per step a block stages the weight tile
-// [64][32] and, per row, the 32 sign bits and 32 validity bits of the step in LDS; the loads
-// of the next step are in flight while the products of this one run.
+// 16 x 16 x 32 products per 32-wide k step).  Per staged step of 64 k (two products deep) a
+// block stages the weight tile [64][64] and, per row, the sign and validity bits of the step
+// in LDS; the loads of the next step are in flight while the products of this one run.
 constexpr int kProjectRows = 256;
 constexpr int kProjectColumns = 64;
-constexpr int kProjectStep = 32;
-constexpr int kProjectWeightPitch = kProjectStep + 8;  // bfloat16 elements per staged weight row
+constexpr int kProjectStep = 32;    // k of one matrix product, and what K must be a multiple of
+// k staged per barrier (128 needs registers beyond three waves per SIMD, and is slower for it)
+constexpr int kProjectStage = 64;
+constexpr int kStageProducts = kProjectStage / kProjectStep;
+constexpr int kProjectWeightPitch = kProjectStage + 8;  // bfloat16 elements per staged weight row
 
 struct ProjectParams {
   const uint32_t* sign_words;  // [tokens][H][nvw]
@@ -1707,33 +1712,40 @@ __device__ __forceinline__ void fill_ternary_table(uint32_t* table, int index) {
   }
 }
 
-// sign bits and validity bits of k = 32 step .. 32 step + 31 of one token
+// Sign bits and validity bits of k = 32 step .. 32 step + 31 of one token.  HEADS: heads per
+// step (4: value width 8, 2: width 16), or 0 where a head spans whole steps (a width that is
+// a multiple of 32: step `step` is then word `step` of the token's words).
+template <int HEADS>
 __device__ __forceinline__ uint2 ternary_step_bits(const ProjectParams& P, int64_t token, int step) {
-  const int k0 = step * kProjectStep;
   uint32_t signs = 0u, valid = 0u;
   if (token < P.tokens) {
-    if (P.Dv >= 32) {  // the step lies inside one head
-      const int head = k0 / P.Dv;
-      const int word = (k0 - head * P.Dv) >> 5;
-      signs = P.sign_words[(token * P.H + head) * P.nvw + word];
-      valid = P.routed[token * P.H + head] == 1 ? 0xffffffffu : 0u;
-    } else {           // 32 / Dv heads, one word each
-      const int heads = 32 / P.Dv;
-      const int head0 = k0 / P.Dv;
-      const uint32_t field = (1u << P.Dv) - 1u;
-      for (int j = 0; j < heads; ++j) {
-        const uint32_t word = P.sign_words[token * P.H + head0 + j] & field;
-        signs |= word << (j * P.Dv);
-        if (P.routed[token * P.H + head0 + j] == 1) valid |= field << (j * P.Dv);
-      }
+    if constexpr (HEADS == 0) {
+      signs = P.sign_words[token * P.H * P.nvw + step];
+      valid = P.routed[token * P.H + step / P.nvw] == 1 ? 0xffffffffu : 0u;
+    } else if constexpr (HEADS == 2) {
+      const int64_t first = token * P.H + 2 * step;
+      const uint2 words = *reinterpret_cast<const uint2*>(P.sign_words + first);
+      const uint32_t flags = *reinterpret_cast<const uint16_t*>(P.routed + first);
+      signs = (words.x & 0xffffu) | (words.y << 16);
+      valid = ((flags & 0xffu) == 1u ? 0xffffu : 0u) | ((flags >> 8) == 1u ? 0xffff0000u : 0u);
+    } else {
+      static_assert(HEADS == 4, "a step holds four, two or a part of one head");
+      const int64_t first = token * P.H + 4 * step;
+      const uint4 words = *reinterpret_cast<const uint4*>(P.sign_words + first);
+      const uint32_t flags = *reinterpret_cast<const uint32_t*>(P.routed + first);
+      signs = (words.x & 0xffu) | ((words.y & 0xffu) << 8) | ((words.z & 0xffu) << 16) | (words.w << 24);
+      valid = ((flags & 0xffu) == 1u ? 0xffu : 0u) | (((flags >> 8) & 0xffu) == 1u ? 0xff00u : 0u) |
+              (((flags >> 16) & 0xffu) == 1u ? 0xff0000u : 0u) | ((flags >> 24) == 1u ? 0xff000000u : 0u);
     }
   }
   return make_uint2(signs, valid);
 }
 
+template <int HEADS>
 __global__ __launch_bounds__(256) void project_routed_bits_kernel(ProjectParams P) {
   __shared__ __attribute__((aligned(16))) uint16_t weight_tile[2][kProjectColumns * kProjectWeightPitch];
-  __shared__ __attribute__((aligned(8))) uint2 row_bits[2][kProjectRows];
+  // (signs, valid) of every product of the stage, per row
+  __shared__ __attribute__((aligned(16))) uint2 row_bits[2][kProjectRows][kStageProducts];
   __shared__ __attribute__((aligned(8))) uint32_t ternary_table[kTernaryTableWords];
   const int thread = threadIdx.x;
   const int lane = thread & 63;
@@ -1752,56 +1764,87 @@ __global__ __launch_bounds__(256) void project_routed_bits_kernel(ProjectParams 
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   }
-  const int steps = P.K / kProjectStep;
-  // what a thread stages per step: 16 bytes of the weight tile and one row's bits
+  const int products = P.K / kProjectStep;           // 32-wide k steps in all
+  const int stages = (products + kStageProducts - 1) / kStageProducts;
+  // what a thread stages per stage: a quarter of one weight row's stage and one row's bits
+  constexpr int kThreadElements = kProjectStage / 4;
+  constexpr int kThreadChunks = kThreadElements / 8;   // of 16 bytes
   const int stage_n = thread >> 2;
-  const int stage_k = (thread & 3) * 8;
+  const int stage_k = (thread & 3) * kThreadElements;
   const uint16_t* weight_row = P.weight + static_cast<int64_t>(n0 + stage_n) * P.K + stage_k;
-  uint4 weight_in = *reinterpret_cast<const uint4*>(weight_row);
-  uint2 bits_in = ternary_step_bits(P, row0 + thread, 0);
-  for (int step = 0; step < steps; ++step) {
-    const int buffer = step & 1;
-    *reinterpret_cast<uint4*>(&weight_tile[buffer][stage_n * kProjectWeightPitch + stage_k]) = weight_in;
-    row_bits[buffer][thread] = bits_in;
+  uint4 weight_in[kThreadChunks];
+  uint2 bits_in[kStageProducts];
+  const auto fetch_stage = [&](int stage) {
+    // (K is a multiple of 32: the last stage may hold fewer products than the others)
+#pragma unroll
+    for (int chunk = 0; chunk < kThreadChunks; ++chunk) {
+      const int k = stage * kProjectStage + stage_k + 8 * chunk;
+      weight_in[chunk] = k + 8 <= P.K
+                             ? *reinterpret_cast<const uint4*>(weight_row + stage * kProjectStage + 8 * chunk)
+                             : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int h = 0; h < kStageProducts; ++h) {
+      const int step = stage * kStageProducts + h;
+      bits_in[h] = step < products ? ternary_step_bits<HEADS>(P, row0 + thread, step) : make_uint2(0u, 0u);
+    }
+  };
+  fetch_stage(0);
+  for (int stage = 0; stage < stages; ++stage) {
+    const int buffer = stage & 1;
+    uint16_t* staged = &weight_tile[buffer][stage_n * kProjectWeightPitch + stage_k];
+#pragma unroll
+    for (int chunk = 0; chunk < kThreadChunks; ++chunk)
+      *reinterpret_cast<uint4*>(staged + 8 * chunk) = weight_in[chunk];
+#pragma unroll
+    for (int h = 0; h < kStageProducts; ++h) row_bits[buffer][thread][h] = bits_in[h];
     __syncthreads();
-    if (step + 1 < steps) {  // the next step's loads are in flight during the products
-      weight_in = *reinterpret_cast<const uint4*>(weight_row + (step + 1) * kProjectStep);
-      bits_in = ternary_step_bits(P, row0 + thread, step + 1);
-    }
-    v4u b_operand[4];
+    if (stage + 1 < stages) fetch_stage(stage + 1);  // in flight during the products
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      b_operand[j] = *reinterpret_cast<const v4u*>(
-          &weight_tile[buffer][(16 * j + li) * kProjectWeightPitch + 8 * lg]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint2 bits = row_bits[buffer][wave * 64 + 16 * i + li];
-      const uint32_t byte = (bits.x >> (8 * lg)) & 0xffu;
-      const uint32_t valid = (bits.y >> (8 * lg)) & 1u;  // a head is valid as a whole
-      const uint2 low = *reinterpret_cast<const uint2*>(
-          ternary_table + 2 * ((valid << 4) | (byte & 15u)));
-      const uint2 high = *reinterpret_cast<const uint2*>(
-          ternary_table + 2 * ((valid << 4) | (byte >> 4)));
-      const v4u a_operand = {low.x, low.y, high.x, high.y};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(a_operand, b_operand[j], acc[i][j]);
-    }
-  }
-  // lane (li, lg) holds rows 4 lg .. 4 lg + 3 of column li of every 16 x 16 tile
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int64_t token = row0 + wave * 64 + 16 * i + 4 * lg + e;
-      if (token >= P.tokens) continue;
+    for (int h = 0; h < kStageProducts; ++h) {
+      v4u b_operand[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int64_t index = token * P.N + n0 + 16 * j + li;
-        float value = acc[i][j][e];
-        if (P.residual != nullptr) value += __uint_as_float(static_cast<uint32_t>(P.residual[index]) << 16);
-        P.out[index] = static_cast<uint16_t>(bf16_nearest(value));
+        b_operand[j] = *reinterpret_cast<const v4u*>(
+            &weight_tile[buffer][(16 * j + li) * kProjectWeightPitch + kProjectStep * h + 8 * lg]);
       }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint2 bits = row_bits[buffer][wave * 64 + 16 * i + li][h];
+        const uint32_t byte = (bits.x >> (8 * lg)) & 0xffu;
+        const uint32_t valid = (bits.y >> (8 * lg)) & 1u;  // a head is valid as a whole
+        const uint2 low = *reinterpret_cast<const uint2*>(
+            ternary_table + 2 * ((valid << 4) | (byte & 15u)));
+        const uint2 high = *reinterpret_cast<const uint2*>(
+            ternary_table + 2 * ((valid << 4) | (byte >> 4)));
+        const v4u a_operand = {low.x, low.y, high.x, high.y};
+        // (the weights as the row operand: a lane then holds four neighbouring output
+        // columns of one token, which leave as one 8-byte store)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(b_operand[j], a_operand, acc[i][j]);
+      }
+    }
+  }
+  // lane (li, lg) holds columns 4 lg .. 4 lg + 3 of every 16-column tile for token li of
+  // every 16-token tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t token = row0 + wave * 64 + 16 * i + li;
+    if (token >= P.tokens) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t index = token * P.N + n0 + 16 * j + 4 * lg;
+      v4f value = acc[i][j];
+      if (P.residual != nullptr) {
+        const uint2 added = *reinterpret_cast<const uint2*>(P.residual + index);
+        value[0] += __uint_as_float(added.x << 16);
+        value[1] += __uint_as_float(added.x & 0xffff0000u);
+        value[2] += __uint_as_float(added.y << 16);
+        value[3] += __uint_as_float(added.y & 0xffff0000u);
+      }
+      *reinterpret_cast<uint2*>(P.out + index) =
+          make_uint2(bf16_nearest(value[0]) | (bf16_nearest(value[1]) << 16),
+                     bf16_nearest(value[2]) | (bf16_nearest(value[3]) << 16));
     }
   }
 }
@@ -1962,9 +2005,24 @@ int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* rout
   P.out = static_cast<uint16_t*>(out);
   P.tokens = tokens;
   P.H = H; P.Dv = Dv; P.nvw = value_words(Dv); P.N = N; P.K = static_cast<int>(K);
-  hipLaunchKernelGGL(project_routed_bits_kernel,
-                     dim3(static_cast<unsigned>(row_blocks), static_cast<unsigned>(N / kProjectColumns)),
-                     dim3(256), 0, static_cast<hipStream_t>(stream), P);
+  // the kernel moves 16 bytes of a weight row or of four heads' words, and 8 bytes of an
+  // output row, per access
+  const auto misaligned = [](const void* pointer, uintptr_t bytes) {
+    return (reinterpret_cast<uintptr_t>(pointer) & (bytes - 1)) != 0;
+  };
+  if (misaligned(weight, 16) || misaligned(sign_words, 16) || misaligned(routed, 4) ||
+      misaligned(out, 8) || misaligned(residual, 8))
+    return fail(1, "project_routed_bits: weight and sign_words must be 16-byte aligned, out and "
+                   "residual 8-byte, routed 4-byte");
+  const dim3 grid(static_cast<unsigned>(row_blocks), static_cast<unsigned>(N / kProjectColumns));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (Dv == 8) {
+    hipLaunchKernelGGL(project_routed_bits_kernel<4>, grid, dim3(256), 0, s, P);
+  } else if (Dv == 16) {
+    hipLaunchKernelGGL(project_routed_bits_kernel<2>, grid, dim3(256), 0, s, P);
+  } else {
+    hipLaunchKernelGGL(project_routed_bits_kernel<0>, grid, dim3(256), 0, s, P);
+  }
   const hipError_t launch = hipGetLastError();
   if (launch != hipSuccess) return fail_hip(launch, "project_routed_bits launch");
   return 0;

@@ -108,3 +108,14 @@ def test_projection_refuses_shapes_it_does_not_tile(cabi):
     weight = torch.zeros(48, 3 * 32, dtype=torch.bfloat16, device=device)
     with pytest.raises(RuntimeError, match="multiple of 64"):
         cabi.project_routed_bits(words, routed, 32, weight)
+
+
+def test_projection_refuses_pointers_it_cannot_load_in_whole_vectors(cabi):
+    device = torch.device("cuda:0")
+    routed = torch.ones(8, 4, dtype=torch.uint8, device=device)
+    words = torch.zeros(8, 4, 1, dtype=torch.int32, device=device)
+    # a contiguous matrix that starts 2 bytes into its allocation
+    weight = torch.zeros(64 * 32 + 1, dtype=torch.bfloat16, device=device)[1:].view(64, 32)
+    assert weight.is_contiguous() and weight.data_ptr() % 16 != 0
+    with pytest.raises(RuntimeError, match="aligned"):
+        cabi.project_routed_bits(words, routed, 8, weight)
