@@ -215,16 +215,15 @@ def measure_workload(name: str, steps: int, warmup: int) -> dict:
     for _ in range(warmup):
         run_step(rosa_soft_amd, config, leaves, cu_seqlens)
     torch.cuda.synchronize()
-    stage_totals = {}
+    cabi.stage_totals()  # the warm-up's events: read and dropped
     begin = time.perf_counter()
     for _ in range(steps):
         run_step(rosa_soft_amd, config, leaves, cu_seqlens)
-        # the events of this step were recorded on the stream; reading them
-        # waits for the step, which the closing synchronize would do anyway
-        for stage, ms in cabi.stage_times().items():
-            stage_totals[stage] = stage_totals.get(stage, 0.0) + ms
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - begin
+    # the library recorded its stage events on the launch stream during the timed steps and
+    # the host waited for none of them; they are read only now
+    stage_means = {stage: total / runs for stage, (total, runs) in cabi.stage_totals().items()}
     cabi.stage_timing(False)
 
     def forward():
@@ -246,7 +245,7 @@ def measure_workload(name: str, steps: int, warmup: int) -> dict:
     return dict(
         name=name, config=config, steps=steps, warmup=warmup,
         ms_per_step=1e3 * elapsed / steps, forward_ms=forward_ms,
-        stage_ms={stage: total / steps for stage, total in stage_totals.items()},
+        stage_ms=stage_means,
         gradient_block_plan=plan,
     )
 

@@ -310,9 +310,13 @@ int rosa_hip_read_offset_error(const void* workspace, void* stream);
  * Stage timing for measurement (no counterpart in the reference, whose
  * benchmark times whole calls with CUDA events, benchmarks/rosa_soft.py:159-173).
  * While enabled, every call above brackets its stages with HIP events recorded
- * on the caller's stream; rosa_hip_stage_times() waits for those events and
- * returns the elapsed milliseconds of the LAST call per stage (-1 for a stage
- * that did not run).  Stages: 0 hard_forward (pack + route + gather),
+ * on the caller's stream, and the host waits for nothing; rosa_hip_stage_times()
+ * waits for those events and returns the elapsed milliseconds of the LAST call
+ * per stage (-1 for a stage that did not run).  rosa_hip_stage_totals() is for a
+ * loop of calls timed as a whole: per stage it returns the summed milliseconds of
+ * the runs since timing was enabled or the totals were last read (of the last 64
+ * of them, if there were more) and how many runs that sum covers (0: none), and
+ * starts a new sum.  Stages: 0 hard_forward (pack + route + gather),
  * 1 vjp_prepare, 2 vjp_row_max, 3 vjp_row_stats, 4 vjp_gradients,
  * 5 vjp_finalize.  Not thread safe; meant for benchmarks.
  */
@@ -320,6 +324,7 @@ int rosa_hip_stage_timing(int enable);
 int rosa_hip_stage_count(void);
 const char* rosa_hip_stage_name(int stage);
 int rosa_hip_stage_times(float* milliseconds, int count);
+int rosa_hip_stage_totals(float* milliseconds, int* runs, int count);
 
 #ifdef __cplusplus
 }

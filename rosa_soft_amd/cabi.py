@@ -47,6 +47,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_stage_count",
     "rosa_hip_stage_name",
     "rosa_hip_stage_times",
+    "rosa_hip_stage_totals",
 )
 
 _DTYPE_CODES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
@@ -183,6 +184,10 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_stage_name.argtypes = [ctypes.c_int]
     library.rosa_hip_stage_times.restype = ctypes.c_int
     library.rosa_hip_stage_times.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_int]
+    library.rosa_hip_stage_totals.restype = ctypes.c_int
+    library.rosa_hip_stage_totals.argtypes = [
+        ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int), ctypes.c_int,
+    ]
     _library = library
     return library
 
@@ -641,4 +646,21 @@ def stage_times() -> dict:
         library.rosa_hip_stage_name(i).decode(): float(buffer[i])
         for i in range(count)
         if buffer[i] >= 0.0
+    }
+
+
+def stage_totals() -> dict:
+    """``{stage: (summed milliseconds, runs)}`` of the calls since timing was enabled or the
+    totals were last read (waits for their events, then starts a new sum).  At most the last
+    64 runs of a stage are summed; ``runs`` says how many were."""
+
+    library = load()
+    count = library.rosa_hip_stage_count()
+    buffer = (ctypes.c_float * count)()
+    runs = (ctypes.c_int * count)()
+    _check(library.rosa_hip_stage_totals(buffer, runs, count), "rosa_hip_stage_totals")
+    return {
+        library.rosa_hip_stage_name(i).decode(): (float(buffer[i]), int(runs[i]))
+        for i in range(count)
+        if runs[i] > 0
     }

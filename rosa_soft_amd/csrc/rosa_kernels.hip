@@ -47,29 +47,32 @@ int fail_hip(hipError_t status, const char* what) {
 
 // Optional stage timing: when enabled, every launch sequence brackets its
 // stages with HIP events recorded on the caller's stream.  Nothing is read
-// back until rosa_hip_stage_times() is called.
+// back, and the host waits for nothing, until rosa_hip_stage_times() or
+// rosa_hip_stage_totals() is called.  Every stage keeps the events of its last
+// kStageRing runs, so that a loop of calls can be timed without a wait per call.
 enum Stage { kStageForward = 0, kStagePrepare, kStageRowMax, kStageRowStats, kStageGradients,
              kStageFinalize, kStageCount };
+constexpr int kStageRing = 64;
 
 struct StageTimer {
   bool enabled = false;
   bool created = false;
-  hipEvent_t begin[kStageCount];
-  hipEvent_t end[kStageCount];
-  bool used[kStageCount];
+  hipEvent_t begin[kStageCount][kStageRing];
+  hipEvent_t end[kStageCount][kStageRing];
+  int64_t runs[kStageCount];   // since timing was enabled or the totals were last read
 };
 
 StageTimer g_timer;
 
 void stage_begin(Stage stage, hipStream_t stream) {
   if (!g_timer.enabled) return;
-  g_timer.used[stage] = true;
-  (void)hipEventRecord(g_timer.begin[stage], stream);
+  (void)hipEventRecord(g_timer.begin[stage][g_timer.runs[stage] % kStageRing], stream);
 }
 
 void stage_end(Stage stage, hipStream_t stream) {
   if (!g_timer.enabled) return;
-  (void)hipEventRecord(g_timer.end[stage], stream);
+  (void)hipEventRecord(g_timer.end[stage][g_timer.runs[stage] % kStageRing], stream);
+  g_timer.runs[stage] += 1;
 }
 
 // ---------------------------------------------------------------------------
@@ -2195,12 +2198,15 @@ void rosa_hip_set_record_budget(size_t bytes) {
 int rosa_hip_stage_timing(int enable) {
   if (enable && !g_timer.created) {
     for (int i = 0; i < kStageCount; ++i) {
-      if (hipEventCreate(&g_timer.begin[i]) != hipSuccess) return fail(5, "hipEventCreate failed");
-      if (hipEventCreate(&g_timer.end[i]) != hipSuccess) return fail(5, "hipEventCreate failed");
+      for (int slot = 0; slot < kStageRing; ++slot) {
+        if (hipEventCreate(&g_timer.begin[i][slot]) != hipSuccess ||
+            hipEventCreate(&g_timer.end[i][slot]) != hipSuccess)
+          return fail(5, "hipEventCreate failed");
+      }
     }
     g_timer.created = true;
   }
-  for (int i = 0; i < kStageCount; ++i) g_timer.used[i] = false;
+  for (int i = 0; i < kStageCount; ++i) g_timer.runs[i] = 0;
   g_timer.enabled = enable != 0;
   return 0;
 }
@@ -2217,12 +2223,34 @@ int rosa_hip_stage_times(float* milliseconds, int count) {
   if (!g_timer.created) return fail(5, "stage timing was never enabled");
   for (int i = 0; i < count && i < kStageCount; ++i) {
     milliseconds[i] = -1.0f;
-    if (!g_timer.used[i]) continue;
-    if (hipEventSynchronize(g_timer.end[i]) != hipSuccess) return fail(5, "event sync failed");
+    if (g_timer.runs[i] == 0) continue;
+    const int slot = static_cast<int>((g_timer.runs[i] - 1) % kStageRing);
+    if (hipEventSynchronize(g_timer.end[i][slot]) != hipSuccess) return fail(5, "event sync failed");
     float ms = 0.0f;
-    if (hipEventElapsedTime(&ms, g_timer.begin[i], g_timer.end[i]) != hipSuccess)
+    if (hipEventElapsedTime(&ms, g_timer.begin[i][slot], g_timer.end[i][slot]) != hipSuccess)
       return fail(5, "event elapsed failed");
     milliseconds[i] = ms;
+  }
+  return 0;
+}
+
+int rosa_hip_stage_totals(float* milliseconds, int* runs, int count) {
+  if (!g_timer.created) return fail(5, "stage timing was never enabled");
+  if (!milliseconds || !runs) return fail(2, "stage_totals: NULL pointer");
+  for (int i = 0; i < count && i < kStageCount; ++i) {
+    const int kept = static_cast<int>(std::min<int64_t>(g_timer.runs[i], kStageRing));
+    double total = 0.0;
+    for (int back = 1; back <= kept; ++back) {
+      const int slot = static_cast<int>((g_timer.runs[i] - back) % kStageRing);
+      if (hipEventSynchronize(g_timer.end[i][slot]) != hipSuccess) return fail(5, "event sync failed");
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, g_timer.begin[i][slot], g_timer.end[i][slot]) != hipSuccess)
+        return fail(5, "event elapsed failed");
+      total += ms;
+    }
+    milliseconds[i] = static_cast<float>(total);
+    runs[i] = kept;
+    g_timer.runs[i] = 0;
   }
   return 0;
 }

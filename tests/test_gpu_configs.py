@@ -199,3 +199,29 @@ def test_one_long_sequence_three_ways(cabi):
     assert torch.count_nonzero(pieces[0][:, 0]) == 0
     assert torch.count_nonzero(pieces[1][:, -1]) == 0
     assert torch.count_nonzero(pieces[2][:, 0]) == 0
+
+
+def test_stage_totals_cover_a_loop_of_calls_without_a_wait_per_call(cabi):
+    device = torch.device("cuda:0")
+    generator = torch.Generator(device=device).manual_seed(9)
+    query = torch.randn(1, 256, 4, 8, device=device, generator=generator)
+    key = torch.randn(1, 256, 4, 8, device=device, generator=generator)
+    value = torch.randn(1, 256, 2, 8, device=device, generator=generator)
+    cabi.stage_timing(True)
+    try:
+        for _ in range(3):
+            cabi.hard_forward(query, key, value, 16)
+        totals = cabi.stage_totals()
+        assert set(totals) == {"hard_forward"}
+        milliseconds, runs = totals["hard_forward"]
+        assert runs == 3 and milliseconds > 0.0
+        last = cabi.stage_times()
+        assert last == {}  # reading the totals started a new sum
+        for _ in range(70):  # more runs than the library keeps events for
+            cabi.hard_forward(query, key, value, 16)
+        assert cabi.stage_times()["hard_forward"] > 0.0
+        milliseconds, runs = cabi.stage_totals()["hard_forward"]
+        assert runs == 64 and milliseconds > 0.0
+        assert cabi.stage_totals() == {}
+    finally:
+        cabi.stage_timing(False)
