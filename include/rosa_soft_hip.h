@@ -98,6 +98,20 @@ void rosa_hip_set_gradient_block_waves(int waves);
 void rosa_hip_set_gradient_piece_rows(int rows);
 
 /*
+ * How the hard forward finds its routes: 0 (the default) = through an index of the keys by
+ * symbol where the shape has one (symbols of six bits or more, sequences of 512 tokens or
+ * more; a row then visits only the routes whose key symbol equals its own, and row blocks
+ * that this does not suit are handed back to the scan over all routes), 1 = always the scan
+ * over all routes, 2 = the index with every row block handed back, 3 = the index at every
+ * shape (2 and 3 are for tests).  The routes are the same in every mode.  The workspace
+ * size does not depend on the mode.  No
+ * counterpart in the reference (its forward kernel steps over every route,
+ * rosa_soft_kernels.cu:367-531); the knob exists for measurements and tests, with the
+ * thread rule of the other setters.
+ */
+void rosa_hip_set_forward_index(int mode);
+
+/*
  * How the backward's gradient kernel will be launched for `problem` (no counterpart in the
  * reference): waves per block (1 or 2), whether row tiles are queued between the two bands
  * of a block, and the dynamic LDS of a block in bytes.  Any of the three may be NULL.

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_set_record_budget",
     "rosa_hip_set_gradient_block_waves",
     "rosa_hip_set_gradient_piece_rows",
+    "rosa_hip_set_forward_index",
     "rosa_hip_measure_atomic_rate",
     "rosa_hip_gradient_block_plan",
     "rosa_hip_gradient_piece_plan",
@@ -126,6 +127,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_set_gradient_block_waves.argtypes = [ctypes.c_int]
     library.rosa_hip_set_gradient_piece_rows.restype = None
     library.rosa_hip_set_gradient_piece_rows.argtypes = [ctypes.c_int]
+    library.rosa_hip_set_forward_index.restype = None
+    library.rosa_hip_set_forward_index.argtypes = [ctypes.c_int]
     library.rosa_hip_gradient_block_plan.restype = ctypes.c_int
     library.rosa_hip_gradient_block_plan.argtypes = [
         problem_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
@@ -596,6 +599,16 @@ def set_gradient_piece_rows(rows: Optional[int]) -> None:
     for the library's choice by shape."""
 
     load().rosa_hip_set_gradient_piece_rows(0 if rows is None else int(rows))
+
+
+def set_forward_index(mode: Optional[str]) -> None:
+    """How the hard forward finds its routes: ``None`` (the library's choice: an index of the
+    keys where the shape suits it), ``"scan"`` (always the scan over all routes),
+    ``"handed_back"`` (the index with every row block handed back to the scan) or ``"always"``
+    (the index at every shape); the last two are for tests."""
+
+    modes = {None: 0, "scan": 1, "handed_back": 2, "always": 3}
+    load().rosa_hip_set_forward_index(modes[mode])
 
 
 def gradient_block_plan(query: Tensor, value: Tensor, max_suffix_length: int,

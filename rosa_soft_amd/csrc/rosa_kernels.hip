@@ -403,11 +403,15 @@ __device__ __forceinline__ RouteWinner scan_routes_narrow(const Symbol* q, const
   return RouteWinner{W - static_cast<int>(best >> shift), static_cast<int>(low - (best & low))};
 }
 
+// `left_over` (or NULL): one byte per block of the grid; the kernel then routes only the
+// row blocks whose byte is set, those that route_candidates_kernel has left to it.
 template <bool VARLEN, bool WIDE>
 __global__ __launch_bounds__(kWave) void hard_route_kernel(
     Layout L, const uint32_t* __restrict__ packed_query,
     const uint32_t* __restrict__ packed_key, int32_t* __restrict__ routes,
-    int32_t* __restrict__ lengths, int32_t* __restrict__ source_token, int shift) {
+    int32_t* __restrict__ lengths, int32_t* __restrict__ source_token, int shift,
+    const uint8_t* __restrict__ left_over) {
+  if (left_over != nullptr && left_over[blockIdx.x] == 0) return;
   const Unit u = decode_unit<VARLEN>(L, blockIdx.x);
   if (!u.valid) return;
   const int blocks = (u.len + 63) >> 6;
@@ -426,6 +430,192 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
   const int route = winner.run > 0 ? winner.route : 0;
   if (routes != nullptr) routes[u.word_base + t] = route;
   if (lengths != nullptr) lengths[u.word_base + t] = winner.run;
+  source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
+}
+
+// ---------------------------------------------------------------------------
+// hard forward from an index of the keys
+// ---------------------------------------------------------------------------
+//
+// A route a of row t has a run of at least one iff k[a - 1] == q[t], and its run is then the
+// number of equal symbols walking back from there.  With symbols of many bits few routes of
+// a row qualify (T / 2^bits of them on random symbols), so instead of stepping over every
+// route a row can visit just those: index_keys_kernel sorts the key positions of every
+// (sequence, head) into buckets by symbol (counting sort in LDS; an entry carries the route,
+// its key symbol and the key symbol before it), and route_candidates_kernel lets every row
+// walk its own bucket.  The winner is the same "longest first, latest on ties" maximum, so
+// the routes are those of hard_route_kernel bit for bit.  Inputs this does not suit are
+// handed back to the scan: a (sequence, head) whose largest bucket is far above the mean
+// (few distinct symbols), and a row block whose walk exceeds its budget of iterations (long
+// matches everywhere, as on periodic inputs); hard_route_kernel then runs for those blocks
+// only.
+constexpr int kIndexThreads = 256;
+constexpr int kIndexBucketsMax = 4096;
+
+__device__ __forceinline__ uint32_t key_bucket(uint32_t symbol, int log_buckets, int hashed) {
+  return hashed ? (symbol * 0x9e3779b1u) >> (32 - log_buckets) : symbol & ((1u << log_buckets) - 1u);
+}
+
+struct KeyIndex {
+  int32_t* bucket_begin;  // [units][buckets + 1]
+  uint4* entries;         // [symbol rows]: (route, key symbol, key symbol before it, 0), by bucket
+  uint8_t* unit_scan;     // [units]: 1 = this (sequence, head) is left to the scan
+  uint8_t* left_over;     // [blocks of the route grid]: 1 = this row block is left to the scan
+  int log_buckets;
+  int hashed;             // symbols of more bits than log_buckets: buckets by a multiplicative hash
+  // what a row block may spend before it is handed back: budget_base + rows above it / 8
+  // bucket entries per lane, and a quarter of that in steps of walking back along runs (two
+  // dependent loads each; on random symbols a row block walks a handful of steps in all)
+  int budget_base;
+};
+
+template <bool VARLEN>
+__global__ __launch_bounds__(kIndexThreads) void index_keys_kernel(
+    Layout L, const uint32_t* __restrict__ packed_key, KeyIndex index) {
+  __shared__ int cursor[kIndexBucketsMax];
+  __shared__ int partial[kIndexThreads];
+  __shared__ int largest;
+  const int unit = blockIdx.x;
+  const int head = unit % L.H;
+  const int seq = unit / L.H;
+  int len;
+  int64_t word_base;
+  if constexpr (VARLEN) {
+    len = L.seq_len[seq];
+    word_base = static_cast<int64_t>(head) * L.N + L.seq_start[seq];
+  } else {
+    len = L.T;
+    word_base = (static_cast<int64_t>(seq) * L.H + head) * L.T;
+  }
+  const int buckets = 1 << index.log_buckets;
+  const int count = max(len - 1, 0);  // key positions 0 .. len - 2 carry routes 1 .. len - 1
+  const uint32_t* k = packed_key + word_base;
+  const int thread = threadIdx.x;
+  for (int b = thread; b < buckets; b += kIndexThreads) cursor[b] = 0;
+  if (thread == 0) largest = 0;
+  __syncthreads();
+  for (int p = thread; p < count; p += kIndexThreads)
+    atomicAdd(&cursor[key_bucket(k[p], index.log_buckets, index.hashed)], 1);
+  __syncthreads();
+  // exclusive prefix sums: a thread owns `per` neighbouring buckets
+  const int per = max(buckets / kIndexThreads, 1);
+  const int first = thread * per;
+  int mine = 0, biggest = 0;
+  if (first < buckets) {
+    for (int b = first; b < first + per; ++b) {
+      mine += cursor[b];
+      biggest = max(biggest, cursor[b]);
+    }
+  }
+  partial[thread] = mine;
+  atomicMax(&largest, biggest);
+  __syncthreads();
+  for (int step = 1; step < kIndexThreads; step <<= 1) {
+    const int below = thread >= step ? partial[thread - step] : 0;
+    __syncthreads();
+    partial[thread] += below;
+    __syncthreads();
+  }
+  int32_t* begin = index.bucket_begin + static_cast<int64_t>(unit) * (buckets + 1);
+  if (first < buckets) {
+    int running = partial[thread] - mine;
+    for (int b = first; b < first + per; ++b) {
+      const int size = cursor[b];
+      cursor[b] = running;
+      begin[b] = running;
+      running += size;
+    }
+  }
+  if (thread == 0) {
+    begin[buckets] = count;
+    // a bucket far above the mean: few distinct symbols, the scan is the better walk
+    index.unit_scan[unit] = largest > max(64, count / 16) ? 1 : 0;
+  }
+  __syncthreads();
+  uint4* entries = index.entries + word_base;
+  for (int p = thread; p < count; p += kIndexThreads) {
+    const uint32_t symbol = k[p];
+    const int slot = atomicAdd(&cursor[key_bucket(symbol, index.log_buckets, index.hashed)], 1);
+    entries[slot] = make_uint4(static_cast<uint32_t>(p + 1), symbol, p >= 1 ? k[p - 1] : 0u, 0u);
+  }
+}
+
+template <bool VARLEN>
+__global__ __launch_bounds__(kWave) void route_candidates_kernel(
+    Layout L, const uint32_t* __restrict__ packed_query,
+    const uint32_t* __restrict__ packed_key, int32_t* __restrict__ routes,
+    int32_t* __restrict__ lengths, int32_t* __restrict__ source_token, KeyIndex index) {
+  const Unit u = decode_unit<VARLEN>(L, blockIdx.x);
+  const int lane = threadIdx.x;
+  if (!u.valid) {
+    if (lane == 0) index.left_over[blockIdx.x] = 0;
+    return;
+  }
+  const int blocks = (u.len + 63) >> 6;
+  if (u.block >= blocks) {
+    if (lane == 0) index.left_over[blockIdx.x] = 0;
+    return;
+  }
+  const int unit = u.seq * L.H + u.head;
+  if (index.unit_scan[unit] != 0) {
+    if (lane == 0) index.left_over[blockIdx.x] = 1;
+    return;
+  }
+  const int row_block = blocks - 1 - u.block;  // as in hard_route_kernel
+  const int t0 = row_block * kWave;
+  const uint32_t* q = packed_query + u.word_base;
+  const uint32_t* k = packed_key + u.word_base;
+  const int t = t0 + lane;
+  const bool row_ok = t < u.len;
+  const uint32_t q_symbol = row_ok ? q[t] : 0u;
+  const uint32_t q_before = (row_ok && t >= 1) ? q[t - 1] : 0u;
+  const int buckets = 1 << index.log_buckets;
+  const int32_t* begin = index.bucket_begin + static_cast<int64_t>(unit) * (buckets + 1);
+  const uint32_t bucket = key_bucket(q_symbol, index.log_buckets, index.hashed);
+  int next = row_ok ? begin[bucket] : 0;
+  const int end = row_ok ? begin[bucket + 1] : 0;
+  const uint4* entries = index.entries + u.word_base;
+  const int budget = index.budget_base + t0 / 8;
+  const int walk_budget = budget / 4;
+  int spent = 0, walked = 0;  // wave-uniform
+  uint64_t best = 0;  // (run << 32) | route
+  uint4 ahead = next < end ? entries[next] : make_uint4(0u, 0u, 0u, 0u);
+  while (__builtin_amdgcn_ballot_w64(next < end) != 0ull) {
+    const bool have = next < end;
+    const uint4 entry = ahead;
+    ++next;
+    if (next < end) ahead = entries[next];
+    const int a = static_cast<int>(entry.x);
+    const bool candidate = have && a <= t && entry.y == q_symbol;
+    const int limit = min(L.W, a);
+    int run = candidate ? 1 : 0;
+    bool walking = candidate && limit >= 2 && entry.z == q_before;
+    if (walking) run = 2;
+    walking = walking && run < limit;
+    while (walked <= walk_budget && __builtin_amdgcn_ballot_w64(walking) != 0ull) {
+      ++walked;
+      if (walking) {
+        if (q[t - run] == k[a - 1 - run]) {
+          ++run;
+          walking = run < limit;
+        } else {
+          walking = false;
+        }
+      }
+    }
+    const uint64_t found = (static_cast<uint64_t>(run) << 32) | static_cast<uint32_t>(a);
+    if (candidate) best = max(best, found);
+    if (++spent > budget || walked > walk_budget) {
+      if (lane == 0) index.left_over[blockIdx.x] = 1;
+      return;
+    }
+  }
+  if (lane == 0) index.left_over[blockIdx.x] = 0;
+  if (!row_ok) return;
+  const int run = static_cast<int>(best >> 32);
+  const int route = run > 0 ? static_cast<int>(best & 0xffffffffu) : 0;
+  if (routes != nullptr) routes[u.word_base + t] = route;
+  if (lengths != nullptr) lengths[u.word_base + t] = run;
   source_token[u.word_base + t] = route > 0 ? u.start + route : -1;
 }
 
@@ -1017,9 +1207,19 @@ int check_problem(const rosa_problem* p, ProblemView* out) {
 // Workspace carving shared by the size queries and the launches.
 struct ForwardWorkspace {
   size_t header, seq_start, seq_len, block_prefix, source_token, total;
+  // the index of the keys (route_candidates_kernel); log_buckets == 0: no room for it
+  int log_buckets, hashed;
+  size_t bucket_begin, entries, unit_scan, left_over;
 };
 
-ForwardWorkspace carve_forward(const ProblemView& v) {
+// Shapes the index of the keys is used for unless the caller says otherwise: symbols of six
+// bits or more (below that most routes of a row match and the scan is the better walk) and
+// sequences long enough for the two extra launches to pay.  The workspace has room for it
+// at every shape, so that the choice can be made per launch.
+constexpr int kIndexSymbolBitsMin = 6;
+constexpr int kIndexLongestMin = 512;
+
+ForwardWorkspace carve_forward(const ProblemView& v, bool with_index = true) {
   ForwardWorkspace w;
   size_t cursor = 0;
   w.header = cursor; cursor += align_up(256);
@@ -1028,9 +1228,33 @@ ForwardWorkspace carve_forward(const ProblemView& v) {
   w.seq_len = cursor; cursor += align_up(sizeof(int32_t) * s);
   w.block_prefix = cursor; cursor += align_up(sizeof(int32_t) * (s + 1));
   w.source_token = cursor; cursor += align_up(sizeof(int32_t) * static_cast<size_t>(v.symbol_rows));
+  w.log_buckets = 0; w.hashed = 0;
+  w.bucket_begin = w.entries = w.unit_scan = w.left_over = 0;
+  const int longest = v.L.varlen ? v.L.N : v.L.T;
+  if (with_index) {
+    // about four keys per bucket on the longest sequence, at most one bucket per symbol
+    int log_buckets = 6;
+    while (log_buckets < 12 && (4 << log_buckets) < longest) ++log_buckets;
+    const size_t units = static_cast<size_t>(v.L.varlen ? v.L.S : v.L.B) * v.L.H;
+    // (many short packed sequences: the bucket tables stay below four bytes per token and head)
+    while (log_buckets > 1 && (units << log_buckets) > static_cast<size_t>(v.symbol_rows)) --log_buckets;
+    w.hashed = v.L.D > log_buckets ? 1 : 0;
+    w.log_buckets = std::min(log_buckets, v.L.D);
+    const size_t blocks = static_cast<size_t>(v.L.slots) * v.L.H;
+    w.bucket_begin = cursor;
+    cursor += align_up(sizeof(int32_t) * units * ((size_t(1) << w.log_buckets) + 1));
+    w.entries = cursor; cursor += align_up(sizeof(uint4) * static_cast<size_t>(v.symbol_rows));
+    w.unit_scan = cursor; cursor += align_up(units);
+    w.left_over = cursor; cursor += align_up(blocks);
+  }
   w.total = cursor;
   return w;
 }
+
+// rosa_hip_set_forward_index: 0 = the index at the shapes above, 1 = never, 2 = the index
+// with no budget at all (every row block is handed back to the scan), 3 = the index at
+// every shape (2 and 3 are for tests)
+std::atomic<int> g_forward_index_mode{0};
 
 constexpr int kValueSlice = 64;  // value dimensions one backward pass covers
 constexpr int kNarrowRow = 8;    // gradient rows up to this many floats are accumulated head-major
@@ -1184,9 +1408,9 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
                 const void* key, const void* value, void* output, int32_t* packed_query,
                 int32_t* packed_key, int32_t* routes, int32_t* lengths, void* workspace,
                 hipStream_t stream, uint32_t* sign_words = nullptr, uint8_t* routed = nullptr,
-                bool words_given = false) {
+                bool words_given = false, bool allow_index = true) {
   Layout L = view.L;
-  const ForwardWorkspace w = carve_forward(view);
+  const ForwardWorkspace w = carve_forward(view, allow_index);
   stage_begin(kStageForward, stream);
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
                            stream);
@@ -1210,21 +1434,47 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   int32_t* source_token = at<int32_t>(workspace, w.source_token);
   const uint32_t* pq = reinterpret_cast<const uint32_t*>(packed_query);
   const uint32_t* pk = reinterpret_cast<const uint32_t*>(packed_key);
+  const int index_mode = g_forward_index_mode.load(std::memory_order_relaxed);
+  const uint8_t* left_over = nullptr;
+  const bool index_suits = L.D >= kIndexSymbolBitsMin && longest >= kIndexLongestMin;
+  if (w.log_buckets > 0 && (index_mode >= 2 || (index_mode == 0 && index_suits))) {
+    KeyIndex index;
+    index.bucket_begin = at<int32_t>(workspace, w.bucket_begin);
+    index.entries = at<uint4>(workspace, w.entries);
+    index.unit_scan = at<uint8_t>(workspace, w.unit_scan);
+    index.left_over = at<uint8_t>(workspace, w.left_over);
+    index.log_buckets = w.log_buckets;
+    index.hashed = w.hashed;
+    index.budget_base = index_mode == 2 ? -(1 << 30) : 64;
+    const unsigned sequences = static_cast<unsigned>(L.varlen ? L.S : L.B) * static_cast<unsigned>(L.H);
+    if (L.varlen) {
+      hipLaunchKernelGGL(index_keys_kernel<true>, dim3(sequences), dim3(kIndexThreads), 0, stream,
+                         L, pk, index);
+      hipLaunchKernelGGL(route_candidates_kernel<true>, dim3(units), dim3(kWave), 0, stream, L, pq,
+                         pk, routes, lengths, source_token, index);
+    } else {
+      hipLaunchKernelGGL(index_keys_kernel<false>, dim3(sequences), dim3(kIndexThreads), 0, stream,
+                         L, pk, index);
+      hipLaunchKernelGGL(route_candidates_kernel<false>, dim3(units), dim3(kWave), 0, stream, L,
+                         pq, pk, routes, lengths, source_token, index);
+    }
+    left_over = index.left_over;
+  }
   if (L.varlen) {
     if (wide) {
       hipLaunchKernelGGL((hard_route_kernel<true, true>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, lengths, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift, left_over);
     } else {
       hipLaunchKernelGGL((hard_route_kernel<true, false>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, lengths, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift, left_over);
     }
   } else {
     if (wide) {
       hipLaunchKernelGGL((hard_route_kernel<false, true>), dim3(units), dim3(kWave), 0, stream, L,
-                         pq, pk, routes, lengths, source_token, shift);
+                         pq, pk, routes, lengths, source_token, shift, left_over);
     } else {
       hipLaunchKernelGGL((hard_route_kernel<false, false>), dim3(units), dim3(kWave), 0, stream,
-                         L, pq, pk, routes, lengths, source_token, shift);
+                         L, pq, pk, routes, lengths, source_token, shift, left_over);
     }
   }
   const int32_t* offset_error = L.varlen ? at<const int32_t>(workspace, w.header) : nullptr;
@@ -1855,27 +2105,29 @@ __global__ __launch_bounds__(256) void project_routed_bits_kernel(ProjectParams 
 int forward_entry(const rosa_problem* problem, const void* query, const void* key,
                   const void* value, void* output, int32_t* packed_query, int32_t* packed_key,
                   int32_t* routes, int32_t* lengths, void* workspace, size_t workspace_bytes,
-                  void* stream, uint32_t* sign_words, uint8_t* routed, bool words_given = false) {
+                  void* stream, uint32_t* sign_words, uint8_t* routed, bool words_given = false,
+                  bool allow_index = true) {
   ProblemView view;
   const int bad = check_problem(problem, &view);
   if (bad != 0) return bad;
   if ((!words_given && (!query || !key)) || !value || !packed_query || !packed_key || !workspace)
     return fail(2, "hard_forward: NULL tensor or workspace pointer");
-  if (workspace_bytes < carve_forward(view).total) return fail(3, "hard_forward: workspace too small");
+  if (workspace_bytes < carve_forward(view, allow_index).total)
+    return fail(3, "hard_forward: workspace too small");
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (problem->dtype) {
     case ROSA_DTYPE_F32:
       return run_forward<ROSA_DTYPE_F32>(problem, view, query, key, value, output, packed_query,
                                          packed_key, routes, lengths, workspace, s, sign_words,
-                                         routed, words_given);
+                                         routed, words_given, allow_index);
     case ROSA_DTYPE_F16:
       return run_forward<ROSA_DTYPE_F16>(problem, view, query, key, value, output, packed_query,
                                          packed_key, routes, lengths, workspace, s, sign_words,
-                                         routed, words_given);
+                                         routed, words_given, allow_index);
     default:
       return run_forward<ROSA_DTYPE_BF16>(problem, view, query, key, value, output, packed_query,
                                           packed_key, routes, lengths, workspace, s, sign_words,
-                                          routed, words_given);
+                                          routed, words_given, allow_index);
   }
 }
 
@@ -2038,7 +2290,9 @@ int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query,
   ProblemView view;
   const int bad = check_problem(problem, &view);
   if (bad != 0) return bad;
-  if (carve_forward(view).total > kStaticScratchBytes) {
+  // the index of the keys (16 more bytes per token and head) is used where it fits as well
+  const bool with_index = carve_forward(view, true).total <= kStaticScratchBytes;
+  if (carve_forward(view, with_index).total > kStaticScratchBytes) {
     return fail(3, "hard_forward_static: the problem needs more than the 16 MiB of static "
                    "scratch (4 bytes per token and head); use rosa_hip_hard_forward");
   }
@@ -2046,7 +2300,8 @@ int rosa_hip_hard_forward_static(const rosa_problem* problem, const void* query,
   const int status = static_scratch_address(&address);
   if (status != 0) return status;
   return forward_entry(problem, query, key, value, output, packed_query, packed_key, routes,
-                       nullptr, address, kStaticScratchBytes, stream, nullptr, nullptr);
+                       nullptr, address, kStaticScratchBytes, stream, nullptr, nullptr, false,
+                       with_index);
 }
 
 int rosa_hip_pack_symbols(int dtype, const void* logits, int64_t rows, int bits, void* symbols,
@@ -2190,6 +2445,8 @@ void rosa_hip_set_gradient_block_waves(int waves) {
 }
 
 void rosa_hip_set_gradient_piece_rows(int rows) { g_gradient_piece_rows = rows < -1 ? 0 : rows; }
+
+void rosa_hip_set_forward_index(int mode) { g_forward_index_mode = (mode >= 1 && mode <= 3) ? mode : 0; }
 
 void rosa_hip_set_record_budget(size_t bytes) {
   g_record_budget_bytes = bytes;  // (size_t)-1: the default

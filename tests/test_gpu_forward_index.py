@@ -1,0 +1,121 @@
+"""The hard forward through the index of the keys (route_candidates_kernel) gives the routes of
+the scan over all routes (hard_route_kernel), which are those of the reference's forward kernel
+(rosa_soft_kernels.cu:367-531: longest matched suffix, latest route on ties, null route for a
+zero run), bit for bit: at shapes below the sizes the library picks the index for by itself,
+with every row block handed back to the scan, on inputs whose row blocks exceed their budget,
+and with symbols wide enough to be bucketed by a hash."""
+
+import pytest
+import torch
+
+from tests.conftest import nonzero_randn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from rosa_soft_amd import cabi as module
+
+    module.load()
+    yield module
+    module.set_forward_index(None)
+
+
+def _pattern_inputs(pattern, batch, length, heads, bits, seed):
+    query = nonzero_randn((batch, length, heads, bits), dtype=torch.float32, seed=seed)
+    key = nonzero_randn((batch, length, heads, bits), dtype=torch.float32, seed=seed + 1)
+    if pattern == "random":
+        return query, key
+    if pattern == "constant":
+        return torch.ones_like(query), torch.ones_like(key)
+    if pattern.startswith("period"):
+        period = int(pattern[len("period"):])
+        motif = nonzero_randn((batch, period, heads, bits), dtype=torch.float32, seed=seed + 2)
+        key = motif.repeat(1, length // period + 1, 1, 1)[:, :length].contiguous()
+        return key.clone(), key
+    assert pattern == "echo"
+    # the second half of the keys repeats the first, and the queries follow the keys one
+    # step behind: long runs, with an earlier and a later route of the same length
+    half = length // 2
+    key[:, half:2 * half] = key[:, :half]
+    query[:, 1:] = key[:, :-1]
+    generator = torch.Generator().manual_seed(seed + 3)
+    noise = torch.rand(batch, length, heads, 1, generator=generator) < 0.02
+    return torch.where(noise, -query, query).contiguous(), key.contiguous()
+
+
+DENSE_CASES = [
+    # batch, length, heads, bits, value heads, value width, window, pattern
+    (2, 700, 4, 8, 2, 8, 16, "random"),
+    (1, 1500, 3, 6, 3, 4, 1, "random"),
+    (1, 2100, 2, 12, 1, 8, 2100, "random"),
+    (2, 513, 2, 32, 2, 16, 7, "random"),       # buckets by hash
+    (1, 900, 2, 20, 1, 8, 40, "echo"),         # buckets by hash, long runs
+    (3, 65, 2, 7, 1, 8, 4, "random"),
+    (1, 1, 1, 8, 1, 8, 3, "random"),
+    (1, 2, 1, 8, 1, 8, 3, "random"),
+    (2, 300, 2, 1, 2, 8, 9, "random"),         # two symbols
+    (2, 300, 2, 3, 1, 8, 300, "random"),
+    (1, 1200, 2, 8, 2, 8, 500, "period5"),     # every row block exceeds its budget
+    (1, 1200, 2, 8, 1, 8, 64, "period300"),    # small buckets, long runs
+    (2, 640, 2, 9, 2, 8, 640, "constant"),     # one bucket
+    (1, 2048, 4, 8, 2, 8, 128, "echo"),
+    (1, 4096, 2, 10, 1, 8, 33, "echo"),
+]
+
+
+@pytest.mark.parametrize("case", DENSE_CASES, ids=lambda c: "-".join(str(x) for x in c))
+def test_indexed_forward_equals_the_scan_and_the_oracle(cabi, c_oracle, case):
+    batch, length, heads, bits, value_heads, width, window, pattern = case
+    device = torch.device("cuda:0")
+    query, key = _pattern_inputs(pattern, batch, length, heads, bits, seed=17 * length + bits)
+    value = nonzero_randn((batch, length, value_heads, width), dtype=torch.float32, seed=5)
+    want_output, want_routes, _ = c_oracle.hard_forward(query, key, value, window)
+    q, k, v = query.to(device), key.to(device), value.to(device)
+    for mode in ("scan", "always", "handed_back", None):
+        cabi.set_forward_index(mode)
+        output, _, _, routes = cabi.hard_forward(q, k, v, window)
+        assert torch.equal(routes.cpu(), want_routes), mode
+        assert torch.equal(output.cpu(), want_output), mode
+    cabi.set_forward_index(None)
+
+
+@pytest.mark.parametrize("bits,window", [(8, 16), (6, 1), (24, 700), (2, 5)])
+def test_indexed_forward_of_packed_sequences_equals_the_scan(cabi, bits, window):
+    device = torch.device("cuda:0")
+    lengths = [700, 1, 0, 513, 64, 2, 65, 1100, 0, 129]
+    total = sum(lengths)
+    offsets = torch.tensor([0] + torch.tensor(lengths).cumsum(0).tolist(), dtype=torch.int32,
+                           device=device)
+    query = nonzero_randn((total, 3, bits), dtype=torch.float32, seed=bits).to(device)
+    key = nonzero_randn((total, 3, bits), dtype=torch.float32, seed=bits + 1).to(device)
+    # a repeated stretch inside the longest sequence, so that long runs exist
+    begin = sum(lengths[:7])
+    key[begin + 500:begin + 900] = key[begin + 50:begin + 450]
+    query[begin + 501:begin + 900] = key[begin + 500:begin + 899]
+    value = nonzero_randn((total, 3, 8), dtype=torch.float32, seed=3).to(device)
+    cabi.set_forward_index("scan")
+    want_output, _, _, want_routes = cabi.hard_forward(query, key, value, window, offsets)
+    assert int((want_routes > 0).sum()) > 0
+    for mode in ("always", "handed_back", None):
+        cabi.set_forward_index(mode)
+        output, _, _, routes = cabi.hard_forward(query, key, value, window, offsets)
+        assert torch.equal(routes, want_routes), mode
+        assert torch.equal(output, want_output), mode
+    cabi.set_forward_index(None)
+
+
+def test_indexed_forward_through_the_entry_point_that_allocates_nothing(cabi):
+    device = torch.device("cuda:0")
+    query = nonzero_randn((2, 900, 4, 8), dtype=torch.float32, seed=41).to(device)
+    key = nonzero_randn((2, 900, 4, 8), dtype=torch.float32, seed=42).to(device)
+    value = nonzero_randn((2, 900, 2, 8), dtype=torch.float32, seed=43).to(device)
+    cabi.set_forward_index("scan")
+    want_output, _, _, want_routes = cabi.hard_forward(query, key, value, 32)
+    cabi.set_forward_index("always")
+    try:
+        output, _, _, routes = cabi.hard_forward_static(query, key, value, 32)
+    finally:
+        cabi.set_forward_index(None)
+    assert torch.equal(routes, want_routes) and torch.equal(output, want_output)
