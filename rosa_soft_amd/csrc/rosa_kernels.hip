@@ -184,6 +184,64 @@ __global__ __launch_bounds__(256) void pack_symbols_ballot_kernel(
   }
 }
 
+// Symbols of whole 16-byte pieces (D * element size a multiple of 16): a thread reads its
+// symbol in 16-byte loads, and a block of kPackTokens tokens x H heads turns its words
+// through LDS, so that they leave head-major in runs of kPackTokens consecutive tokens (the
+// kernel above writes every word to a line of its own).  Dynamic LDS: two tiles of
+// [H][kPackTokens + 1] words.
+constexpr int kPackTokens = 16;
+constexpr int kPackHeadsMax = 256;
+
+template <int DTYPE>
+__global__ __launch_bounds__(256) void pack_symbols_tile_kernel(
+    const void* __restrict__ query, const void* __restrict__ key,
+    int32_t* __restrict__ packed_query, int32_t* __restrict__ packed_key, int64_t tokens, int D,
+    int H, int T, int N, int varlen) {
+  extern __shared__ uint32_t pack_tile[];
+  constexpr int kPiece = DTYPE == ROSA_DTYPE_F32 ? 4 : 8;  // elements in 16 bytes
+  constexpr int kPitch = kPackTokens + 1;
+  uint32_t* q_tile = pack_tile;
+  uint32_t* k_tile = pack_tile + H * kPitch;
+  const int64_t token0 = static_cast<int64_t>(blockIdx.x) * kPackTokens;
+  const int here = static_cast<int>(min<int64_t>(kPackTokens, tokens - token0));
+  const int rows = here * H;
+  const int pieces = D / kPiece;
+  const uint4* q_pieces = reinterpret_cast<const uint4*>(query) + token0 * H * pieces;
+  const uint4* k_pieces = reinterpret_cast<const uint4*>(key) + token0 * H * pieces;
+  for (int r = threadIdx.x; r < rows; r += blockDim.x) {
+    uint32_t q_word = 0u, k_word = 0u;
+    for (int piece = 0; piece < pieces; ++piece) {
+      const uint4 q_in = q_pieces[static_cast<int64_t>(r) * pieces + piece];
+      const uint4 k_in = k_pieces[static_cast<int64_t>(r) * pieces + piece];
+#pragma unroll
+      for (int e = 0; e < kPiece; ++e) {
+        if (load_as_float<DTYPE>(&q_in, e) > 0.0f) q_word |= 1u << (piece * kPiece + e);
+        if (load_as_float<DTYPE>(&k_in, e) > 0.0f) k_word |= 1u << (piece * kPiece + e);
+      }
+    }
+    const int local = r / H;
+    const int h = r - local * H;
+    q_tile[h * kPitch + local] = q_word;
+    k_tile[h * kPitch + local] = k_word;
+  }
+  __syncthreads();
+  for (int index = threadIdx.x; index < H * kPackTokens; index += blockDim.x) {
+    const int h = index / kPackTokens;
+    const int local = index - h * kPackTokens;
+    if (local >= here) continue;
+    const int64_t token = token0 + local;
+    int64_t dst;
+    if (varlen) {
+      dst = static_cast<int64_t>(h) * N + token;
+    } else {
+      const int64_t b = token / T;
+      dst = (b * H + h) * T + (token - b * T);
+    }
+    packed_query[dst] = static_cast<int32_t>(q_tile[h * kPitch + local]);
+    packed_key[dst] = static_cast<int32_t>(k_tile[h * kPitch + local]);
+  }
+}
+
 // Widths that do not divide 64: one lane per symbol.
 template <int DTYPE>
 __global__ __launch_bounds__(256) void pack_symbols_rows_kernel(
@@ -449,7 +507,7 @@ __global__ __launch_bounds__(kWave) void hard_route_kernel(
 // (few distinct symbols), and a row block whose walk exceeds its budget of iterations (long
 // matches everywhere, as on periodic inputs); hard_route_kernel then runs for those blocks
 // only.
-constexpr int kIndexThreads = 256;
+constexpr int kIndexThreads = 1024;
 constexpr int kIndexBucketsMax = 4096;
 
 __device__ __forceinline__ uint32_t key_bucket(uint32_t symbol, int log_buckets, int hashed) {
@@ -532,11 +590,18 @@ __global__ __launch_bounds__(kIndexThreads) void index_keys_kernel(
     index.unit_scan[unit] = largest > max(64, count / 16) ? 1 : 0;
   }
   __syncthreads();
+  // The positions go out in passes of kIndexThreads with a barrier between the passes: inside
+  // a bucket the entries of an earlier pass then lie before those of a later one, and a row
+  // can stop at the first entry of a pass that begins beyond it.
   uint4* entries = index.entries + word_base;
-  for (int p = thread; p < count; p += kIndexThreads) {
-    const uint32_t symbol = k[p];
-    const int slot = atomicAdd(&cursor[key_bucket(symbol, index.log_buckets, index.hashed)], 1);
-    entries[slot] = make_uint4(static_cast<uint32_t>(p + 1), symbol, p >= 1 ? k[p - 1] : 0u, 0u);
+  for (int p0 = 0; p0 < count; p0 += kIndexThreads) {
+    const int p = p0 + thread;
+    if (p < count) {
+      const uint32_t symbol = k[p];
+      const int slot = atomicAdd(&cursor[key_bucket(symbol, index.log_buckets, index.hashed)], 1);
+      entries[slot] = make_uint4(static_cast<uint32_t>(p + 1), symbol, p >= 1 ? k[p - 1] : 0u, 0u);
+    }
+    __syncthreads();
   }
 }
 
@@ -586,6 +651,8 @@ __global__ __launch_bounds__(kWave) void route_candidates_kernel(
     ++next;
     if (next < end) ahead = entries[next];
     const int a = static_cast<int>(entry.x);
+    // an entry of a pass of the index that begins beyond this row: so do all that follow
+    if (have && ((a - 1) & ~(kIndexThreads - 1)) >= t) next = end;
     const bool candidate = have && a <= t && entry.y == q_symbol;
     const int limit = min(L.W, a);
     int run = candidate ? 1 : 0;
@@ -654,6 +721,44 @@ __global__ __launch_bounds__(256) void gather_values_kernel(
     sign = x > 0.0f ? 1 : -1;
   }
   store_sign<DTYPE>(output, index, sign);
+}
+
+// The same with 16 bytes of a row per thread, for value widths of whole 16-byte pieces.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void gather_value_pieces_kernel(
+    const int32_t* __restrict__ source_token, const void* __restrict__ value,
+    void* __restrict__ output, int64_t pieces, int pieces_per_row, int H, int Hv, int Dv, int T,
+    int N, int varlen, const int32_t* __restrict__ offset_error) {
+  constexpr int kPiece = DTYPE == ROSA_DTYPE_F32 ? 4 : 8;  // elements in 16 bytes
+  const int64_t piece = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (piece >= pieces) return;
+  uint4 out = make_uint4(0u, 0u, 0u, 0u);
+  if (offset_error != nullptr && *offset_error != 0) {
+#pragma unroll
+    for (int e = 0; e < kPiece; ++e) store_nan<DTYPE>(&out, e);
+  } else {
+    const int64_t row = piece / pieces_per_row;
+    const int part = static_cast<int>(piece - row * pieces_per_row);
+    const int64_t token = row / H;
+    const int h = static_cast<int>(row - token * H);
+    int64_t word;
+    if (varlen) {
+      word = static_cast<int64_t>(h) * N + token;
+    } else {
+      const int64_t b = token / T;
+      word = (b * H + h) * T + (token - b * T);
+    }
+    const int source = source_token[word];
+    if (source >= 0) {
+      const int hv = h / (H / Hv);
+      const uint4 in = reinterpret_cast<const uint4*>(value)[
+          ((static_cast<int64_t>(source) * Hv + hv) * Dv) / kPiece + part];
+#pragma unroll
+      for (int e = 0; e < kPiece; ++e)
+        store_sign<DTYPE>(&out, e, load_as_float<DTYPE>(&in, e) > 0.0f ? 1 : -1);
+    }
+  }
+  reinterpret_cast<uint4*>(output)[piece] = out;
 }
 
 // The same output as sign and validity bits, for a consumer that expands the ternary
@@ -1415,8 +1520,18 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   launch_prepare_sequences(p, L, workspace, w.seq_start, w.seq_len, w.block_prefix, w.header,
                            stream);
   const int64_t elements = view.symbol_rows * L.D;
+  constexpr int kPackPiece = DTYPE == ROSA_DTYPE_F32 ? 4 : 8;  // elements in 16 bytes
+  const bool whole_symbol_pieces =
+      L.D % kPackPiece == 0 && L.H <= kPackHeadsMax &&
+      ((reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(key)) & 15u) == 0;
   if (words_given) {
     // a producer (the projection in front of the operator) has written the symbol words
+  } else if (whole_symbol_pieces) {
+    const size_t tile_bytes = sizeof(uint32_t) * 2 * static_cast<size_t>(L.H) * (kPackTokens + 1);
+    hipLaunchKernelGGL(pack_symbols_tile_kernel<DTYPE>,
+                       dim3(blocks_for(view.tokens, kPackTokens)), dim3(256), tile_bytes, stream,
+                       query, key, packed_query, packed_key, view.tokens, L.D, L.H, L.T, L.N,
+                       L.varlen);
   } else if (64 % L.D == 0) {
     hipLaunchKernelGGL(pack_symbols_ballot_kernel<DTYPE>, dim3(blocks_for(elements, 256)),
                        dim3(256), 0, stream, query, key, packed_query, packed_key, elements, L.D,
@@ -1486,9 +1601,20 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
                        L.Dv, nvw, L.T, L.N, L.varlen, offset_error);
   } else {
     const int64_t out_elements = view.symbol_rows * L.Dv;
-    hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)),
-                       dim3(256), 0, stream, source_token, value, output, out_elements, L.H,
-                       L.Hv, L.Dv, L.T, L.N, L.varlen, offset_error);
+    constexpr int kPiece = DTYPE == ROSA_DTYPE_F32 ? 4 : 8;  // elements in 16 bytes
+    const bool whole_pieces =
+        L.Dv % kPiece == 0 &&
+        ((reinterpret_cast<uintptr_t>(value) | reinterpret_cast<uintptr_t>(output)) & 15u) == 0;
+    if (whole_pieces) {
+      const int64_t pieces = out_elements / kPiece;
+      hipLaunchKernelGGL(gather_value_pieces_kernel<DTYPE>, dim3(blocks_for(pieces, 256)),
+                         dim3(256), 0, stream, source_token, value, output, pieces,
+                         L.Dv / kPiece, L.H, L.Hv, L.Dv, L.T, L.N, L.varlen, offset_error);
+    } else {
+      hipLaunchKernelGGL(gather_values_kernel<DTYPE>, dim3(blocks_for(out_elements, 256)),
+                         dim3(256), 0, stream, source_token, value, output, out_elements, L.H,
+                         L.Hv, L.Dv, L.T, L.N, L.varlen, offset_error);
+    }
   }
   stage_end(kStageForward, stream);
   const hipError_t status = hipGetLastError();
