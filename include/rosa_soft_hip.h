@@ -229,7 +229,8 @@ int rosa_hip_project_routed_bits(const uint32_t* sign_words, const uint8_t* rout
  * library's device image (one copy per GPU, held until the process ends), so the call
  * takes no workspace argument and calls no allocator; it handles problems whose forward
  * workspace fits, i.e. about tokens * H <= 4 190 000, and returns 3 with a message
- * beyond that.  All calls on one GPU share that GPU's array: calls that overlap in time
+ * beyond that (up to about tokens * H <= 680 000 the array also holds the index of the
+ * keys, see rosa_hip_set_forward_index; beyond that the call scans all routes).  All calls on one GPU share that GPU's array: calls that overlap in time
  * on one GPU (different streams or threads) race and must be ordered by the caller.
  * The first call on a device looks up the array's address (hipGetSymbolAddress), which is
  * not a stream operation: make that call before recording the stream into a graph; every
@@ -286,6 +287,14 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
  * consecutive updates need no host traffic; the caller keeps
  * history length + chunk length <= capacity.  `longest_chunk` is the largest number of new
  * tokens of any slot (small chunks are routed by a per-row kernel).
+ * `workspace` (optional) lets an update with a long chunk route through an index of the keys
+ * by symbol, rebuilt by that update over every run's whole history (see
+ * rosa_hip_set_forward_index; same routes): `longest_total` is then the largest history
+ * length + chunk length of any slot, and `workspace_bytes` at least
+ * rosa_hip_router_workspace_bytes(update), which is 0 for updates that would not use it
+ * (symbols below six bits, chunks of up to 8 tokens, histories below 512 tokens).  With
+ * `workspace` NULL every route is scanned.  The workspace carries nothing from one update to
+ * the next.
  */
 typedef struct rosa_router_update {
   int32_t S, H, Hp, W;
@@ -304,8 +313,12 @@ typedef struct rosa_router_update {
   const uint8_t* payload;
   uint8_t* output;
   int64_t* matched_key_end;
+  int32_t longest_total;
+  void* workspace;
+  size_t workspace_bytes;
 } rosa_router_update;
 
+size_t rosa_hip_router_workspace_bytes(const rosa_router_update* update);
 int rosa_hip_router_update(const rosa_router_update* update, void* stream);
 
 /*

@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = (
     "rosa_hip_pack_symbols",
     "rosa_hip_surrogate_vjp",
     "rosa_hip_router_update",
+    "rosa_hip_router_workspace_bytes",
     "rosa_hip_read_offset_error",
     "rosa_hip_stage_timing",
     "rosa_hip_stage_count",
@@ -94,6 +95,9 @@ class RosaRouterUpdate(ctypes.Structure):
         ("payload", ctypes.c_void_p),
         ("output", ctypes.c_void_p),
         ("matched_key_end", ctypes.c_void_p),
+        ("longest_total", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -170,6 +174,8 @@ def load() -> ctypes.CDLL:
     library.rosa_hip_pack_symbols.argtypes = [
         ctypes.c_int, vp, ctypes.c_int64, ctypes.c_int, vp, ctypes.c_int, vp,
     ]
+    library.rosa_hip_router_workspace_bytes.restype = ctypes.c_size_t
+    library.rosa_hip_router_workspace_bytes.argtypes = [ctypes.POINTER(RosaRouterUpdate)]
     library.rosa_hip_router_update.restype = ctypes.c_int
     library.rosa_hip_router_update.argtypes = [ctypes.POINTER(RosaRouterUpdate), vp]
     library.rosa_hip_surrogate_vjp.restype = ctypes.c_int
@@ -571,14 +577,25 @@ def vjp_workspace_bytes(query: Tensor, value: Tensor, max_suffix_length: int,
     return int(load().rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, int(dropout)))
 
 
-def router_update(update: RosaRouterUpdate, device: torch.device) -> None:
-    """Enqueue one streaming-router update on the current stream of ``device``."""
+def router_update(update: RosaRouterUpdate, device: torch.device) -> Optional[Tensor]:
+    """Enqueue one streaming-router update on the current stream of ``device``.
 
+    ``update.longest_total`` must be set.  Returns the workspace the update uses (or ``None``):
+    the launches are stream-ordered, so the caller keeps it alive until they have run.
+    """
+
+    workspace = None
     with torch.cuda.device(device):
+        size = int(load().rosa_hip_router_workspace_bytes(ctypes.byref(update)))
+        if size > 0:
+            workspace = torch.empty(size, dtype=torch.uint8, device=device)
+            update.workspace = workspace.data_ptr()
+            update.workspace_bytes = size
         status = load().rosa_hip_router_update(
             ctypes.byref(update), torch.cuda.current_stream(device).cuda_stream
         )
     _check(status, "rosa_hip_router_update")
+    return workspace
 
 
 def set_record_budget(limit_bytes: Optional[int]) -> None:

@@ -1925,6 +1925,14 @@ struct RouterUpdate {
   int64_t* matched_key_end;      // [tokens][H]
   int tokens;
   int blocks_per_run;            // blocks of the routing grid that share one (slot, head)
+  // the index of the keys of every run, rebuilt by an update that uses it (NULL: none)
+  int32_t* bucket_begin;         // [runs][2^qk_bits + 1]
+  int32_t* bucket_routes;        // [runs][index_stride]: the routes, by bucket
+  uint8_t* run_scan;             // [runs]: 1 = the run is left to the scan
+  uint8_t* left_over;            // [blocks of the routing grid]: 1 = left to the scan
+  int index_stride;
+  int log_buckets;
+  int budget_base;
 };
 
 __device__ __forceinline__ int router_chunk_begin(const RouterUpdate& U, int slot) {
@@ -1961,6 +1969,8 @@ __global__ __launch_bounds__(256) void router_append_kernel(RouterUpdate U) {
 // the routes exactly like hard_route_kernel; the first row block starts at the slot's old
 // length, so its predecessor row lies in the history.
 __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
+  // (behind router_candidates_kernel: only the row blocks that kernel has left over)
+  if (U.left_over != nullptr && U.left_over[blockIdx.x] == 0) return;
   // one-dimensional grid: (slot, head) run-major, so that slots * heads is not bounded by
   // the 65535 blocks of the other grid dimensions
   const int run = static_cast<int>(blockIdx.x / static_cast<unsigned>(U.blocks_per_run));
@@ -1994,6 +2004,130 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
       : uint8_t(0);
 }
 
+// The index of the keys for the router (see index_keys_kernel): byte symbols, one bucket per
+// symbol, the whole history of a run indexed anew by every update that routes a long chunk.
+// An entry is the route alone; the key symbol is the bucket's, the one before it is read.
+__global__ __launch_bounds__(kIndexThreads) void router_index_kernel(RouterUpdate U) {
+  __shared__ int cursor[256];
+  __shared__ int partial[256];
+  __shared__ int largest;
+  const int run = blockIdx.x;
+  const int slot = run / U.H;
+  const int new_length = U.history_lengths[slot] +
+                         (router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot));
+  const int count = max(new_length - 1, 0);
+  const int buckets = 1 << U.log_buckets;
+  const uint8_t* k = U.key_history + static_cast<int64_t>(run) * U.capacity;
+  const int thread = threadIdx.x;
+  if (thread < 256) cursor[thread] = 0;
+  if (thread == 0) largest = 0;
+  __syncthreads();
+  for (int p = thread; p < count; p += kIndexThreads) atomicAdd(&cursor[k[p]], 1);
+  __syncthreads();
+  const int mine = thread < buckets ? cursor[thread] : 0;
+  if (thread < 256) partial[thread] = mine;
+  if (thread < buckets) atomicMax(&largest, mine);
+  __syncthreads();
+  for (int step = 1; step < 256; step <<= 1) {
+    const int below = (thread < 256 && thread >= step) ? partial[thread - step] : 0;
+    __syncthreads();
+    if (thread < 256) partial[thread] += below;
+    __syncthreads();
+  }
+  int32_t* begin = U.bucket_begin + static_cast<int64_t>(run) * (buckets + 1);
+  if (thread < buckets) {
+    cursor[thread] = partial[thread] - mine;
+    begin[thread] = partial[thread] - mine;
+  }
+  if (thread == 0) {
+    begin[buckets] = count;
+    U.run_scan[run] = largest > max(64, count / 16) ? 1 : 0;
+  }
+  __syncthreads();
+  int32_t* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
+  for (int p0 = 0; p0 < count; p0 += kIndexThreads) {  // ordered passes, as in index_keys_kernel
+    const int p = p0 + thread;
+    if (p < count) routes[atomicAdd(&cursor[k[p]], 1)] = p + 1;
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kWave) void router_candidates_kernel(RouterUpdate U) {
+  const int run = static_cast<int>(blockIdx.x / static_cast<unsigned>(U.blocks_per_run));
+  const int row_block = static_cast<int>(blockIdx.x - static_cast<unsigned>(run) * U.blocks_per_run);
+  const int slot = run / U.H;
+  const int head = run - slot * U.H;
+  const int lane = threadIdx.x;
+  const int old_length = U.history_lengths[slot];
+  const int chunk_begin = router_chunk_begin(U, slot);
+  const int new_length = old_length + (router_chunk_begin(U, slot + 1) - chunk_begin);
+  const int t0 = old_length + row_block * kWave;
+  if (t0 >= new_length || U.run_scan[run] != 0) {
+    if (lane == 0) U.left_over[blockIdx.x] = t0 < new_length ? 1 : 0;
+    return;
+  }
+  const int64_t run_base = static_cast<int64_t>(run) * U.capacity;
+  const uint8_t* q = U.query_history + run_base;
+  const uint8_t* k = U.key_history + run_base;
+  const int t = t0 + lane;
+  const bool row_ok = t < new_length;
+  const uint32_t q_symbol = row_ok ? q[t] : 0u;
+  const uint32_t q_before = (row_ok && t >= 1) ? q[t - 1] : 0u;
+  const int buckets = 1 << U.log_buckets;
+  const int32_t* begin = U.bucket_begin + static_cast<int64_t>(run) * (buckets + 1);
+  int next = row_ok ? begin[q_symbol] : 0;
+  const int end = row_ok ? begin[q_symbol + 1] : 0;
+  const int32_t* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
+  const int budget = U.budget_base + t0 / 8;
+  const int walk_budget = budget / 4;
+  int spent = 0, walked = 0;  // wave-uniform
+  uint64_t best = 0;          // (run << 32) | route
+  int ahead = next < end ? routes[next] : 0;
+  uint32_t ahead_before = ahead >= 2 ? k[ahead - 2] : 0x100u;
+  while (__builtin_amdgcn_ballot_w64(next < end) != 0ull) {
+    const bool have = next < end;
+    const int a = ahead;
+    const uint32_t key_before = ahead_before;
+    ++next;
+    if (next < end) {
+      ahead = routes[next];
+      ahead_before = ahead >= 2 ? k[ahead - 2] : 0x100u;
+    }
+    if (have && ((a - 1) & ~(kIndexThreads - 1)) >= t) next = end;
+    const bool candidate = have && a <= t;
+    const int limit = min(U.W, a);
+    int length = candidate ? 1 : 0;
+    bool walking = candidate && limit >= 2 && key_before == q_before;
+    if (walking) length = 2;
+    walking = walking && length < limit;
+    while (walked <= walk_budget && __builtin_amdgcn_ballot_w64(walking) != 0ull) {
+      ++walked;
+      if (walking) {
+        if (q[t - length] == k[a - 1 - length]) {
+          ++length;
+          walking = length < limit;
+        } else {
+          walking = false;
+        }
+      }
+    }
+    const uint64_t found = (static_cast<uint64_t>(length) << 32) | static_cast<uint32_t>(a);
+    if (candidate) best = max(best, found);
+    if (++spent > budget || walked > walk_budget) {
+      if (lane == 0) U.left_over[blockIdx.x] = 1;
+      return;
+    }
+  }
+  if (lane == 0) U.left_over[blockIdx.x] = 0;
+  if (!row_ok) return;
+  const int route = (best >> 32) > 0 ? static_cast<int>(best & 0xffffffffu) : 0;
+  const int64_t token = chunk_begin + (t - old_length);
+  const int payload_head = head / (U.H / U.Hp);
+  U.matched_key_end[token * U.H + head] = route > 0 ? route - 1 : -1;
+  U.output[token * U.H + head] = route > 0
+      ? U.payload_history[(static_cast<int64_t>(slot) * U.Hp + payload_head) * U.capacity + route]
+      : uint8_t(0);
+}
 
 // Few new rows per slot (decoding): one wave per (slot, head, new row); the lanes share the
 // routes of the row, each comparing its suffixes directly, and the wave keeps the maximum of
@@ -2304,6 +2438,36 @@ void launch_pack_rows(const void* logits, int64_t rows, int bits, void* symbols,
   }
 }
 
+// The router's index of the keys in the caller's workspace: bucket offsets, routes by bucket,
+// one byte per run and one per block of the routing grid.
+struct RouterWorkspace {
+  size_t bucket_begin, bucket_routes, run_scan, left_over, total;
+  int blocks_per_run;
+};
+
+// Updates the index is used for: symbols of six bits or more (as in the training forward),
+// chunks beyond the per-row kernel's, and histories long enough for the extra launches to pay.
+constexpr int kRouterIndexLongestMin = 512;
+
+bool router_index_suits(const rosa_router_update& u) {
+  return u.qk_bits >= kIndexSymbolBitsMin && u.longest_chunk > kRouterDecodeRows &&
+         u.longest_total >= kRouterIndexLongestMin;
+}
+
+RouterWorkspace carve_router(const rosa_router_update& u) {
+  RouterWorkspace w;
+  const size_t runs = static_cast<size_t>(u.S) * u.H;
+  w.blocks_per_run = (u.longest_chunk + kWave - 1) / kWave;
+  size_t cursor = 0;
+  w.bucket_begin = cursor; cursor += align_up(sizeof(int32_t) * runs * ((size_t(1) << u.qk_bits) + 1));
+  w.bucket_routes = cursor;
+  cursor += align_up(sizeof(int32_t) * runs * static_cast<size_t>(std::max(u.longest_total, 1)));
+  w.run_scan = cursor; cursor += align_up(runs);
+  w.left_over = cursor; cursor += align_up(runs * static_cast<size_t>(std::max(w.blocks_per_run, 1)));
+  w.total = cursor;
+  return w;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -2511,6 +2675,13 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query, const
   }
 }
 
+size_t rosa_hip_router_workspace_bytes(const rosa_router_update* update) {
+  if (update == nullptr || update->S < 1 || update->H < 1 || update->qk_bits < 1 ||
+      update->qk_bits > 8 || update->longest_chunk < 0 || update->longest_total < 0)
+    return 0;
+  return router_index_suits(*update) ? carve_router(*update).total : 0;
+}
+
 int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   if (update == nullptr) return fail(1, "router update is NULL");
   const rosa_router_update& u = *update;
@@ -2543,6 +2714,24 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   U.matched_key_end = u.matched_key_end;
   U.tokens = u.tokens;
   U.blocks_per_run = 1;
+  U.bucket_begin = nullptr; U.bucket_routes = nullptr; U.run_scan = nullptr; U.left_over = nullptr;
+  U.index_stride = 0; U.log_buckets = 0; U.budget_base = 0;
+  const int index_mode = g_forward_index_mode.load(std::memory_order_relaxed);
+  bool indexed = false;
+  if (u.workspace != nullptr && index_mode != 1 && router_index_suits(u)) {
+    if (u.longest_total > u.capacity)
+      return fail(1, "router: longest_total exceeds the capacity of a run");
+    const RouterWorkspace w = carve_router(u);
+    if (u.workspace_bytes < w.total) return fail(3, "router: workspace too small");
+    U.bucket_begin = at<int32_t>(u.workspace, w.bucket_begin);
+    U.bucket_routes = at<int32_t>(u.workspace, w.bucket_routes);
+    U.run_scan = at<uint8_t>(u.workspace, w.run_scan);
+    U.left_over = at<uint8_t>(u.workspace, w.left_over);
+    U.index_stride = std::max(u.longest_total, 1);
+    U.log_buckets = u.qk_bits;
+    U.budget_base = index_mode == 2 ? -(1 << 30) : 64;
+    indexed = true;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t symbols = static_cast<int64_t>(u.tokens) * u.H;
   hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
@@ -2556,6 +2745,12 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
       hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
                          s, U);
     } else {
+      if (indexed) {
+        hipLaunchKernelGGL(router_index_kernel, dim3(static_cast<unsigned>(runs)),
+                           dim3(kIndexThreads), 0, s, U);
+        hipLaunchKernelGGL(router_candidates_kernel, dim3(static_cast<unsigned>(blocks)),
+                           dim3(kWave), 0, s, U);
+      }
       hipLaunchKernelGGL(router_route_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
                          s, U);
     }

@@ -505,9 +505,12 @@ class RosaRuntime:
         update.query, update.key, update.payload = \
             query.data_ptr(), key.data_ptr(), payload.data_ptr()
         update.output, update.matched_key_end = output.data_ptr(), ends.data_ptr()
-        cabi.router_update(update, self._device)
-        if tables is not None:  # stream-ordered launch: keep the table alive until it has run
-            tables.record_stream(torch.cuda.current_stream(self._device))
+        update.longest_total = max(old + new for old, new in zip(self._lengths, chunk_lengths))
+        workspace = cabi.router_update(update, self._device)
+        # stream-ordered launches: keep what they read alive until they have run
+        for held in (tables, workspace):
+            if held is not None:
+                held.record_stream(torch.cuda.current_stream(self._device))
         self._lengths = [old + new for old, new in zip(self._lengths, chunk_lengths)]
         return output, ends
 

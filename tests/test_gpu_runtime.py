@@ -342,3 +342,78 @@ def test_updates_on_different_streams_are_serialised(rosa):
         torch.cuda.synchronize()
     assert torch.equal(torch.cat([r[0] for r in results], dim=1).cpu(), want[0])
     assert torch.equal(torch.cat([r[1] for r in results], dim=1).cpu(), want[1])
+
+
+@pytest.mark.parametrize("pattern", ["random", "period7", "constant"])
+def test_long_chunks_route_through_the_index_of_the_keys(rosa, pattern):
+    # chunks beyond 8 rows on histories of 512 tokens or more take the index of the keys
+    # (8- and 6-bit symbols here); periodic and constant inputs hand their row blocks back.
+    # The scan over all routes gives the expectation (the oracle as well where it is quick).
+    from rosa_soft_amd import cabi
+
+    batch, tokens, heads, payload_heads = 2, 1500, 4, 2
+    for bits in (8, 6):
+        query = random_packed((batch, tokens, heads), bits, 50 + bits)
+        key = random_packed((batch, tokens, heads), bits, 60 + bits)
+        if pattern == "period7":
+            key = key[:, :7].repeat(1, tokens // 7 + 1, 1)[:, :tokens].contiguous()
+            query = torch.roll(key, 1, dims=1).contiguous()
+        elif pattern == "constant":
+            key = torch.full_like(key, 3)
+            query = torch.full_like(query, 3)
+        else:
+            # a repeated stretch, so that long runs and ties exist
+            key[:, 900:1300] = key[:, 100:500]
+            query[:, 901:1300] = key[:, 900:1299]
+        payload = random_packed((batch, tokens, payload_heads), 8, 70 + bits)
+        results = {}
+        for mode in ("scan", None, "handed_back"):
+            outputs, positions = [], []
+            cabi.set_forward_index(mode)
+            try:
+                with rosa.RosaRuntime(heads, payload_heads, bits, 8, 40) as runtime:
+                    for begin, end in [(0, 700), (700, 705), (705, 1400), (1400, 1500)]:
+                        output, ends = runtime.update_packed(
+                            query[:, begin:end].to(DEVICE), key[:, begin:end].to(DEVICE),
+                            payload[:, begin:end].to(DEVICE))
+                        outputs.append(output)
+                        positions.append(ends)
+            finally:
+                cabi.set_forward_index(None)
+            results[mode] = (torch.cat(outputs, dim=1).cpu(), torch.cat(positions, dim=1).cpu())
+        for mode in (None, "handed_back"):
+            assert torch.equal(results[mode][0], results["scan"][0]), (bits, mode)
+            assert torch.equal(results[mode][1], results["scan"][1]), (bits, mode)
+        assert int((results["scan"][1] >= 0).sum()) > 0
+        if pattern == "random" and bits == 8:
+            want = expect_dense(query, key, payload, bits, 8, 40)
+            assert torch.equal(results[None][0], want[0]) and torch.equal(results[None][1], want[1])
+
+
+def test_ragged_long_chunks_route_through_the_index_of_the_keys(rosa):
+    heads, payload_heads, bits = 3, 3, 8
+    lengths = [[600, 0, 900], [700, 650, 9], [64, 800, 300]]  # per update, per slot
+    totals = [sum(step[slot] for step in lengths) for slot in range(3)]
+    streams = []
+    for slot, total in enumerate(totals):
+        query = random_packed((1, total, heads), bits, 80 + slot)
+        key = random_packed((1, total, heads), bits, 90 + slot)
+        payload = random_packed((1, total, payload_heads), bits, 100 + slot)
+        streams.append((query, key, payload, expect_dense(query, key, payload, bits, bits, 33)))
+    done = [0, 0, 0]
+    with rosa.RosaRuntime(heads, payload_heads, bits, bits, 33) as runtime:
+        for step in lengths:
+            parts = [[s[i][0, done[slot]:done[slot] + step[slot]] for slot, s in enumerate(streams)]
+                     for i in range(3)]
+            offsets = [0]
+            for length in step:
+                offsets.append(offsets[-1] + length)
+            output, ends = runtime.update_packed(
+                torch.cat(parts[0]).to(DEVICE), torch.cat(parts[1]).to(DEVICE),
+                torch.cat(parts[2]).to(DEVICE), cu_seqlens=torch.tensor(offsets, dtype=torch.int32))
+            for slot, s in enumerate(streams):
+                rows = slice(offsets[slot], offsets[slot + 1])
+                want = s[3]
+                assert torch.equal(output[rows].cpu(), want[0][0, done[slot]:done[slot] + step[slot]])
+                assert torch.equal(ends[rows].cpu(), want[1][0, done[slot]:done[slot] + step[slot]])
+                done[slot] += step[slot]
