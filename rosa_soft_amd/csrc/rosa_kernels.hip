@@ -1927,7 +1927,7 @@ struct RouterUpdate {
   int blocks_per_run;            // blocks of the routing grid that share one (slot, head)
   // the index of the keys of every run, rebuilt by an update that uses it (NULL: none)
   int32_t* bucket_begin;         // [runs][2^qk_bits + 1]
-  int32_t* bucket_routes;        // [runs][index_stride]: the routes, by bucket
+  uint2* bucket_routes;          // [runs][index_stride]: (route, key symbol before it), by bucket
   uint8_t* run_scan;             // [runs]: 1 = the run is left to the scan
   uint8_t* left_over;            // [blocks of the routing grid]: 1 = left to the scan
   int index_stride;
@@ -2006,7 +2006,7 @@ __global__ __launch_bounds__(kWave) void router_route_kernel(RouterUpdate U) {
 
 // The index of the keys for the router (see index_keys_kernel): byte symbols, one bucket per
 // symbol, the whole history of a run indexed anew by every update that routes a long chunk.
-// An entry is the route alone; the key symbol is the bucket's, the one before it is read.
+// An entry is the route and the key symbol before it; the key symbol itself is the bucket's.
 __global__ __launch_bounds__(kIndexThreads) void router_index_kernel(RouterUpdate U) {
   __shared__ int cursor[256];
   __shared__ int partial[256];
@@ -2044,10 +2044,14 @@ __global__ __launch_bounds__(kIndexThreads) void router_index_kernel(RouterUpdat
     U.run_scan[run] = largest > max(64, count / 16) ? 1 : 0;
   }
   __syncthreads();
-  int32_t* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
+  uint2* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
   for (int p0 = 0; p0 < count; p0 += kIndexThreads) {  // ordered passes, as in index_keys_kernel
     const int p = p0 + thread;
-    if (p < count) routes[atomicAdd(&cursor[k[p]], 1)] = p + 1;
+    if (p < count) {
+      // (route 1 has no key before it: a value no symbol takes)
+      routes[atomicAdd(&cursor[k[p]], 1)] =
+          make_uint2(static_cast<uint32_t>(p + 1), p >= 1 ? static_cast<uint32_t>(k[p - 1]) : 0x100u);
+    }
     __syncthreads();
   }
 }
@@ -2077,22 +2081,18 @@ __global__ __launch_bounds__(kWave) void router_candidates_kernel(RouterUpdate U
   const int32_t* begin = U.bucket_begin + static_cast<int64_t>(run) * (buckets + 1);
   int next = row_ok ? begin[q_symbol] : 0;
   const int end = row_ok ? begin[q_symbol + 1] : 0;
-  const int32_t* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
+  const uint2* routes = U.bucket_routes + static_cast<int64_t>(run) * U.index_stride;
   const int budget = U.budget_base + t0 / 8;
   const int walk_budget = budget / 4;
   int spent = 0, walked = 0;  // wave-uniform
   uint64_t best = 0;          // (run << 32) | route
-  int ahead = next < end ? routes[next] : 0;
-  uint32_t ahead_before = ahead >= 2 ? k[ahead - 2] : 0x100u;
+  uint2 ahead = next < end ? routes[next] : make_uint2(0u, 0x100u);
   while (__builtin_amdgcn_ballot_w64(next < end) != 0ull) {
     const bool have = next < end;
-    const int a = ahead;
-    const uint32_t key_before = ahead_before;
+    const int a = static_cast<int>(ahead.x);
+    const uint32_t key_before = ahead.y;
     ++next;
-    if (next < end) {
-      ahead = routes[next];
-      ahead_before = ahead >= 2 ? k[ahead - 2] : 0x100u;
-    }
+    if (next < end) ahead = routes[next];
     if (have && ((a - 1) & ~(kIndexThreads - 1)) >= t) next = end;
     const bool candidate = have && a <= t;
     const int limit = min(U.W, a);
@@ -2461,7 +2461,7 @@ RouterWorkspace carve_router(const rosa_router_update& u) {
   size_t cursor = 0;
   w.bucket_begin = cursor; cursor += align_up(sizeof(int32_t) * runs * ((size_t(1) << u.qk_bits) + 1));
   w.bucket_routes = cursor;
-  cursor += align_up(sizeof(int32_t) * runs * static_cast<size_t>(std::max(u.longest_total, 1)));
+  cursor += align_up(sizeof(uint2) * runs * static_cast<size_t>(std::max(u.longest_total, 1)));
   w.run_scan = cursor; cursor += align_up(runs);
   w.left_over = cursor; cursor += align_up(runs * static_cast<size_t>(std::max(w.blocks_per_run, 1)));
   w.total = cursor;
@@ -2724,7 +2724,7 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
     const RouterWorkspace w = carve_router(u);
     if (u.workspace_bytes < w.total) return fail(3, "router: workspace too small");
     U.bucket_begin = at<int32_t>(u.workspace, w.bucket_begin);
-    U.bucket_routes = at<int32_t>(u.workspace, w.bucket_routes);
+    U.bucket_routes = at<uint2>(u.workspace, w.bucket_routes);
     U.run_scan = at<uint8_t>(u.workspace, w.run_scan);
     U.left_over = at<uint8_t>(u.workspace, w.left_over);
     U.index_stride = std::max(u.longest_total, 1);
