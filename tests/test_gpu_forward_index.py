@@ -119,3 +119,35 @@ def test_indexed_forward_through_the_entry_point_that_allocates_nothing(cabi):
     finally:
         cabi.set_forward_index(None)
     assert torch.equal(routes, want_routes) and torch.equal(output, want_output)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [
+    # batch, length, heads, bits, value heads, value width
+    (2, 37, 3, 8, 3, 8),      # symbols and rows of whole 16-byte pieces, a block across two batches
+    (1, 130, 5, 16, 1, 24),
+    (3, 16, 2, 32, 2, 64),
+    (2, 50, 4, 4, 2, 4),      # whole pieces in float32 only
+    (1, 70, 2, 5, 2, 3),      # never whole pieces: one lane per symbol, one thread per element
+])
+def test_packed_words_and_gathered_output_of_every_kernel_variant(cabi, c_oracle, dtype, shape):
+    batch, length, heads, bits, value_heads, width = shape
+    device = torch.device("cuda:0")
+    query = nonzero_randn((batch, length, heads, bits), dtype=dtype, seed=1)
+    key = nonzero_randn((batch, length, heads, bits), dtype=dtype, seed=2)
+    value = nonzero_randn((batch, length, value_heads, width), dtype=dtype, seed=3)
+    output, packed_q, packed_k, routes = cabi.hard_forward(
+        query.to(device), key.to(device), value.to(device), 6)
+    weights = (1 << torch.arange(bits, dtype=torch.int64))
+    for packed, source in ((packed_q, query), (packed_k, key)):
+        want = ((source.float() > 0).to(torch.int64) * weights).sum(-1).permute(0, 2, 1)
+        assert torch.equal(packed.cpu().to(torch.int64) & 0xffffffff, want)
+    want_output, want_routes, _ = c_oracle.hard_forward(query, key, value, 6)
+    assert torch.equal(routes.cpu(), want_routes)
+    assert torch.equal(output.cpu(), want_output)
+    # packed sequences: the same tokens as one sequence per batch entry
+    offsets = torch.arange(batch + 1, dtype=torch.int32, device=device) * length
+    flat = [x.to(device).flatten(0, 1).contiguous() for x in (query, key, value)]
+    output_packed, words_q, _, _ = cabi.hard_forward(flat[0], flat[1], flat[2], 6, offsets)
+    assert torch.equal(output_packed.cpu(), want_output.flatten(0, 1))
+    assert torch.equal(words_q.cpu().view(heads, batch, length).permute(1, 0, 2), packed_q.cpu())
