@@ -151,3 +151,46 @@ def test_packed_words_and_gathered_output_of_every_kernel_variant(cabi, c_oracle
     output_packed, words_q, _, _ = cabi.hard_forward(flat[0], flat[1], flat[2], 6, offsets)
     assert torch.equal(output_packed.cpu(), want_output.flatten(0, 1))
     assert torch.equal(words_q.cpu().view(heads, batch, length).permute(1, 0, 2), packed_q.cpu())
+
+
+def test_indexed_forward_over_the_random_sweep_of_shapes(cabi, c_oracle):
+    """The forward of 300 cases of the sweep's case generator (symbol widths 1 to 32, lengths
+    around the 64-row blocks, random, shifted, periodic and constant inputs, three dtypes,
+    packed batches with empty sequences) with the index at every shape, against the oracle."""
+
+    import random
+
+    import numpy as np
+
+    from tests.test_gpu_parity import make_case
+    from tests.test_gpu_sweep import SHORT, draw_case, draw_run
+
+    device = torch.device("cuda:0")
+    rng = random.Random(4242)
+    cabi.set_forward_index("always")
+    try:
+        for index in range(300):
+            c = draw_case(rng, SHORT + [511, 777, 1024])
+            _, parts = draw_run(rng, c)
+            label = f"case {index}: {c} {parts}"
+            if not c["packed"]:
+                q, k, v, _ = make_case(c["B"], c["T"], c["H"], c["D"], c["Hv"], c["Dv"], c["dtype"],
+                                       seed=index, pattern=c["pattern"])
+                want_out, want_routes, _ = c_oracle.hard_forward(q, k, v, c["W"])
+                out, _, _, routes = cabi.hard_forward(q.to(device), k.to(device), v.to(device), c["W"])
+            else:
+                offsets = [0, *np.cumsum(parts).tolist()]
+                total = offsets[-1]
+                q = nonzero_randn((total, c["H"], c["D"]), seed=index + 1).to(c["dtype"])
+                k = nonzero_randn((total, c["H"], c["D"]), seed=index + 2).to(c["dtype"])
+                if c["pattern"] != "random":
+                    k = q.roll(2, dims=0).clone()
+                v = nonzero_randn((total, c["Hv"], c["Dv"]), seed=index + 3).to(c["dtype"])
+                want_out, want_routes = c_oracle.varlen_hard_forward(q, k, v, offsets, c["W"])
+                out, _, _, routes = cabi.hard_forward(
+                    q.to(device), k.to(device), v.to(device), c["W"],
+                    torch.tensor(offsets, dtype=torch.int32, device=device))
+            assert torch.equal(routes.cpu(), want_routes), label
+            assert torch.equal(out.cpu().float(), want_out.float()), label
+    finally:
+        cabi.set_forward_index(None)
