@@ -194,3 +194,25 @@ def test_indexed_forward_over_the_random_sweep_of_shapes(cabi, c_oracle):
             assert torch.equal(out.cpu().float(), want_out.float()), label
     finally:
         cabi.set_forward_index(None)
+
+
+@pytest.mark.parametrize("bits", [8, 12, 30])
+def test_indexed_forward_of_one_long_sequence_equals_the_scan(cabi, bits):
+    # 32 768 tokens: 32 passes of the index build, 4 096 buckets (by hash at 30 bits), and with
+    # 8-bit symbols buckets of 128 routes; a repeated stretch gives runs up to the window
+    device = torch.device("cuda:0")
+    length = 32768
+    query = nonzero_randn((1, length, 2, bits), dtype=torch.float32, seed=bits).to(device)
+    key = nonzero_randn((1, length, 2, bits), dtype=torch.float32, seed=bits + 1).to(device)
+    key[:, 20000:26000] = key[:, 3000:9000]
+    query[:, 20001:26000] = key[:, 20000:25999]
+    value = nonzero_randn((1, length, 1, 8), dtype=torch.float32, seed=3).to(device)
+    cabi.set_forward_index("scan")
+    try:
+        want_output, _, _, want_routes = cabi.hard_forward(query, key, value, 300)
+        cabi.set_forward_index(None)
+        output, _, _, routes = cabi.hard_forward(query, key, value, 300)
+    finally:
+        cabi.set_forward_index(None)
+    assert int((want_routes > 0).sum()) > length // 4
+    assert torch.equal(routes, want_routes) and torch.equal(output, want_output)
