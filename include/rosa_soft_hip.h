@@ -99,8 +99,8 @@ void rosa_hip_set_gradient_piece_rows(int rows);
 
 /*
  * How the hard forward finds its routes: 0 (the default) = through an index of the keys by
- * symbol where the shape has one (symbols of six bits or more, sequences of 512 tokens or
- * more; a row then visits only the routes whose key symbol equals its own, and row blocks
+ * symbol where the shape suits it (symbols of six bits or more, sequences of 512 tokens or
+ * more, in a packed batch on average; a row then visits only the routes whose key symbol equals its own, and row blocks
  * that this does not suit are handed back to the scan over all routes), 1 = always the scan
  * over all routes, 2 = the index with every row block handed back, 3 = the index at every
  * shape (2 and 3 are for tests).  The routes are the same in every mode.  The workspace

@@ -1551,7 +1551,10 @@ int run_forward(const rosa_problem* p, const ProblemView& view, const void* quer
   const uint32_t* pk = reinterpret_cast<const uint32_t*>(packed_key);
   const int index_mode = g_forward_index_mode.load(std::memory_order_relaxed);
   const uint8_t* left_over = nullptr;
-  const bool index_suits = L.D >= kIndexSymbolBitsMin && longest >= kIndexLongestMin;
+  // (a packed batch is judged by its mean sequence length: the host does not know the
+  // lengths, and a block per (sequence, head) costs more than it saves on short sequences)
+  const int typical = L.varlen ? L.N / std::max(L.S, 1) : L.T;
+  const bool index_suits = L.D >= kIndexSymbolBitsMin && typical >= kIndexLongestMin;
   if (w.log_buckets > 0 && (index_mode >= 2 || (index_mode == 0 && index_suits))) {
     KeyIndex index;
     index.bucket_begin = at<int32_t>(workspace, w.bucket_begin);
