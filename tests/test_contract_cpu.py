@@ -235,9 +235,25 @@ def test_c_abi_library_exports_every_declared_symbol():
     problem = cabi.RosaProblem(dtype=0, B=2, T=128, N=256, S=0, H=4, D=8, Hv=2, Dv=8, W=16)
     assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) >= 256 * 4 * 4
     assert loaded.rosa_hip_vjp_workspace_bytes(ctypes.byref(problem), 7, 1.0, 0) > 0
+    # the forward's workspace has room for the index of the keys: the source token of every
+    # row (4 bytes), an entry per row (16) and the bucket offsets (at most 4 per row)
+    rows = 256 * 4
+    assert 20 * rows <= loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) <= 26 * rows + 4096
     problem.D = 33
     assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) == 0
     assert b"[1, 32]" in loaded.rosa_hip_last_error()
+    # the router's workspace: only updates that route a long chunk through the index need one
+    update = cabi.RosaRouterUpdate(S=2, H=4, Hp=2, W=16, qk_bits=8, payload_bits=8, capacity=4096,
+                                   tokens=2 * 700, longest_chunk=700, uniform_chunk=700,
+                                   longest_total=700)
+    size = loaded.rosa_hip_router_workspace_bytes(ctypes.byref(update))
+    assert 8 * 8 * 700 <= size <= 8 * 8 * 700 + 8 * 257 * 4 + 8192
+    for field, value in (("longest_chunk", 8), ("qk_bits", 5), ("longest_total", 500)):
+        other = cabi.RosaRouterUpdate(S=2, H=4, Hp=2, W=16, qk_bits=8, payload_bits=8,
+                                      capacity=4096, tokens=2 * 700, longest_chunk=700,
+                                      uniform_chunk=700, longest_total=700)
+        setattr(other, field, value)
+        assert loaded.rosa_hip_router_workspace_bytes(ctypes.byref(other)) == 0, field
 
 
 def test_backward_workspace_sizes_at_training_shapes():
