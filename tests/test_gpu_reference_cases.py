@@ -1,0 +1,191 @@
+"""Behaviours the reference's own device tests pin, restated against the HIP operators: what the
+backward controls may change (tests/test_soft_cuda.py:666-690), that the dense backward finds a
+useful route by gradient descent (:716-743), the window clamp and the parameter checks
+(:849-885), loss scaling on a float16 tail (tests/test_soft_integration.py:175-216), and, for
+packed sequences, that nothing crosses a sequence boundary and that the first value of a sequence
+is never routed (tests/test_soft_varlen.py:78-147), grouped heads with non-contiguous inputs and
+offsets (:923-955), and the sequence-count limit (:234-254)."""
+
+import math
+
+import pytest
+import torch
+
+from tests.conftest import nonzero_randn
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def rosa():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import rosa_soft_amd
+
+    assert rosa_soft_amd.BUILD_CAPABILITIES.variant == "rocm"
+    return rosa_soft_amd
+
+
+def _gradients(operator, inputs, grad_output, *extra, **controls):
+    leaves = tuple(t.detach().clone().to(DEVICE).requires_grad_() for t in inputs)
+    output = operator(*leaves, *extra, **controls)
+    gradients = torch.autograd.grad(output, leaves, grad_output.to(DEVICE))
+    return output.detach(), gradients
+
+
+def test_backward_controls_change_the_gradients_and_never_the_output(rosa):
+    inputs = (nonzero_randn((1, 10, 2, 5), seed=70), nonzero_randn((1, 10, 2, 5), seed=71),
+              nonzero_randn((1, 10, 1, 3), seed=72))
+    grad_output = nonzero_randn((1, 10, 2, 3), seed=73)
+
+    def run(scale, mismatch_scale):
+        return _gradients(rosa.rosa_soft, inputs, grad_output, max_suffix_length=6, scale=scale,
+                          mismatch_scale=mismatch_scale)
+
+    base_output, base_gradients = run(2.0, 3.0)
+    for output, gradients in (run(0.7, 3.0), run(2.0, 7.0)):
+        assert torch.equal(output, base_output)
+        assert any(not torch.allclose(got, base) for got, base in zip(gradients, base_gradients))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gradient_descent_on_one_query_logit_finds_the_useful_route(rosa, seed):
+    # the last row can only match the first key, whose successor holds the wanted value, if its
+    # one query logit turns positive: the surrogate gradient must push it there within six steps
+    torch.manual_seed(seed)
+    length = 33
+    logit = torch.nn.Parameter(torch.tensor(-0.5, device=DEVICE))
+    optimizer = torch.optim.SGD([logit], lr=1.0)
+    steps = 0
+    for steps in range(1, 13):
+        optimizer.zero_grad(set_to_none=True)
+        query = torch.ones(1, length, 1, 1, device=DEVICE)
+        query[0, -1, 0, 0] = logit
+        key = -torch.ones_like(query)
+        key[:, 0] = 1
+        value = -torch.ones_like(query)
+        value[:, 1] = 1
+        output = rosa.rosa_soft(query, key, value, max_suffix_length=1, scale=2.0, mismatch_scale=3.0)
+        (output[0, -1, 0, 0] - 1).square().backward()
+        optimizer.step()
+        if logit.item() > 0:
+            break
+    assert steps <= 6 and logit.item() > 0
+
+
+def test_a_window_beyond_the_sequence_is_the_whole_sequence_and_must_be_an_integer(rosa):
+    inputs = tuple(t.to(DEVICE) for t in (nonzero_randn((1, 7, 1, 3), seed=110),
+                                          nonzero_randn((1, 7, 1, 3), seed=111),
+                                          nonzero_randn((1, 7, 1, 2), seed=112)))
+    whole = rosa.rosa_soft(*inputs, max_suffix_length=7)
+    huge = rosa.rosa_soft(*inputs, max_suffix_length=10 ** 9)
+    assert torch.equal(whole, huge)
+    for invalid in (True, 1.5):
+        with pytest.raises(TypeError, match="integer"):
+            rosa.rosa_soft(*inputs, max_suffix_length=invalid)
+
+
+@pytest.mark.parametrize("controls,message", [
+    ({"max_suffix_length": 0}, "max_suffix_length"),
+    ({"scale": True}, "scale"),
+    ({"scale": 0.0}, "scale"),
+    ({"scale": 1e-300}, "scale"),
+    ({"scale": 1e300}, "scale"),
+    ({"dropout_p": True}, "dropout_p"),
+    ({"dropout_p": -0.1}, "dropout_p"),
+    ({"dropout_p": 1.0}, "dropout_p"),
+    ({"dropout_p": math.nan}, "dropout_p"),
+    ({"dropout_p": math.inf}, "dropout_p"),
+    ({"mismatch_scale": 0.0}, "mismatch_scale"),
+    ({"mismatch_scale": True}, "mismatch_scale"),
+    ({"mismatch_scale": 1e-300}, "mismatch_scale"),
+    ({"mismatch_scale": 1e300}, "mismatch_scale"),
+])
+def test_controls_outside_their_range_are_rejected_on_the_device_path(rosa, controls, message):
+    tensor = torch.ones(1, 5, 1, 1, device=DEVICE)
+    with pytest.raises(ValueError, match=message):
+        rosa.rosa_soft(tensor, tensor, tensor, **controls)
+
+
+def _final_row_value_gradient(rosa, dtype, loss_scale=1.0):
+    tokens = 40
+    query = torch.ones(1, tokens, 1, 4, device=DEVICE, dtype=dtype, requires_grad=True)
+    key = torch.ones_like(query, requires_grad=True)
+    value = torch.arange(tokens, device=DEVICE, dtype=dtype).reshape(1, tokens, 1, 1).requires_grad_()
+    output = rosa.rosa_soft(query, key, value, max_suffix_length=32)
+    (output[0, -1, 0, 0] * loss_scale).backward()
+    return value.grad.detach().float().flatten() / loss_scale
+
+
+def test_loss_scaling_brings_a_float16_tail_gradient_closer_to_float32(rosa):
+    plain = _final_row_value_gradient(rosa, torch.float16)
+    scaled = _final_row_value_gradient(rosa, torch.float16, loss_scale=1024.0)
+    exact = _final_row_value_gradient(rosa, torch.float32)
+    # position zero is the null value and never receives a route gradient
+    assert torch.count_nonzero(exact[1:]) == exact.numel() - 1
+    assert torch.count_nonzero(scaled[1:]) == scaled.numel() - 1
+    assert torch.linalg.vector_norm(scaled - exact) < torch.linalg.vector_norm(plain - exact)
+
+
+def _offsets(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEVICE)
+
+
+def test_packed_sequences_do_not_see_each_other(rosa):
+    inputs = (nonzero_randn((9, 1, 3), seed=10), nonzero_randn((9, 1, 3), seed=11),
+              nonzero_randn((9, 1, 2), seed=12))
+    grad_output = nonzero_randn((9, 1, 2), seed=13)
+    offsets = _offsets([0, 4, 9])
+
+    def run(tensors):
+        return _gradients(rosa.rosa_soft_varlen, tensors, grad_output, offsets, max_suffix_length=5,
+                          scale=2.0, mismatch_scale=9.0)
+
+    base_output, base_gradients = run(inputs)
+    changed = tuple(t.clone() for t in inputs)
+    for tensor in changed:
+        tensor[:4].mul_(-2.0)
+    changed_output, changed_gradients = run(changed)
+    assert torch.equal(changed_output[4:], base_output[4:])
+    for got, base in zip(changed_gradients, base_gradients):
+        # (the sums of the second sequence are the same terms in an order that the atomics choose)
+        torch.testing.assert_close(got[4:], base[4:], rtol=1e-5, atol=1e-6 * float(base.abs().max()))
+        assert not torch.allclose(got[:4], base[:4])
+
+
+def test_the_first_value_of_a_packed_sequence_is_never_routed(rosa):
+    query = nonzero_randn((7, 1, 2), seed=20).to(DEVICE).requires_grad_()
+    key = nonzero_randn((7, 1, 2), seed=21).to(DEVICE).requires_grad_()
+    value = nonzero_randn((7, 1, 3), seed=22).to(DEVICE).requires_grad_()
+    output = rosa.rosa_soft_varlen(query, key, value, _offsets([0, 1, 4, 7]))
+    output.sum().backward()
+    assert torch.count_nonzero(output[[0, 1, 4]]) == 0
+    assert torch.count_nonzero(value.grad[[0, 1, 4]]) == 0
+
+
+def test_packed_grouped_heads_with_strided_inputs_and_offsets(rosa, c_oracle):
+    total = 11
+    query = nonzero_randn((total, 5, 4), seed=60).to(DEVICE).transpose(1, 2).requires_grad_()
+    key = nonzero_randn((total, 5, 4), seed=61).to(DEVICE).transpose(1, 2).requires_grad_()
+    value = nonzero_randn((total, 3, 2), seed=62).to(DEVICE).transpose(1, 2).requires_grad_()
+    storage = _offsets([0, -1, 4, -1, 11])
+    offsets = storage[::2]
+    assert not offsets.is_contiguous() and not query.is_contiguous()
+    output = rosa.rosa_soft_varlen(query, key, value, offsets, max_suffix_length=6)
+    output.sum().backward()
+    assert output.shape == (total, 4, 3)
+    assert all(t.grad is not None and torch.isfinite(t.grad).all() for t in (query, key, value))
+    want, _ = c_oracle.varlen_hard_forward(query.detach().cpu().contiguous(),
+                                           key.detach().cpu().contiguous(),
+                                           value.detach().cpu().contiguous(), [0, 4, 11], 6)
+    assert torch.equal(output.detach().cpu(), want)
+
+
+def test_more_packed_sequences_than_the_kernels_can_index_are_refused(rosa):
+    query = torch.ones(1, 1, 2, device=DEVICE)
+    value = torch.ones(1, 1, 2, device=DEVICE)
+    offsets = torch.zeros(1, dtype=torch.int32, device=DEVICE).expand(2_147_483_521)
+    with pytest.raises(RuntimeError, match="number of packed sequences is too large"):
+        torch.ops.rosa_soft.hard_forward_varlen(query, query.clone(), value, offsets, 1)
