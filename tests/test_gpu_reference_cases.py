@@ -189,3 +189,79 @@ def test_more_packed_sequences_than_the_kernels_can_index_are_refused(rosa):
     offsets = torch.zeros(1, dtype=torch.int32, device=DEVICE).expand(2_147_483_521)
     with pytest.raises(RuntimeError, match="number of packed sequences is too large"):
         torch.ops.rosa_soft.hard_forward_varlen(query, query.clone(), value, offsets, 1)
+
+
+# The shapes and controls of the reference's device tests that aim at single paths of its
+# kernels (large value widths with only the query gradient, the query-utility cache, key
+# aggregation over 512 and 1 024 rows, a window of one with 64-wide values, dropout, the three
+# dtypes): batch, length, heads, bits, value heads, value width, window, scale, dropout,
+# mismatch scale, gradient mask (1 query, 2 key, 4 value), dtype
+DENSE_SHAPES_OF_THE_REFERENCE = [
+    *[(1, 9, 2, 4, 1, width, 6, 1.4, p, 3.0, 1, torch.float32)   # test_soft_cuda.py:210-264
+      for width in (32, 64, 128) for p in (0.0, 0.2)],
+    (1, 129, 1, 8, 1, 64, 8, 1.4, 0.0, 3.0, 1, torch.float32),    # :267-315
+    *[(1, 512, 1, 8, 1, 8, 32, 1.2, p, 3.0, 2, torch.float32) for p in (0.0, 0.2)],   # :318-366
+    *[(1, 1024, 1, 8, 1, 8, 32, 1.2, p, 3.0, 3, torch.float32) for p in (0.0, 0.2)],
+    *[(1, 67, 2, 8, 1, 64, 1, 1.4, p, 3.0, 4, torch.float32) for p in (0.0, 0.2)],    # :368-420
+    *[(1, 9, 2, 4, 1, 3, 6, 1.5, p, 4.0, 7, torch.float32) for p in (0.1, 0.5)],      # :423-466
+    *[(1, 7, 2, 5, 1, 3, 5, 1.4, 0.0, 2.6, 7, dtype)                                  # :468-509
+      for dtype in (torch.float16, torch.bfloat16)],
+]
+
+
+@pytest.mark.parametrize("case", DENSE_SHAPES_OF_THE_REFERENCE,
+                         ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_dense_shapes_of_the_reference_device_tests(c_oracle, case):
+    from rosa_soft_amd import cabi
+    from tests.test_gpu_parity import assert_gradients_close, make_case, run_device
+
+    batch, length, heads, bits, value_heads, width, window, scale, p, ms, mask, dtype = case
+    query, key, value, grad_output = make_case(batch, length, heads, bits, value_heads, width,
+                                               dtype, seed=length + width)
+    seed = 24680 if p > 0 else None
+    out, _, _, routes, grads = run_device(cabi, query, key, value, grad_output, window, scale, p,
+                                          ms, seed, mask)
+    want_out, want_routes, _ = c_oracle.hard_forward(query, key, value, window)
+    assert torch.equal(routes.cpu(), want_routes) and torch.equal(out.cpu().float(), want_out.float())
+    want = c_oracle.surrogate_vjp(query, key, value, grad_output, max_suffix_length=window,
+                                  scale=scale, dropout_p=p, mismatch_scale=ms, seed=seed)
+    for bit, got, expected, name in zip((1, 2, 4), grads, want, "qkv"):
+        if mask & bit:
+            assert_gradients_close(got, expected, f"d{name}")
+
+
+# lengths, heads, bits, value width, window, scale, dropout, mismatch scale
+PACKED_SHAPES_OF_THE_REFERENCE = [
+    *[((3, 0, 5, 2), 2, 3, 2, 4, 1.3, p, 7.0) for p in (0.0, 0.2)],   # test_soft_varlen.py:396-480
+    *[((256,), 1, 8, 3, 4, 1.2, p, 3.0) for p in (0.0, 0.2)],          # :482-560
+    ((256,), 1, 8, 64, 4, 1.2, 0.2, 3.0),                              # :562-640
+    ((257,), 2, 8, 3, 9, 1.4, 0.2, 3.0),                               # :642-713
+    ((1027,), 1, 4, 1, 2, 1.4, 0.2, 3.0),                              # :715-786
+    *[((67,), 2, 8, 64, 9, 1.2, p, 3.0) for p in (0.0, 0.2)],          # :788-862
+]
+
+
+@pytest.mark.parametrize("case", PACKED_SHAPES_OF_THE_REFERENCE, ids=lambda c: str(c))
+def test_packed_shapes_of_the_reference_device_tests(c_oracle, case):
+    import numpy as np
+
+    from rosa_soft_amd import cabi
+    from tests.test_gpu_parity import assert_gradients_close, run_device
+
+    lengths, heads, bits, width, window, scale, p, ms = case
+    offsets = [0, *np.cumsum(lengths).tolist()]
+    total = offsets[-1]
+    query = nonzero_randn((total, heads, bits), seed=40)
+    key = nonzero_randn((total, heads, bits), seed=41)
+    value = nonzero_randn((total, 1, width), seed=42)
+    grad_output = nonzero_randn((total, heads, width), seed=43, floor=0.0)
+    seed = 13579 if p > 0 else None
+    out, _, _, routes, grads = run_device(cabi, query, key, value, grad_output, window, scale, p,
+                                          ms, seed, 7, offsets)
+    want_out, want_routes = c_oracle.varlen_hard_forward(query, key, value, offsets, window)
+    assert torch.equal(routes.cpu(), want_routes) and torch.equal(out.cpu().float(), want_out.float())
+    want = c_oracle.varlen_surrogate_vjp(query, key, value, offsets, grad_output,
+                                         max_suffix_length=window, scale=scale, dropout_p=p,
+                                         mismatch_scale=ms, seed=seed)
+    for got, expected, name in zip(grads, want, "qkv"):
+        assert_gradients_close(got, expected, f"d{name}")
