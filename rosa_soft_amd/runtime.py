@@ -277,10 +277,9 @@ class RosaRuntime:
 
     # ------------------------------------------------------------------ statistics
 
-    @property
     def stats(self) -> Tuple[int, int, int]:
-        """Stored key, query and payload symbols (the reference counts automaton states,
-        edges and payload symbols; the third entry means the same thing)."""
+        """Stored key, query and payload symbols (rosa_soft/runtime.py:552-555 counts automaton
+        states, edges and payload symbols; the third entry means the same thing)."""
 
         self._require_open()
         tokens = sum(self._lengths)
@@ -293,6 +292,12 @@ class RosaRuntime:
         logical = tokens * (2 * self._num_heads + self._num_payload_heads)
         slots = max(self._slot_count, 0)
         return {
+            # the reference's names (rosa_soft/runtime.py:557-576); its states and edges belong
+            # to suffix automata, which this runtime does not build: the stored key and query
+            # symbols stand in their place, as in stats()
+            "states": tokens * self._num_heads,
+            "edges": tokens * self._num_heads,
+            "automata": slots * self._num_heads,
             "key_symbols": tokens * self._num_heads,
             "query_symbols": tokens * self._num_heads,
             "payload_symbols": tokens * self._num_payload_heads,

@@ -45,7 +45,7 @@ def test_packed_dense_matches_oracle(rosa, horizon):
     want = expect_dense(query, key, payload, bits, bits, horizon)
     with rosa.RosaRuntime(heads, payload_heads, bits, bits, horizon) as runtime:
         got = runtime.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
-        stats = runtime.stats
+        stats = runtime.stats()
     assert got[0].dtype == torch.uint8 and got[1].dtype == torch.int64
     assert got[0].device.type == "cuda"
     assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[1].cpu(), want[1])
@@ -165,7 +165,7 @@ def test_lifecycle_slot_and_sequence_id_checks(rosa):
     with pytest.raises(ValueError, match="must be unique"):
         runtime.update_packed(symbols, symbols, symbols, sequence_ids=[7, 7])
     runtime.reset()
-    assert runtime.stats == (0, 0, 0)
+    assert runtime.stats() == (0, 0, 0)
     runtime.update_packed(symbols[:1], symbols[:1], symbols[:1])
     with pytest.raises(RuntimeError, match="slot count is fixed"):
         runtime.update_packed(symbols, symbols, symbols)
@@ -417,3 +417,140 @@ def test_ragged_long_chunks_route_through_the_index_of_the_keys(rosa):
                 assert torch.equal(output[rows].cpu(), want[0][0, done[slot]:done[slot] + step[slot]])
                 assert torch.equal(ends[rows].cpu(), want[1][0, done[slot]:done[slot] + step[slot]])
                 done[slot] += step[slot]
+
+
+# --------------------------------------------------------------------------- the reference's
+# interface tests (tests/test_runtime.py:344-1008) restated for the device runtime
+
+def test_packed_inputs_ignore_bits_above_the_declared_width(rosa):
+    generator = torch.Generator().manual_seed(19)
+    query = torch.randint(0, 2, (2, 32, 3), dtype=torch.uint8, generator=generator)
+    key = torch.randint(0, 2, query.shape, dtype=torch.uint8, generator=generator)
+    payload = torch.randint(0, 4, (2, 32, 1), dtype=torch.uint8, generator=generator)
+    query_high = torch.randint(0, 128, query.shape, dtype=torch.uint8, generator=generator).mul_(2)
+    key_high = torch.randint(0, 128, key.shape, dtype=torch.uint8, generator=generator).mul_(2)
+    payload_high = torch.randint(0, 64, payload.shape, dtype=torch.uint8, generator=generator).mul_(4)
+    with rosa.RosaRuntime(3, 1, 1, 2, 5) as canonical:
+        want = canonical.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
+    with rosa.RosaRuntime(3, 1, 1, 2, 5) as noisy:
+        got = noisy.update_packed((query | query_high).to(DEVICE), (key | key_high).to(DEVICE),
+                                  (payload | payload_high).to(DEVICE))
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_grouped_payload_history_is_stored_once_per_payload_head(rosa):
+    batch, tokens, heads, payload_heads = 3, 7, 6, 2
+    query = random_packed((batch, tokens, heads), 2, 32)
+    key = random_packed((batch, tokens, heads), 2, 33)
+    payload = random_packed((batch, tokens, payload_heads), 3, 34)
+    with rosa.RosaRuntime(heads, payload_heads, 2, 3, 4) as runtime:
+        got = runtime.update_packed(query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE))
+        stats = runtime.stats()
+        detailed = runtime.memory_stats()
+    want = expect_dense(query, key, payload, 2, 3, 4)
+    assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[1].cpu(), want[1])
+    assert stats[2] == batch * tokens * payload_heads
+    assert detailed["payload_symbols"] == stats[2]
+    assert detailed["automata"] == batch * heads and detailed["sequences"] == batch
+
+
+def test_long_chunked_history_preserves_global_successor_positions(rosa):
+    # one symbol throughout: every row matches the key before it as far as the horizon reaches,
+    # and the latest route wins, so row t answers with the payload at t and the end position t - 1
+    chunk_tokens, heads = 16_384, 2
+    query = torch.zeros(1, chunk_tokens, heads, dtype=torch.uint8, device=DEVICE)
+    key = torch.zeros_like(query)
+    payload = (torch.arange(chunk_tokens * 2, dtype=torch.int64).remainder(2).to(torch.uint8)
+               .view(1, chunk_tokens * 2, 1).to(DEVICE))
+    with rosa.RosaRuntime(heads, 1, qk_bits=1, payload_bits=1, max_suffix_length=32) as runtime:
+        first = runtime.update_packed(query, key, payload[:, :chunk_tokens])
+        second = runtime.update_packed(query, key, payload[:, chunk_tokens:])
+        stats = runtime.memory_stats()
+    output = torch.cat((first[0], second[0]), dim=1)
+    ends = torch.cat((first[1], second[1]), dim=1)
+    want_output = payload.expand(-1, -1, heads).clone()
+    want_output[:, 0] = 0
+    want_ends = (torch.arange(chunk_tokens * 2, dtype=torch.int64, device=DEVICE) - 1
+                 ).view(1, -1, 1).expand(-1, -1, heads)
+    assert torch.equal(output, want_output) and torch.equal(ends, want_ends)
+    assert stats["payload_symbols"] == chunk_tokens * 2
+    assert stats["sequences"] == 1 and stats["automata"] == heads
+
+
+def test_constructor_names_and_read_only_configuration(rosa):
+    import inspect
+
+    parameters = inspect.signature(rosa.RosaRuntime).parameters
+    assert tuple(parameters)[:5] == (
+        "num_heads", "num_payload_heads", "qk_bits", "payload_bits", "max_suffix_length")
+    # (what this runtime adds, the device of its histories, is optional)
+    assert all(p.default is not inspect.Parameter.empty for p in list(parameters.values())[5:])
+    expected = dict(num_heads=4, num_payload_heads=2, qk_bits=3, payload_bits=5, max_suffix_length=7)
+    runtime = rosa.RosaRuntime(**expected)
+    try:
+        for name, value in expected.items():
+            assert getattr(runtime, name) == value
+            with pytest.raises(AttributeError):
+                setattr(runtime, name, value + 1)
+            assert getattr(runtime, name) == value
+    finally:
+        runtime.close()
+
+
+def test_closed_runtime_rejects_statistics_and_updates(rosa):
+    runtime = rosa.RosaRuntime(1, 1, 1, 1, 1)
+    runtime.close()
+    runtime.close()
+    packed = torch.zeros(1, 1, 1, dtype=torch.uint8, device=DEVICE)
+    with pytest.raises(RuntimeError, match="closed"):
+        runtime.stats()
+    with pytest.raises(RuntimeError, match="closed"):
+        runtime.update_packed(packed, packed, packed)
+
+
+def test_empty_dense_update_and_empty_batches(rosa):
+    packed = torch.empty(2, 0, 1, dtype=torch.uint8, device=DEVICE)
+    with rosa.RosaRuntime(1, 1, 1, 1, 3) as runtime:
+        output, ends = runtime.update_packed(packed, packed, packed)
+        assert runtime.stats()[2] == 0
+    assert output.shape == (2, 0, 1) and ends.shape == (2, 0, 1)
+    none = torch.empty(0, 3, 1, dtype=torch.uint8, device=DEVICE)
+    varlen = torch.empty(0, 1, dtype=torch.uint8, device=DEVICE)
+    with rosa.RosaRuntime(1, 1, 1, 1, 2) as runtime:
+        with pytest.raises(ValueError, match="batch"):
+            runtime.update_packed(none, none, none)
+        with pytest.raises(ValueError, match="at least one sequence"):
+            runtime.update_packed(varlen, varlen, varlen, cu_seqlens=torch.tensor([0]))
+
+
+@pytest.mark.parametrize("name,args", [
+    ("num_heads", (1.5,)),
+    ("qk_bits", (1, None, True)),
+    ("max_suffix_length", (1, None, 1, 1, False)),
+])
+def test_constructor_rejects_values_that_are_not_integers(rosa, name, args):
+    with pytest.raises(TypeError, match=name):
+        rosa.RosaRuntime(*args)
+
+
+@pytest.mark.parametrize("qk_bits,payload_bits", [(0, 1), (9, 1), (1, 0), (1, 9)])
+def test_symbol_widths_are_limited_to_one_through_eight(rosa, qk_bits, payload_bits):
+    with pytest.raises(ValueError, match=r"in \[1, 8\]"):
+        rosa.RosaRuntime(1, 1, qk_bits, payload_bits, 1)
+
+
+def test_update_on_a_side_stream_matches_blocking_and_snapshots_its_inputs(rosa):
+    query = random_packed((1, 32, 2), 3, 20).to(DEVICE)
+    key = random_packed((1, 32, 2), 3, 21).to(DEVICE)
+    payload = random_packed((1, 32, 1), 3, 22).to(DEVICE)
+    with rosa.RosaRuntime(2, 1, 3, 3, 4) as blocking:
+        want = blocking.update_packed(query, key, payload)
+    stream = torch.cuda.Stream()
+    with rosa.RosaRuntime(2, 1, 3, 3, 4) as asynchronous:
+        work = asynchronous.update_packed(query, key, payload, stream=stream, async_op=True)
+        # the caller may reuse its tensors as soon as the call returns
+        query.fill_(7)
+        key.zero_()
+        payload.fill_(6)
+        got = work.wait()
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
