@@ -265,3 +265,71 @@ def test_packed_shapes_of_the_reference_device_tests(c_oracle, case):
                                          mismatch_scale=ms, seed=seed)
     for got, expected, name in zip(grads, want, "qkv"):
         assert_gradients_close(got, expected, f"d{name}")
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_mixed_precision_projections_and_a_gradient_scaler(rosa, varlen):
+    # tests/test_soft_integration.py:15-90: float16 logits out of autocast projections, dropout,
+    # a scaled loss, finite parameter gradients, an optimizer step
+    torch.manual_seed(3)
+    width, heads, bits, value_width, tokens = 6, 2, 3, 2, 9
+    projections = [torch.nn.Linear(width, n, device=DEVICE)
+                   for n in (heads * bits, heads * bits, value_width)]
+    parameters = [p for layer in projections for p in layer.parameters()]
+    optimizer = torch.optim.SGD(parameters, lr=0.01)
+    scaler = torch.amp.GradScaler("cuda", init_scale=128.0)
+    source = torch.randn(tokens, width, device=DEVICE)
+    optimizer.zero_grad(set_to_none=True)
+    with torch.autocast("cuda", dtype=torch.float16):
+        query = projections[0](source).reshape(tokens, heads, bits)
+        key = projections[1](source).reshape(tokens, heads, bits)
+        value = projections[2](source).reshape(tokens, 1, value_width)
+        if varlen:
+            output = rosa.rosa_soft_varlen(query, key, value, _offsets([0, 4, tokens]),
+                                           max_suffix_length=5, dropout_p=0.1)
+        else:
+            output = rosa.rosa_soft(query.unsqueeze(0), key.unsqueeze(0), value.unsqueeze(0),
+                                    max_suffix_length=5, dropout_p=0.1)
+        loss = output.float().square().mean()
+    assert query.dtype == torch.float16 and output.dtype == torch.float16
+    scaler.scale(loss).backward()
+    scaler.unscale_(optimizer)
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in parameters)
+    before = [p.detach().clone() for p in parameters]
+    scaler.step(optimizer)
+    scaler.update()
+    assert any(not torch.equal(p, old) for p, old in zip(parameters, before))
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("dropout_p", [0.0, 0.2])
+def test_activation_checkpointing_replays_the_same_outputs_and_gradients(rosa, varlen, dropout_p):
+    # tests/test_soft_integration.py:93-172: the recomputed forward draws the same dropout seed
+    from torch.utils.checkpoint import checkpoint
+
+    generator = torch.Generator(device=DEVICE).manual_seed(100)
+    inputs = (torch.randn(9, 1, 3, generator=generator, device=DEVICE),
+              torch.randn(9, 1, 3, generator=generator, device=DEVICE),
+              torch.randn(9, 1, 2, generator=generator, device=DEVICE))
+    offsets = _offsets([0, 4, 9])
+
+    def operator(*tensors):
+        if varlen:
+            return rosa.rosa_soft_varlen(*tensors, offsets, max_suffix_length=5, dropout_p=dropout_p)
+        return rosa.rosa_soft(*(t.unsqueeze(0) for t in tensors), max_suffix_length=5,
+                              dropout_p=dropout_p).squeeze(0)
+
+    def run(use_checkpoint):
+        torch.cuda.manual_seed(101)
+        leaves = tuple(t.detach().clone().requires_grad_() for t in inputs)
+        if use_checkpoint:
+            output = checkpoint(operator, *leaves, use_reentrant=False, preserve_rng_state=True)
+        else:
+            output = operator(*leaves)
+        return output.detach(), torch.autograd.grad(output.sum(), leaves)
+
+    direct_output, direct_gradients = run(False)
+    replayed_output, replayed_gradients = run(True)
+    assert torch.equal(replayed_output, direct_output)
+    for replayed, direct in zip(replayed_gradients, direct_gradients):
+        torch.testing.assert_close(replayed, direct, rtol=2e-5, atol=2e-6)
