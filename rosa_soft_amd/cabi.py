@@ -586,7 +586,9 @@ def router_update(update: RosaRouterUpdate, device: torch.device) -> Optional[Te
 
     workspace = None
     with torch.cuda.device(device):
-        size = int(load().rosa_hip_router_workspace_bytes(ctypes.byref(update)))
+        # (chunks of up to 8 tokens never use a workspace: decoding steps skip the query)
+        size = (int(load().rosa_hip_router_workspace_bytes(ctypes.byref(update)))
+                if update.longest_chunk > 8 else 0)
         if size > 0:
             workspace = torch.empty(size, dtype=torch.uint8, device=device)
             update.workspace = workspace.data_ptr()
