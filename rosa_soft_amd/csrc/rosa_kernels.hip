@@ -1323,6 +1323,7 @@ struct ForwardWorkspace {
 // at every shape, so that the choice can be made per launch.
 constexpr int kIndexSymbolBitsMin = 6;
 constexpr int kIndexLongestMin = 512;
+constexpr int64_t kIndexRowsMax = int64_t(1) << 26;
 
 ForwardWorkspace carve_forward(const ProblemView& v, bool with_index = true) {
   ForwardWorkspace w;
@@ -1336,7 +1337,8 @@ ForwardWorkspace carve_forward(const ProblemView& v, bool with_index = true) {
   w.log_buckets = 0; w.hashed = 0;
   w.bucket_begin = w.entries = w.unit_scan = w.left_over = 0;
   const int longest = v.L.varlen ? v.L.N : v.L.T;
-  if (with_index) {
+  // (beyond 64 M rows, 1.5 GiB of index, the forward keeps to the scan and its 4 bytes per row)
+  if (with_index && v.symbol_rows <= kIndexRowsMax) {
     // about four keys per bucket on the longest sequence, at most one bucket per symbol
     int log_buckets = 6;
     while (log_buckets < 12 && (4 << log_buckets) < longest) ++log_buckets;

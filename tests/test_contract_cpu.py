@@ -239,6 +239,9 @@ def test_c_abi_library_exports_every_declared_symbol():
     # row (4 bytes), an entry per row (16) and the bucket offsets (at most 4 per row)
     rows = 256 * 4
     assert 20 * rows <= loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) <= 26 * rows + 4096
+    # beyond 64 M rows the workspace holds no index: 4 bytes per row and the tables
+    huge = cabi.RosaProblem(dtype=0, B=1, T=1 << 21, N=1 << 21, S=0, H=64, D=8, Hv=2, Dv=8, W=16)
+    assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(huge)) <= 4 * (1 << 27) + 4096
     problem.D = 33
     assert loaded.rosa_hip_forward_workspace_bytes(ctypes.byref(problem)) == 0
     assert b"[1, 32]" in loaded.rosa_hip_last_error()
