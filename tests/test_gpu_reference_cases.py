@@ -333,3 +333,57 @@ def test_activation_checkpointing_replays_the_same_outputs_and_gradients(rosa, v
     assert torch.equal(replayed_output, direct_output)
     for replayed, direct in zip(replayed_gradients, direct_gradients):
         torch.testing.assert_close(replayed, direct, rtol=2e-5, atol=2e-6)
+
+
+def test_training_without_dropout_draws_nothing_from_the_generator_and_repeats(rosa):
+    # tests/test_soft_cuda.py:745-769
+    inputs = (nonzero_randn((1, 8, 2, 4), seed=90), nonzero_randn((1, 8, 2, 4), seed=91),
+              nonzero_randn((1, 8, 1, 3), seed=92))
+    grad_output = nonzero_randn((1, 8, 2, 3), seed=93)
+    state = torch.cuda.get_rng_state()
+    first = _gradients(rosa.rosa_soft, inputs, grad_output, max_suffix_length=5)
+    assert torch.equal(state, torch.cuda.get_rng_state())
+    torch.cuda.manual_seed(123456)
+    second = _gradients(rosa.rosa_soft, inputs, grad_output, max_suffix_length=5)
+    assert torch.equal(first[0], second[0])
+    for left, right in zip(first[1], second[1]):
+        torch.testing.assert_close(left, right, rtol=2e-6, atol=2e-7)
+
+
+def test_dropout_is_seeded_by_the_generator_and_touches_only_the_backward(rosa):
+    # tests/test_soft_cuda.py:772-810
+    inputs = (nonzero_randn((1, 8, 2, 4), seed=94), nonzero_randn((1, 8, 2, 4), seed=95),
+              nonzero_randn((1, 8, 1, 3), seed=96))
+    grad_output = nonzero_randn((1, 8, 2, 3), seed=97)
+
+    def run(seed):
+        torch.cuda.manual_seed(seed)
+        return _gradients(rosa.rosa_soft, inputs, grad_output, max_suffix_length=5, dropout_p=0.5)
+
+    first, replay, changed = run(98), run(98), run(99)
+    assert torch.equal(first[0], replay[0]) and torch.equal(first[0], changed[0])
+    for want, got in zip(first[1], replay[1]):
+        torch.testing.assert_close(want, got, rtol=2e-6, atol=2e-7)
+    assert any(not torch.allclose(want, got) for want, got in zip(first[1], changed[1]))
+    state = torch.cuda.get_rng_state()
+    with torch.no_grad():
+        rosa.rosa_soft(*(t.to(DEVICE) for t in inputs), dropout_p=0.5)
+    assert torch.equal(state, torch.cuda.get_rng_state())
+
+
+def test_strided_inputs_and_a_sequence_of_one_token(rosa):
+    # tests/test_soft_cuda.py:813-846
+    query = nonzero_randn((2, 3, 9, 4), seed=100).to(DEVICE).transpose(1, 2)
+    key = nonzero_randn((2, 3, 9, 4), seed=101).to(DEVICE).transpose(1, 2)
+    value = nonzero_randn((2, 1, 9, 5), seed=102).to(DEVICE).transpose(1, 2)
+    leaves = tuple(t.requires_grad_() for t in (query, key, value))
+    output = rosa.rosa_soft(*leaves, max_suffix_length=7)
+    output.backward(torch.randn_like(output))
+    assert output.shape == (2, 9, 3, 5)
+    assert all(t.grad is not None and torch.isfinite(t.grad).all() for t in leaves)
+    single = tuple(torch.ones(2, 1, heads, width, device=DEVICE, requires_grad=True)
+                   for heads, width in ((2, 3), (2, 3), (1, 4)))
+    single_output = rosa.rosa_soft(*single)
+    gradients = torch.autograd.grad(single_output.sum(), single)
+    assert torch.equal(single_output, torch.zeros_like(single_output))
+    assert all(torch.equal(g, torch.zeros_like(g)) for g in gradients)
