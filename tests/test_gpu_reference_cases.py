@@ -387,3 +387,46 @@ def test_strided_inputs_and_a_sequence_of_one_token(rosa):
     gradients = torch.autograd.grad(single_output.sum(), single)
     assert torch.equal(single_output, torch.zeros_like(single_output))
     assert all(torch.equal(g, torch.zeros_like(g)) for g in gradients)
+
+
+def _oracle_gradients(inputs, grad_output, **controls):
+    from oracle.rosa_oracle import rosa_soft_oracle
+
+    leaves = tuple(t.detach().clone().cpu().requires_grad_() for t in inputs)
+    output = rosa_soft_oracle(*leaves, **controls)
+    return output.detach(), torch.autograd.grad(output, leaves, grad_output.cpu())
+
+
+def test_non_finite_logits_follow_the_policy_of_the_oracle(rosa):
+    # tests/test_soft_cuda.py:570-611: infinities and a NaN among the logits and values; the
+    # output is the oracle's, the gradients are NaN where the oracle's are and close elsewhere
+    inf, nan = math.inf, math.nan
+    query = torch.tensor([[[[inf, -0.5]], [[0.4, -inf]], [[nan, -1.0]]]])
+    key = torch.tensor([[[[-1.0, inf]], [[-inf, -0.7]], [[0.2, 0.3]]]])
+    value = torch.tensor([[[[inf, -1.0]], [[-inf, 0.2]], [[0.5, -0.4]]]])
+    grad_output = nonzero_randn((1, 3, 1, 2), seed=60)
+    controls = dict(max_suffix_length=3, scale=1.0, mismatch_scale=3.0)
+    want, want_gradients = _oracle_gradients((query, key, value), grad_output, **controls)
+    got, got_gradients = _gradients(rosa.rosa_soft, (query, key, value), grad_output, **controls)
+    assert torch.equal(got.cpu(), want)
+    for observed, reference in zip(got_gradients, want_gradients):
+        observed = observed.cpu()
+        assert torch.equal(torch.isnan(observed), torch.isnan(reference))
+        finite = torch.isfinite(observed) & torch.isfinite(reference)
+        torch.testing.assert_close(observed[finite], reference[finite], rtol=2e-5, atol=2e-6)
+
+
+def test_softsign_jacobian_from_tiny_to_saturated_logits(rosa):
+    # tests/test_soft_cuda.py:614-663: magnitudes from 1e-6 to 1e8 in every position
+    magnitudes = torch.tensor([1e-6, -1e-3, 0.2, -1.0, 10.0, -100.0, 1e4, -1e8])
+    length = magnitudes.numel()
+    query = torch.stack([magnitudes.roll(i) for i in range(length)]).reshape(1, length, 1, -1)
+    key = torch.stack([magnitudes.flip(0).roll(i) for i in range(length)]).reshape_as(query)
+    value = torch.stack([magnitudes[:5].roll(i) for i in range(length)]).reshape(1, length, 1, 5)
+    grad_output = torch.stack([(magnitudes[:5].abs() + 1e-4).roll(-i)
+                               for i in range(length)]).reshape_as(value)
+    controls = dict(max_suffix_length=7, scale=1.7, mismatch_scale=3.0)
+    _, want_gradients = _oracle_gradients((query, key, value), grad_output, **controls)
+    _, got_gradients = _gradients(rosa.rosa_soft, (query, key, value), grad_output, **controls)
+    for observed, reference in zip(got_gradients, want_gradients):
+        torch.testing.assert_close(observed.cpu(), reference, rtol=4e-5, atol=3e-6)
