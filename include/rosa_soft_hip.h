@@ -293,8 +293,9 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
  * length + chunk length of any slot, and `workspace_bytes` at least
  * rosa_hip_router_workspace_bytes(update), which is 0 for updates that would not use it
  * (symbols below six bits, chunks of up to 8 tokens, histories below 512 tokens).  With
- * `workspace` NULL every route is scanned.  The workspace carries nothing from one update to
- * the next.
+ * `workspace` NULL every route is scanned.  A run that is longer than `longest_total` says
+ * finds no room in the index and is scanned as well.  The workspace carries nothing from one
+ * update to the next.
  */
 typedef struct rosa_router_update {
   int32_t S, H, Hp, W;

@@ -2024,6 +2024,12 @@ __global__ __launch_bounds__(kIndexThreads) void router_index_kernel(RouterUpdat
   const int buckets = 1 << U.log_buckets;
   const uint8_t* k = U.key_history + static_cast<int64_t>(run) * U.capacity;
   const int thread = threadIdx.x;
+  if (count > U.index_stride) {
+    // the caller's longest_total was too small for this run: no room for its routes, the scan
+    // takes it
+    if (thread == 0) U.run_scan[run] = 1;
+    return;
+  }
   if (thread < 256) cursor[thread] = 0;
   if (thread == 0) largest = 0;
   __syncthreads();

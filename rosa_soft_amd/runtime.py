@@ -338,8 +338,12 @@ class RosaRuntime:
         self._slot_count = len(self._lengths)
         stored = state_dict["key_history"].size(-1)
         self._grow(max(stored, 1))
-        for name in ("query_history", "key_history", "payload_history"):
-            getattr(self, "_" + name)[..., :stored] = state_dict[name].to(self._device)
+        # (the kernels rely on stored symbols within their declared width, as updates store them)
+        widths = {"query_history": self._qk_bits, "key_history": self._qk_bits,
+                  "payload_history": self._payload_bits}
+        for name, bits in widths.items():
+            symbols = state_dict[name].to(self._device)
+            getattr(self, "_" + name)[..., :stored] = symbols & ((1 << bits) - 1)
 
     # ------------------------------------------------------------------ updates
 

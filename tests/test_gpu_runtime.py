@@ -554,3 +554,69 @@ def test_update_on_a_side_stream_matches_blocking_and_snapshots_its_inputs(rosa)
         payload.fill_(6)
         got = work.wait()
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_router_update_with_an_understated_longest_total_falls_back_to_the_scan(rosa):
+    # the C ABI takes the longest history + chunk length from the caller; a run that is longer
+    # than stated has no room in the index and must be routed by the scan, not out of bounds
+    import ctypes
+
+    from rosa_soft_amd import cabi
+
+    tokens, capacity = 600, 1024
+    query = random_packed((tokens, 1), 8, 5).to(DEVICE)
+    key = random_packed((tokens, 1), 8, 6).to(DEVICE)
+    key[300:500] = key[20:220]
+    query[301:500] = key[300:499]
+    payload = random_packed((tokens, 1), 8, 7).to(DEVICE)
+
+    def run(longest_total, mode):
+        lengths = torch.zeros(1, dtype=torch.int32, device=DEVICE)
+        histories = [torch.zeros(1, 1, capacity, dtype=torch.uint8, device=DEVICE) for _ in range(3)]
+        output = torch.empty(tokens, 1, dtype=torch.uint8, device=DEVICE)
+        ends = torch.empty(tokens, 1, dtype=torch.int64, device=DEVICE)
+        update = cabi.RosaRouterUpdate(
+            S=1, H=1, Hp=1, W=64, qk_bits=8, payload_bits=8, capacity=capacity, tokens=tokens,
+            longest_chunk=tokens, uniform_chunk=tokens, longest_total=longest_total)
+        update.history_lengths = lengths.data_ptr()
+        update.query_history, update.key_history, update.payload_history = (
+            h.data_ptr() for h in histories)
+        update.query, update.key, update.payload = query.data_ptr(), key.data_ptr(), payload.data_ptr()
+        update.output, update.matched_key_end = output.data_ptr(), ends.data_ptr()
+        cabi.set_forward_index(mode)
+        try:
+            workspace = cabi.router_update(update, torch.device(DEVICE))
+        finally:
+            cabi.set_forward_index(None)
+        torch.cuda.synchronize()
+        return output, ends, workspace
+
+    want_output, want_ends, _ = run(tokens, "scan")
+    assert int((want_ends >= 0).sum()) > 200
+    for stated in (tokens, 512):
+        output, ends, workspace = run(stated, None)
+        assert workspace is not None
+        assert torch.equal(output, want_output) and torch.equal(ends, want_ends), stated
+
+
+def test_loaded_state_is_reduced_to_the_declared_symbol_widths(rosa):
+    # a state dictionary with bits above the widths (written by hand, or damaged) must behave
+    # like the same state without them: long chunks then go through the index of the keys,
+    # which buckets stored symbols by their value
+    heads, bits, horizon, tokens = 2, 6, 9, 700
+    query = random_packed((1, 2 * tokens, heads), bits, 41)
+    key = random_packed((1, 2 * tokens, heads), bits, 42)
+    payload = random_packed((1, 2 * tokens, 1), bits, 43)
+    want = expect_dense(query, key, payload, bits, bits, horizon)
+    with rosa.RosaRuntime(heads, 1, bits, bits, horizon) as first:
+        first.update_packed(query[:, :tokens].to(DEVICE), key[:, :tokens].to(DEVICE),
+                            payload[:, :tokens].to(DEVICE))
+        saved = first.state_dict()
+    for name in ("query_history", "key_history", "payload_history"):
+        saved[name] = saved[name] | 0xC0
+    with rosa.RosaRuntime(heads, 1, bits, bits, horizon) as second:
+        second.load_state_dict(saved)
+        output, ends = second.update_packed(query[:, tokens:].to(DEVICE), key[:, tokens:].to(DEVICE),
+                                            payload[:, tokens:].to(DEVICE))
+    assert torch.equal(ends.cpu(), want[1][:, tokens:])
+    assert torch.equal(output.cpu(), want[0][:, tokens:])
