@@ -9,6 +9,7 @@ fails loudly when the library has not been built: there is no CPU fallback.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 from typing import Optional, Sequence, Tuple
@@ -585,7 +586,10 @@ def router_update(update: RosaRouterUpdate, device: torch.device) -> Optional[Te
     """
 
     workspace = None
-    with torch.cuda.device(device):
+    # (the device guard costs a decoding step several microseconds: only where it changes anything)
+    guard = (torch.cuda.device(device) if torch.cuda.current_device() != device.index
+             else contextlib.nullcontext())
+    with guard:
         # (chunks of up to 8 tokens never use a workspace: decoding steps skip the query)
         size = (int(load().rosa_hip_router_workspace_bytes(ctypes.byref(update)))
                 if update.longest_chunk > 8 else 0)

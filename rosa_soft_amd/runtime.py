@@ -253,6 +253,7 @@ class RosaRuntime:
         self._key_history: Optional[Tensor] = None      # [S, H, capacity] uint8
         self._payload_history: Optional[Tensor] = None  # [S, Hp, capacity] uint8
         self._last_update = None            # event recorded after the latest update's launches
+        self._last_stream = None            # ... and the stream they went to
 
     def _require_open(self) -> None:
         if self._state != "OPEN":
@@ -417,7 +418,7 @@ class RosaRuntime:
             # runtime does the same): this one starts after the previous one has finished
             # with the histories, including a growth copy.
             working_stream = torch.cuda.current_stream(self._device)
-            if self._last_update is not None:
+            if self._last_update is not None and working_stream != self._last_stream:
                 working_stream.wait_event(self._last_update)
             output, ends = self._route(
                 query.to(self._device), key.to(self._device), payload.to(self._device), offsets
@@ -431,8 +432,12 @@ class RosaRuntime:
                     ends.unsqueeze(-1) >= 0, unpacked,
                     torch.zeros((), dtype=output_dtype, device=self._device),
                 )
-            self._last_update = torch.cuda.Event()
+            # (one event, recorded anew by every update; an update on the stream of the one
+            # before it is ordered by the stream itself)
+            if self._last_update is None:
+                self._last_update = torch.cuda.Event()
             self._last_update.record(working_stream)
+            self._last_stream = working_stream
             if caller_device != self._device:
                 output, ends = output.to(caller_device), ends.to(caller_device)
             if run_stream is not None:
