@@ -296,6 +296,10 @@ int rosa_hip_surrogate_vjp(const rosa_problem* problem, const void* query,
  * `workspace` NULL every route is scanned.  A run that is longer than `longest_total` says
  * finds no room in the index and is scanned as well.  The workspace carries nothing from one
  * update to the next.
+ * `history_lengths_out` [S] (optional, another array than `history_lengths`): the advanced
+ * lengths are written there and `history_lengths` is left as it was; the caller passes that
+ * array as `history_lengths` of the next update.  A decoding step (chunks of up to 8 tokens)
+ * is then a single kernel launch, because no wave has to wait for the lengths to change.
  */
 typedef struct rosa_router_update {
   int32_t S, H, Hp, W;
@@ -317,6 +321,7 @@ typedef struct rosa_router_update {
   int32_t longest_total;
   void* workspace;
   size_t workspace_bytes;
+  int32_t* history_lengths_out;
 } rosa_router_update;
 
 size_t rosa_hip_router_workspace_bytes(const rosa_router_update* update);

@@ -99,6 +99,7 @@ class RosaRouterUpdate(ctypes.Structure):
         ("longest_total", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_size_t),
+        ("history_lengths_out", ctypes.c_void_p),
     ]
 
 

@@ -1920,6 +1920,7 @@ struct RouterUpdate {
   const int32_t* chunk_offsets;  // [S + 1] token offsets of the chunk per slot, or NULL:
   int uniform_chunk;             //   then every slot brings this many tokens
   int32_t* history_lengths;      // [S] tokens a slot held before this chunk (advanced at the end)
+  int32_t* history_lengths_out;  // [S] or NULL: where the advanced lengths go instead
   uint8_t* query_history;        // [S][H][capacity]
   uint8_t* key_history;          // [S][H][capacity]
   uint8_t* payload_history;      // [S][Hp][capacity]
@@ -2183,7 +2184,92 @@ __global__ __launch_bounds__(kWave) void router_decode_kernel(RouterUpdate U) {
 __global__ __launch_bounds__(256) void router_advance_kernel(RouterUpdate U) {
   const int slot = blockIdx.x * blockDim.x + threadIdx.x;
   if (slot >= U.S) return;
-  U.history_lengths[slot] += router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot);
+  const int chunk = router_chunk_begin(U, slot + 1) - router_chunk_begin(U, slot);
+  if (U.history_lengths_out != nullptr) {
+    U.history_lengths_out[slot] = U.history_lengths[slot] + chunk;
+  } else {
+    U.history_lengths[slot] += chunk;
+  }
+}
+
+// A decoding step as one launch: where the advanced lengths go to an array of their own, a
+// wave can append its row, route it and leave the new length without waiting for any other
+// wave (three launches otherwise: append, route, advance, each waiting for the one before).
+// Symbols at positions from the old length on are the chunk's own and are read from the
+// update's inputs, so that no wave depends on another's append.
+__global__ __launch_bounds__(kWave) void router_decode_step_kernel(RouterUpdate U) {
+  const int run = static_cast<int>(blockIdx.x / static_cast<unsigned>(U.blocks_per_run));
+  const int row = static_cast<int>(blockIdx.x - static_cast<unsigned>(run) * U.blocks_per_run);
+  const int slot = run / U.H;
+  const int head = run - slot * U.H;
+  const int lane = threadIdx.x;
+  const int old_length = U.history_lengths[slot];
+  const int chunk_begin = router_chunk_begin(U, slot);
+  const int rows = router_chunk_begin(U, slot + 1) - chunk_begin;
+  if (head == 0 && row == 0 && lane == 0) U.history_lengths_out[slot] = old_length + rows;
+  if (row >= rows) return;
+  const int t = old_length + row;
+  const int64_t run_base = static_cast<int64_t>(run) * U.capacity;
+  const uint8_t* q_history = U.query_history + run_base;
+  const uint8_t* k_history = U.key_history + run_base;
+  const uint8_t* q_new = U.query + static_cast<int64_t>(chunk_begin) * U.H + head;
+  const uint8_t* k_new = U.key + static_cast<int64_t>(chunk_begin) * U.H + head;
+  const auto q_at = [&](int position) -> uint32_t {
+    return position < old_length
+        ? q_history[position]
+        : q_new[static_cast<int64_t>(position - old_length) * U.H] & U.qk_mask;
+  };
+  const auto k_at = [&](int position) -> uint32_t {
+    return position < old_length
+        ? k_history[position]
+        : k_new[static_cast<int64_t>(position - old_length) * U.H] & U.qk_mask;
+  };
+  const int payload_head = head / (U.H / U.Hp);
+  const int64_t payload_base = (static_cast<int64_t>(slot) * U.Hp + payload_head) * U.capacity;
+  if (lane == 0) {  // this row's symbols join the histories
+    U.query_history[run_base + t] = static_cast<uint8_t>(q_at(t));
+    U.key_history[run_base + t] = static_cast<uint8_t>(k_at(t));
+    if (head < U.Hp) {
+      U.payload_history[(static_cast<int64_t>(slot) * U.Hp + head) * U.capacity + t] =
+          U.payload[static_cast<int64_t>(chunk_begin + row) * U.Hp + head] & U.payload_mask;
+    }
+  }
+  const uint32_t q_symbol = q_at(t);
+  unsigned long long best = 0ull;
+  constexpr int kAhead = 4;  // key symbols a lane has in flight
+  for (int a0 = 1 + lane; a0 <= t; a0 += kAhead * kWave) {
+    uint32_t keys[kAhead];
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      const int a = a0 + j * kWave;
+      keys[j] = a <= t ? k_at(a - 1) : 0x100u;
+    }
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j) {
+      if (keys[j] != q_symbol) continue;
+      const int a = a0 + j * kWave;
+      const int limit = min(U.W, a);
+      int length = 1;
+      while (length < limit && q_at(t - length) == k_at(a - 1 - length)) ++length;
+      best = max(best, (static_cast<unsigned long long>(length) << 32) | static_cast<uint32_t>(a));
+    }
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    best = max(best, static_cast<unsigned long long>(__shfl_xor(best, offset, kWave)));
+  }
+  if (lane != 0) return;
+  const int route = (best >> 32) > 0 ? static_cast<int>(best & 0xffffffffull) : 0;
+  const int64_t token = chunk_begin + row;
+  uint8_t symbol = 0;
+  if (route > 0) {  // the payload that follows the matched key: position `route`
+    symbol = route < old_length
+        ? U.payload_history[payload_base + route]
+        : U.payload[static_cast<int64_t>(chunk_begin + route - old_length) * U.Hp + payload_head] &
+              U.payload_mask;
+  }
+  U.matched_key_end[token * U.H + head] = route > 0 ? route - 1 : -1;
+  U.output[token * U.H + head] = symbol;
 }
 
 // ---------------------------------------------------------------------------
@@ -2717,6 +2803,7 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   U.chunk_offsets = u.chunk_offsets;
   U.uniform_chunk = u.uniform_chunk;
   U.history_lengths = u.history_lengths;
+  U.history_lengths_out = u.history_lengths_out;
   U.query_history = u.query_history;
   U.key_history = u.key_history;
   U.payload_history = u.payload_history;
@@ -2745,28 +2832,37 @@ int rosa_hip_router_update(const rosa_router_update* update, void* stream) {
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t symbols = static_cast<int64_t>(u.tokens) * u.H;
-  hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
   const int64_t runs = static_cast<int64_t>(u.S) * u.H;
-  if (u.longest_chunk > 0) {
-    const bool decode = u.longest_chunk <= kRouterDecodeRows;
-    U.blocks_per_run = decode ? u.longest_chunk : (u.longest_chunk + kWave - 1) / kWave;
+  const bool decode = u.longest_chunk > 0 && u.longest_chunk <= kRouterDecodeRows;
+  if (decode && u.history_lengths_out != nullptr) {
+    // a decoding step with the lengths going to an array of their own: one launch
+    U.blocks_per_run = u.longest_chunk;
     const int64_t blocks = runs * U.blocks_per_run;
     if (blocks > INT32_MAX) return fail(1, "router: slots * heads * row blocks must fit in int32");
-    if (decode) {
-      hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
-                         s, U);
-    } else {
-      if (indexed) {
-        hipLaunchKernelGGL(router_index_kernel, dim3(static_cast<unsigned>(runs)),
-                           dim3(kIndexThreads), 0, s, U);
-        hipLaunchKernelGGL(router_candidates_kernel, dim3(static_cast<unsigned>(blocks)),
-                           dim3(kWave), 0, s, U);
+    hipLaunchKernelGGL(router_decode_step_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave),
+                       0, s, U);
+  } else {
+    hipLaunchKernelGGL(router_append_kernel, dim3(blocks_for(symbols, 256)), dim3(256), 0, s, U);
+    if (u.longest_chunk > 0) {
+      U.blocks_per_run = decode ? u.longest_chunk : (u.longest_chunk + kWave - 1) / kWave;
+      const int64_t blocks = runs * U.blocks_per_run;
+      if (blocks > INT32_MAX) return fail(1, "router: slots * heads * row blocks must fit in int32");
+      if (decode) {
+        hipLaunchKernelGGL(router_decode_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave),
+                           0, s, U);
+      } else {
+        if (indexed) {
+          hipLaunchKernelGGL(router_index_kernel, dim3(static_cast<unsigned>(runs)),
+                             dim3(kIndexThreads), 0, s, U);
+          hipLaunchKernelGGL(router_candidates_kernel, dim3(static_cast<unsigned>(blocks)),
+                             dim3(kWave), 0, s, U);
+        }
+        hipLaunchKernelGGL(router_route_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave),
+                           0, s, U);
       }
-      hipLaunchKernelGGL(router_route_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kWave), 0,
-                         s, U);
     }
+    hipLaunchKernelGGL(router_advance_kernel, dim3(blocks_for(u.S, 256)), dim3(256), 0, s, U);
   }
-  hipLaunchKernelGGL(router_advance_kernel, dim3(blocks_for(u.S, 256)), dim3(256), 0, s, U);
   const hipError_t status = hipGetLastError();
   if (status != hipSuccess) return fail_hip(status, "router launch");
   return 0;

@@ -500,7 +500,10 @@ class RosaRuntime:
         chunk_lengths = [after - before for before, after in zip(offsets[:-1], offsets[1:])]
         self._grow(max(old + new for old, new in zip(self._lengths, chunk_lengths)))
         if self._device_lengths is None:
+            # two arrays taking turns: an update reads one and writes the advanced lengths to the
+            # other, which makes a decoding step one launch
             self._device_lengths = torch.tensor(self._lengths, dtype=torch.int32).to(self._device)
+            self._device_lengths_next = torch.empty_like(self._device_lengths)
         uniform = all(length == chunk_lengths[0] for length in chunk_lengths)
         tables = None if uniform else torch.tensor(offsets, dtype=torch.int32).to(self._device)
         update = cabi.RosaRouterUpdate()
@@ -513,6 +516,7 @@ class RosaRuntime:
         update.uniform_chunk = chunk_lengths[0] if uniform else 0
         update.chunk_offsets = None if uniform else tables.data_ptr()
         update.history_lengths = self._device_lengths.data_ptr()
+        update.history_lengths_out = self._device_lengths_next.data_ptr()
         update.query_history = self._query_history.data_ptr()
         update.key_history = self._key_history.data_ptr()
         update.payload_history = self._payload_history.data_ptr()
@@ -525,6 +529,8 @@ class RosaRuntime:
         for held in (tables, workspace):
             if held is not None:
                 held.record_stream(torch.cuda.current_stream(self._device))
+        self._device_lengths, self._device_lengths_next = \
+            self._device_lengths_next, self._device_lengths
         self._lengths = [old + new for old, new in zip(self._lengths, chunk_lengths)]
         return output, ends
 

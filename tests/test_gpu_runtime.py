@@ -620,3 +620,69 @@ def test_loaded_state_is_reduced_to_the_declared_symbol_widths(rosa):
                                             payload[:, tokens:].to(DEVICE))
     assert torch.equal(ends.cpu(), want[1][:, tokens:])
     assert torch.equal(output.cpu(), want[0][:, tokens:])
+
+
+def test_decoding_steps_in_place_and_through_the_single_launch_agree(rosa):
+    # the C ABI advances `history_lengths` in place unless `history_lengths_out` is given; the
+    # runtime gives it (a decoding step is then one launch).  Both against the oracle, with
+    # chunks of 1, 3 and 8 rows after a prefill, ragged across two slots.
+    from rosa_soft_amd import cabi
+
+    heads, payload_heads, bits, horizon, capacity = 4, 2, 3, 6, 256
+    steps = [[40, 37], [1, 1], [3, 0], [8, 5], [1, 2]]  # rows per slot, per update
+    totals = [sum(step[slot] for step in steps) for slot in range(2)]
+    streams = []
+    for slot, total in enumerate(totals):
+        q = random_packed((1, total, heads), bits, 200 + slot)
+        k = random_packed((1, total, heads), bits, 210 + slot)
+        p = random_packed((1, total, payload_heads), bits, 220 + slot)
+        streams.append((q[0], k[0], p[0], expect_dense(q, k, p, bits, bits, horizon)))
+
+    def updates():
+        done = [0, 0]
+        for step in steps:
+            parts = [torch.cat([s[i][done[slot]:done[slot] + step[slot]] for slot, s in enumerate(streams)])
+                     for i in range(3)]
+            want_output = torch.cat([s[3][0][0, done[slot]:done[slot] + step[slot]]
+                                     for slot, s in enumerate(streams)])
+            want_ends = torch.cat([s[3][1][0, done[slot]:done[slot] + step[slot]]
+                                   for slot, s in enumerate(streams)])
+            offsets = [0, step[0], step[0] + step[1]]
+            yield parts, offsets, want_output, want_ends
+            done = [done[slot] + step[slot] for slot in range(2)]
+
+    # in place, straight through the C ABI
+    lengths = torch.zeros(2, dtype=torch.int32, device=DEVICE)
+    histories = [torch.zeros(2, n, capacity, dtype=torch.uint8, device=DEVICE)
+                 for n in (heads, heads, payload_heads)]
+    for (query, key, payload), offsets, want_output, want_ends in updates():
+        tokens = offsets[-1]
+        query, key, payload = (t.to(DEVICE).contiguous() for t in (query, key, payload))
+        table = torch.tensor(offsets, dtype=torch.int32, device=DEVICE)
+        output = torch.empty(tokens, heads, dtype=torch.uint8, device=DEVICE)
+        ends = torch.empty(tokens, heads, dtype=torch.int64, device=DEVICE)
+        update = cabi.RosaRouterUpdate(
+            S=2, H=heads, Hp=payload_heads, W=horizon, qk_bits=bits, payload_bits=bits,
+            capacity=capacity, tokens=tokens, longest_chunk=max(offsets[1], offsets[2] - offsets[1]),
+            uniform_chunk=0, longest_total=capacity)
+        update.chunk_offsets = table.data_ptr()
+        update.history_lengths = lengths.data_ptr()
+        update.query_history, update.key_history, update.payload_history = (
+            h.data_ptr() for h in histories)
+        update.query, update.key, update.payload = query.data_ptr(), key.data_ptr(), payload.data_ptr()
+        update.output, update.matched_key_end = output.data_ptr(), ends.data_ptr()
+        cabi.router_update(update, torch.device(DEVICE))
+        torch.cuda.synchronize()
+        assert torch.equal(output.cpu(), want_output) and torch.equal(ends.cpu(), want_ends)
+    assert lengths.tolist() == totals
+    # the runtime: lengths to the other array, decoding steps in one launch
+    with rosa.RosaRuntime(heads, payload_heads, bits, bits, horizon) as runtime:
+        for (query, key, payload), offsets, want_output, want_ends in updates():
+            output, ends = runtime.update_packed(
+                query.to(DEVICE), key.to(DEVICE), payload.to(DEVICE),
+                cu_seqlens=torch.tensor(offsets, dtype=torch.int32))
+            assert torch.equal(output.cpu(), want_output) and torch.equal(ends.cpu(), want_ends)
+        histories_after = (runtime._query_history, runtime._key_history, runtime._payload_history)
+        for mine, theirs in zip(histories, histories_after):
+            width = min(mine.size(-1), theirs.size(-1), max(totals))
+            assert torch.equal(mine[..., :width], theirs[..., :width])
